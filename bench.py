@@ -1,0 +1,307 @@
+#!/usr/bin/env python3
+"""Benchmark of the KV data-movement path on one MI355X.
+
+Workload (default, ``qwen2_7b_migrate``): the Qwen2-7B KV shape — 28 layers of
+``[2, 60000, 16, 4, 128]`` bf16 (51.3 GiB per pool) — and a batch of 32 migrating
+requests with prompt lengths U{512..4096} plus a 1024-token image prefix
+(96..320 blocks each). One *step* moves every request of the batch: pack from the
+source pool under its block table into a contiguous transfer buffer
+(``KVWorker.extract_kv_blocks``), then unpack into a second, independently
+allocated pool under a different table (``KVWorker.write_kv_blocks``), request
+by request as the reference does. Everything is resident in HBM before the timed
+region (pools, block tables); values are synthetic N(0, 0.5).
+
+Prints ONE JSON line. ``value`` is whole-job GB/s = algorithmic bytes (read +
+write of pack and of unpack = 4 x payload) / wall time of the timed steps.
+``roofline`` prices the block-move kernel (pack and unpack are two instances of
+the same kernel) against the 8 TB/s HBM peak from HIP-event times of its launches
+inside the timed region. ``cpu_baseline`` times the reference's torch expressions
+(oracle ``ref_*``) on the host cores for a bounded sample of the same batch.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--blocks", type=int, default=60000, help="pool size in blocks (BASELINE: 60000)")
+    ap.add_argument("--requests", type=int, default=32)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements (append, batched, copy)")
+    ap.add_argument("--variant", type=int, default=0, help="block-move launch variant (tuning)")
+    return ap.parse_args()
+
+
+def make_requests(num_requests, num_blocks, seed):
+    """Block tables of the batch: disjoint slices of two different permutations."""
+    g = torch.Generator().manual_seed(seed)
+    prompts = torch.randint(512, 4097, (num_requests,), generator=g)
+    nblk = [(int(p) + 1024 + 15) // 16 for p in prompts]
+    total = sum(nblk)
+    if total > num_blocks:
+        raise SystemExit(f"pool of {num_blocks} blocks cannot hold the batch ({total} blocks)")
+    sperm = torch.randperm(num_blocks, generator=g)
+    dperm = torch.randperm(num_blocks, generator=torch.Generator().manual_seed(seed + 1000))
+    tables, off = [], 0
+    for n in nblk:
+        tables.append((sperm[off:off + n].clone(), dperm[off:off + n].clone()))
+        off += n
+    return tables, total
+
+
+def cpu_baseline(tables, L, bs, H, D, dtype, budget_s=20.0):
+    """The reference's torch path on the host cores, on a reduced pool (bytes moved depend
+    on the blocks per request, not on the pool size) and the first requests of the batch."""
+    from oracle import kv_oracle as orc
+
+    sample = tables[:8]
+    nb = sum(len(s) for s, _ in sample)
+    NBc = max(nb, 2048)
+    torch.manual_seed(0)
+    src = [torch.randn((2, NBc, bs, H, D)).mul_(0.5).to(dtype) for _ in range(L)]
+    dst = [torch.zeros((2, NBc, bs, H, D), dtype=dtype) for _ in range(L)]
+    # remap the sample's tables into the reduced pool, keeping them scattered and disjoint
+    g = torch.Generator().manual_seed(7)
+    sp, dp = torch.randperm(NBc, generator=g), torch.randperm(NBc, generator=g)
+    off, tabs = 0, []
+    for s, _ in sample:
+        tabs.append((sp[off:off + len(s)].tolist(), dp[off:off + len(s)].tolist()))
+        off += len(s)
+    chunk = bs * H * D * src[0].element_size()
+    bytes_per_pass = 4 * nb * L * 2 * chunk
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 5 and (time.perf_counter() - t_start < budget_s or len(times) < 2):
+        t0 = time.perf_counter()
+        for si, di in tabs:
+            buf = orc.ref_extract_kv_blocks(src, si)
+            orc.ref_write_kv_blocks(dst, di, buf)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {
+        "value": round(bytes_per_pass / med / 1e9, 3),
+        "unit": "GB/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"first {len(sample)} of the batch's requests ({nb} blocks, {bytes_per_pass / 1e9:.2f} GB algorithmic "
+                  f"per pass) on pools reduced to {NBc} blocks; torch index + stack / indexed assignment on CPU; "
+                  f"median of {len(times)} passes ({med:.2f} s each)",
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the cross-GPU hop is replaced by a second pool on the "
+              "same device); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the KV kernels have no CPU fallback", file=sys.stderr)
+        sys.exit(2)
+
+    from elasticmm_amd import _lib, kv_ops
+    from elasticmm_amd.kv_ops import PoolView
+    from elasticmm_amd.worker import KVWorker
+
+    lib = _lib.load()
+    if args.variant:
+        lib.emm_set_move_variant(args.variant)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L, bs, H, D, dtype = 28, 16, 4, 128, torch.bfloat16
+    NB = args.blocks
+    chunk = bs * H * D * 2
+    tables, total_blocks = make_requests(args.requests, NB, seed=2)
+
+    src_w, dst_w = KVWorker(0, "cuda:0", bs), KVWorker(1, "cuda:0", bs)
+    src_w.init_kvcache(NB, num_layers=L, num_kv_heads=H, head_size=D, dtype=dtype, monolithic=True)
+    dst_w.init_kvcache(NB, num_layers=L, num_kv_heads=H, head_size=D, dtype=dtype, monolithic=True)
+    g = torch.Generator(device=dev).manual_seed(2)
+    for t in src_w.kv_cache:
+        t.normal_(0.0, 0.5, generator=g)
+    for t in dst_w.kv_cache:
+        t.zero_()
+    dev_tables = [(s.to(dev), d.to(dev)) for s, d in tables]
+    torch.cuda.synchronize()
+
+    payload = total_blocks * L * 2 * chunk       # bytes held by the batch's blocks
+    bytes_per_step = 4 * payload                 # pack: read + write, unpack: read + write
+
+    def step(events=None):
+        for si, di in dev_tables:
+            if events is not None:
+                e0, e1, e2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+                e0.record()
+            buf = src_w.extract_kv_blocks(si)
+            if events is not None:
+                e1.record()
+            dst_w.write_kv_blocks(di, buf)
+            if events is not None:
+                e2.record()
+                events.append((e0, e1, e2, si.numel()))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    events = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(events)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    wall = t1 - t0
+    ms_per_step = wall / args.steps * 1e3
+    value = bytes_per_step * args.steps / wall / 1e9
+
+    # per-launch kernel time of the block-move kernel (pack and unpack instances)
+    pack_ms = sum(e0.elapsed_time(e1) for e0, e1, _, _ in events)
+    unpack_ms = sum(e1.elapsed_time(e2) for _, e1, e2, _ in events)
+    launches = 2 * len(events)
+    kern_bytes = sum(2 * 2 * n * L * 2 * chunk for *_, n in events)  # per request: pack 2x + unpack 2x payload
+    achieved = kern_bytes / ((pack_ms + unpack_ms) * 1e-3) / 1e9
+    roofline = {
+        "bound": "hbm",
+        "kernel": "emm_block_move_kernel (pack + unpack instances)",
+        "achieved": round(achieved, 1),
+        "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBPS, 4),
+        "traffic": None,
+        "launches": launches,
+        "avg_launch_us": round((pack_ms + unpack_ms) * 1e3 / launches, 2),
+        "avg_bytes_per_launch": int(kern_bytes / launches),
+        "pack_GBps": round(kern_bytes / 2 / (pack_ms * 1e-3) / 1e9, 1),
+        "unpack_GBps": round(kern_bytes / 2 / (unpack_ms * 1e-3) / 1e9, 1),
+    }
+
+    # spot check inside the bench: the last request really arrived
+    si, di = dev_tables[-1]
+    assert torch.equal(dst_w.kv_cache[L - 1][:, di], src_w.kv_cache[L - 1][:, si]), "migration check failed"
+
+    extra = {}
+    if not args.no_extra:
+        extra = secondary(src_w, dst_w, dev_tables, payload, L, bs, H, D, NB, dev)
+
+    result = {
+        "metric": "KV pack+unpack GB/s",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8",
+        "data": "synthetic",
+        "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "config": {
+            "workload": "qwen2_7b_migrate: 28 layers x [2,%d,16,4,128] bf16 x 2 pools, %d requests (%d blocks, "
+                        "%.2f GB payload), per-request pack -> unpack under a different block table"
+                        % (NB, len(tables), total_blocks, payload / 1e9),
+            "num_layers": L, "num_blocks": NB, "block_size": bs, "kv_heads": H, "head_dim": D,
+            "requests": len(tables), "blocks_moved": total_blocks, "algorithmic_bytes_per_step": bytes_per_step,
+        },
+        "roofline": roofline,
+        "extra": extra,
+    }
+    if not args.no_cpu_baseline:
+        # free the device pools first: the host leg needs nothing from them
+        result["cpu_baseline"] = cpu_baseline(tables, L, bs, H, D, dtype)
+    print(json.dumps(result), flush=True)
+
+
+def timed(fn, iters, warmup=2):
+    """Median and min milliseconds of fn() over iters runs, HIP events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(iters):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        e1.synchronize()
+        ts.append(e0.elapsed_time(e1))
+    ts.sort()
+    return ts[len(ts) // 2], ts[0]
+
+
+def secondary(src_w, dst_w, dev_tables, payload, L, bs, H, D, NB, dev):
+    """Other shapes of the same path, reported next to the headline (not bench lines of their own)."""
+    from elasticmm_amd import cache_ops, kv_ops
+
+    out = {}
+    chunk = bs * H * D * 2
+    sp, dp = src_w.pool, dst_w.pool
+    # one launch for the whole batch (concatenated tables)
+    all_si = torch.cat([s for s, _ in dev_tables])
+    all_di = torch.cat([d for _, d in dev_tables])
+    buf = torch.empty(sp.packed_shape(all_si.numel()), dtype=sp.dtype, device=dev)
+    med, mn = timed(lambda: kv_ops.kv_pack(sp, all_si, out=buf), 10)
+    out["batched_pack_GBps"] = round(2 * payload / (med * 1e-3) / 1e9, 1)
+    med, mn = timed(lambda: kv_ops.kv_unpack(dp, all_di, buf), 10)
+    out["batched_unpack_GBps"] = round(2 * payload / (med * 1e-3) / 1e9, 1)
+    med, mn = timed(lambda: kv_ops.kv_migrate(sp, all_si, dp, all_di), 10)
+    out["fused_migrate_GBps"] = round(2 * payload / (med * 1e-3) / 1e9, 1)
+    # yardsticks: plain copies of the same byte count
+    flat = buf.view(-1)
+    other = torch.empty_like(flat)
+    med, mn = timed(lambda: kv_ops.stream_copy(flat, other), 10)
+    out["plain_copy_same_engine_GBps"] = round(2 * payload / (med * 1e-3) / 1e9, 1)
+    med, mn = timed(lambda: other.copy_(flat), 10)
+    out["torch_copy_GBps"] = round(2 * payload / (med * 1e-3) / 1e9, 1)
+    del other, buf
+    # copy_blocks: half of the batch's blocks to free blocks of the same pool
+    P = all_si.numel() // 2
+    used = torch.zeros(NB, dtype=torch.bool, device=dev)
+    used[all_si] = True
+    free = (~used).nonzero().squeeze(1)
+    if free.numel() >= P:
+        mapping = torch.stack([all_si[:P], free[:P]], 1).contiguous()
+        med, mn = timed(lambda: kv_ops.copy_blocks(sp, mapping), 10)
+        out["copy_blocks_GBps"] = round(2 * P * L * 2 * chunk / (med * 1e-3) / 1e9, 1)
+    # append (reshape_and_cache): 256 decode tokens + one 8192-token prefill chunk, 5% padded
+    T = 8448
+    g = torch.Generator(device=dev).manual_seed(3)
+    slots = torch.randperm(NB * bs, device=dev, generator=g)[:T].clone()
+    slots[torch.rand(T, device=dev, generator=g) < 0.05] = -1
+    valid = int((slots >= 0).sum())
+    keys = [torch.randn((T, H, D), device=dev, generator=g).to(torch.bfloat16) for _ in range(L)]
+    values = [torch.randn((T, H, D), device=dev, generator=g).to(torch.bfloat16) for _ in range(L)]
+    kv = src_w.kv_cache
+    row = H * D * 2
+    step_bytes = L * (valid * 2 * row * 2 + 8 * T)
+
+    def per_layer():
+        for l in range(L):
+            cache_ops.reshape_and_cache_flash(keys[l], values[l], kv[l][0], kv[l][1], slots, "auto")
+
+    med, mn = timed(per_layer, 20)
+    out["append_per_layer_launches"] = {"tokens_per_s": round(valid / (med * 1e-3)), "ms_per_step": round(med, 4),
+                                        "GBps": round(step_bytes / (med * 1e-3) / 1e9, 1)}
+    med, mn = timed(lambda: cache_ops.reshape_and_cache_flash_layers(keys, values, kv, slots, "auto"), 20)
+    out["append_one_launch"] = {"tokens_per_s": round(valid / (med * 1e-3)), "ms_per_step": round(med, 4),
+                                "GBps": round(step_bytes / (med * 1e-3) / 1e9, 1)}
+    out["append_tokens"] = {"T": T, "valid": valid, "layers": L}
+    return out
+
+
+if __name__ == "__main__":
+    main()

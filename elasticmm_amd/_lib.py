@@ -1,0 +1,82 @@
+"""ctypes binding of libemm_kv.so (the C ABI of include/emm_kv.h).
+
+There is no fallback: if the shared object is missing or an entry point fails,
+the caller gets an exception.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p, POINTER
+
+from .build import library_path
+
+EMM_KV_ABI_VERSION = 1
+EMM_MAX_LAYERS = 96
+EMM_MAX_SEGMENTS = 96
+EMM_DTYPE_BF16 = 0
+EMM_DTYPE_F16 = 1
+
+_P = c_void_p
+_PP = POINTER(c_void_p)
+_I64P = POINTER(c_int64)
+
+# name -> (restype, argtypes); mirrors include/emm_kv.h one to one
+SIGNATURES = {
+    "emm_last_error": (c_char_p, []),
+    "emm_abi_version": (c_int, []),
+    "emm_set_move_variant": (c_int, [c_int]),
+    "emm_kv_pack": (c_int, [_PP, c_int, c_int, c_int64, c_int64, _P, c_int64, _P, _P]),
+    "emm_kv_unpack": (c_int, [_PP, c_int, c_int, c_int64, c_int64, _P, c_int64, _P, _P]),
+    "emm_copy_blocks": (c_int, [_PP, c_int, c_int, c_int64, c_int64, _P, c_int64, _P]),
+    "emm_kv_migrate": (c_int, [_PP, c_int64, _PP, c_int64, c_int, c_int, c_int64, _P, _P, c_int64, _P]),
+    "emm_kv_unpack_dequant_fp8": (c_int, [_PP, c_int, c_int64, c_int64, _P, c_int64, _P, _P, _P, c_int, _P]),
+    "emm_reshape_and_cache": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, _P]),
+    "emm_reshape_and_cache_layers": (c_int, [_PP, _PP, _PP, _PP, c_int, _P, c_int64, c_int64, c_int64, c_int64,
+                                             c_int64, _P]),
+    "emm_reshape_and_cache_fp8": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                          _P, _P, c_int, _P]),
+    "emm_reshape_and_cache_fp8_layers": (c_int, [_PP, _PP, _PP, _PP, c_int, _P, c_int64, c_int64, c_int64,
+                                                 c_int64, c_int64, _P, _P, c_int, _P]),
+    "emm_concat_rows": (c_int, [_PP, _I64P, c_int, _P, c_int64, _P]),
+    "emm_stream_copy": (c_int, [_P, _P, c_int64, _P]),
+}
+
+_lib = None
+
+
+class EmmError(RuntimeError):
+    """An entry point of libemm_kv.so returned a non-zero code."""
+
+
+def load() -> ctypes.CDLL:
+    """Load libemm_kv.so once; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = library_path()
+    if not os.path.exists(path):
+        raise RuntimeError(
+            f"{path} is missing: the HIP library has not been built "
+            "(run `python -m elasticmm_amd.build`). There is no CPU fallback.")
+    lib = ctypes.CDLL(path)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    ver = lib.emm_abi_version()
+    if ver != EMM_KV_ABI_VERSION:
+        raise RuntimeError(f"libemm_kv.so ABI version {ver}, expected {EMM_KV_ABI_VERSION}")
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().emm_last_error().decode("utf-8", "replace")
+        raise EmmError(f"{what} failed with code {rc}: {msg}")
+
+
+def ptr_table(ptrs) -> ctypes.Array:
+    """A host array of device pointers for the `layer_ptrs`-style arguments."""
+    return (c_void_p * len(ptrs))(*ptrs)

@@ -1,0 +1,58 @@
+"""vLLM-shaped cache operators: ``reshape_and_cache_flash`` and ``copy_blocks``.
+
+The reference reaches both inside vLLM (``vllm>=0.10.1``, V0 engine): the append
+from ``model_runner.execute_model`` (elasticmm/engine/v0/worker_steps.py:281, :438)
+on the pool bound at elasticmm/engine/v0/worker.py:408-412, and ``copy_blocks``
+through ``CacheEngine`` (worker.py:380). The signatures below keep vLLM's argument
+order so an attention backend can call them unchanged.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence
+
+import torch
+
+from . import kv_ops
+from .kv_ops import PoolView
+
+
+def reshape_and_cache_flash(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor,
+                            value_cache: torch.Tensor, slot_mapping: torch.Tensor, kv_cache_dtype: str = "auto",
+                            k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None) -> None:
+    """key, value ``[num_tokens, num_heads, head_size]``; caches
+    ``[num_blocks, block_size, num_heads, head_size]``; ``slot_mapping`` int64
+    ``[num_tokens]`` with -1 for padded tokens. ``kv_cache_dtype`` is "auto" (cache
+    dtype == key dtype, bit copy) or "fp8" / "fp8_e4m3" (cache is 1 byte wide and
+    is written as ``e4m3fn(float(x) / scale)``)."""
+    if kv_cache_dtype == "auto":
+        if key_cache.element_size() != key.element_size():
+            raise ValueError("kv_cache_dtype='auto' needs a cache of the key's element size")
+        kv_ops.reshape_and_cache(key, value, key_cache, value_cache, slot_mapping)
+    elif kv_cache_dtype in ("fp8", "fp8_e4m3"):
+        if key_cache.element_size() != 1:
+            raise ValueError("fp8 KV cache must be a 1-byte tensor (float8_e4m3fn or uint8)")
+        kv_ops.reshape_and_cache(key, value, key_cache, value_cache, slot_mapping, k_scale, v_scale)
+    else:
+        raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
+
+
+def reshape_and_cache_flash_layers(keys: Sequence[torch.Tensor], values: Sequence[torch.Tensor],
+                                   kv_caches: Sequence[torch.Tensor], slot_mapping: torch.Tensor,
+                                   kv_cache_dtype: str = "auto", k_scales=None, v_scales=None) -> None:
+    """All layers of a step in one launch. ``kv_caches[l]`` is ``[2, num_blocks, block_size, H, D]``."""
+    key_caches = [c[0] for c in kv_caches]
+    value_caches = [c[1] for c in kv_caches]
+    if kv_cache_dtype == "auto":
+        kv_ops.reshape_and_cache_layers(keys, values, key_caches, value_caches, slot_mapping)
+    elif kv_cache_dtype in ("fp8", "fp8_e4m3"):
+        kv_ops.reshape_and_cache_layers(keys, values, key_caches, value_caches, slot_mapping, k_scales, v_scales)
+    else:
+        raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
+
+
+def copy_blocks(kv_caches: List[torch.Tensor], block_mapping: torch.Tensor) -> None:
+    """``kv_caches``: list of ``[2, num_blocks, block_size, H, D]``; ``block_mapping``: int64
+    ``[num_pairs, 2]`` of (src, dst). One launch covers every layer, K and V."""
+    if len(kv_caches) == 0 or block_mapping.numel() == 0:
+        return
+    kv_ops.copy_blocks(PoolView(kv_caches), block_mapping)

@@ -1,0 +1,957 @@
+// libemm_kv — KV-cache data-movement kernels for gfx950 (MI355X) behind the C ABI
+// declared in include/emm_kv.h.
+//
+// Everything here is HBM-bandwidth work: the kernels move 16 bytes per lane per
+// access, every wave touches 1 KiB of contiguous memory per instruction, all
+// loads of a tile are issued before the first store, and loads/stores are
+// non-temporal (streaming data is never re-read, so it should not displace
+// other lines in L2 / Infinity Cache). Block-table entries and slot-mapping
+// entries are wave-uniform: they are fetched once per wave on the scalar path
+// (or broadcast with readfirstlane) and all address arithmetic that depends on
+// them stays in scalar registers.
+//
+// Pool layout (per layer): [num_kv, num_blocks, chunk] contiguous, where
+// chunk = block_size * num_kv_heads * head_dim elements.
+// Transfer-buffer layout: [num_layers, num_kv, n, chunk] contiguous.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+#include <string.h>
+
+#include "emm_kv.h"
+
+namespace {
+
+// ----------------------------------------------------------------------------
+// error reporting
+// ----------------------------------------------------------------------------
+thread_local char g_last_error[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char *what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess)
+    return fail(EMM_ELAUNCH, "%s: launch failed: %s", what, hipGetErrorString(e));
+  return EMM_OK;
+}
+
+// ----------------------------------------------------------------------------
+// vector types and streaming accessors
+// ----------------------------------------------------------------------------
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <int BYTES> struct VecOf;
+template <> struct VecOf<16> { typedef u32x4 type; };
+template <> struct VecOf<8> { typedef u32x2 type; };
+template <> struct VecOf<4> { typedef uint32_t type; };
+template <> struct VecOf<2> { typedef uint16_t type; };
+template <> struct VecOf<1> { typedef uint8_t type; };
+
+template <typename V, bool NT>
+__device__ __forceinline__ V ld(const char *p) {
+  if constexpr (NT)
+    return __builtin_nontemporal_load(reinterpret_cast<const V *>(p));
+  else
+    return *reinterpret_cast<const V *>(p);
+}
+
+template <typename V, bool NT>
+__device__ __forceinline__ void st(char *p, V v) {
+  if constexpr (NT)
+    __builtin_nontemporal_store(v, reinterpret_cast<V *>(p));
+  else
+    *reinterpret_cast<V *>(p) = v;
+}
+
+constexpr int kThreads = 256; // 4 wavefronts of 64 lanes
+
+// Copy one tile of U * kThreads vectors: vector (u * kThreads + tid) of the
+// tile. All U loads are in flight before the first store. `limit` is the number
+// of bytes valid from `src`/`dst` on (tail tiles are predicated per lane).
+template <typename V, int U, bool NTL, bool NTS>
+__device__ __forceinline__ void copy_tile(const char *__restrict__ src,
+                                          char *__restrict__ dst,
+                                          int64_t limit) {
+  constexpr int64_t VB = sizeof(V);
+  const int64_t lane_off = (int64_t)threadIdx.x * VB;
+  V v[U];
+  if (limit >= (int64_t)U * kThreads * VB) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      v[u] = ld<V, NTL>(src + lane_off + (int64_t)u * kThreads * VB);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      st<V, NTS>(dst + lane_off + (int64_t)u * kThreads * VB, v[u]);
+  } else {
+    // tail tile: lanes past the end re-read vector 0 (always valid, limit > 0)
+    // so the loads stay unconditional and in flight together; only the stores
+    // are predicated
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t off = lane_off + (int64_t)u * kThreads * VB;
+      v[u] = ld<V, NTL>(src + (off < limit ? off : 0));
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t off = lane_off + (int64_t)u * kThreads * VB;
+      if (off < limit) st<V, NTS>(dst + off, v[u]);
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------
+// block move: pack / unpack / copy_blocks / migrate / plain copy
+// ----------------------------------------------------------------------------
+// One side of a move is either a block pool (per-layer base pointers, block
+// chosen through an int64 index array) or a linear transfer buffer.
+struct MoveParams {
+  const char *src_layers[EMM_MAX_LAYERS]; // pool source: per-layer bases
+  char *dst_layers[EMM_MAX_LAYERS];       // pool destination: per-layer bases
+  const char *src_linear;                 // linear source base
+  char *dst_linear;                       // linear destination base
+  const int64_t *src_idx;                 // block ids on the source side
+  const int64_t *dst_idx;                 // block ids on the destination side
+  int64_t idx_stride;                     // elements between consecutive ids
+  int64_t src_num_blocks;
+  int64_t dst_num_blocks;
+  int64_t chunk_bytes;
+  int64_t n;                // blocks moved per (layer, kv) plane
+  uint32_t tiles_per_chunk; // ceil(chunk_bytes / tile_bytes)
+  uint32_t num_kv;
+};
+
+// grid: x = n * tiles_per_chunk, y = num_kv, z = num_layers. The x-major
+// dispatch order walks the transfer buffer linearly.
+template <typename V, int U, bool SRC_POOL, bool DST_POOL, bool NTL, bool NTS>
+__global__ __launch_bounds__(kThreads) void emm_block_move_kernel(
+    const MoveParams p) {
+  constexpr int64_t TILE = (int64_t)U * kThreads * sizeof(V);
+  uint32_t j = blockIdx.x, tile = 0;
+  if (p.tiles_per_chunk != 1) {
+    j = blockIdx.x / p.tiles_per_chunk;
+    tile = blockIdx.x - j * p.tiles_per_chunk;
+  }
+  const uint32_t kv = blockIdx.y;
+  const uint32_t l = blockIdx.z;
+  const int64_t chunk = p.chunk_bytes;
+  const int64_t tile_off = (int64_t)tile * TILE;
+  const int64_t linear_off =
+      (((int64_t)l * p.num_kv + kv) * p.n + j) * chunk + tile_off;
+
+  const char *src;
+  if constexpr (SRC_POOL) {
+    const int64_t b = p.src_idx[(int64_t)j * p.idx_stride];
+    if ((uint64_t)b >= (uint64_t)p.src_num_blocks) return; // padding / invalid
+    src = p.src_layers[l] + ((int64_t)kv * p.src_num_blocks + b) * chunk + tile_off;
+  } else {
+    src = p.src_linear + linear_off;
+  }
+  char *dst;
+  if constexpr (DST_POOL) {
+    const int64_t b = p.dst_idx[(int64_t)j * p.idx_stride];
+    if ((uint64_t)b >= (uint64_t)p.dst_num_blocks) return;
+    dst = p.dst_layers[l] + ((int64_t)kv * p.dst_num_blocks + b) * chunk + tile_off;
+  } else {
+    dst = p.dst_linear + linear_off;
+  }
+  copy_tile<V, U, NTL, NTS>(src, dst, chunk - tile_off);
+}
+
+int g_move_variant = 0;
+
+struct MoveCfg {
+  int vec;  // bytes per lane access
+  int unroll;
+  bool ntl, nts;
+};
+
+bool aligned(const void *p, int a) { return ((uintptr_t)p & (uintptr_t)(a - 1)) == 0; }
+
+template <typename V, int U, bool SP, bool DP>
+void launch_move_nt(const MoveParams &p, dim3 grid, bool ntl, bool nts, hipStream_t s) {
+  if (ntl && nts)
+    emm_block_move_kernel<V, U, SP, DP, true, true><<<grid, kThreads, 0, s>>>(p);
+  else if (ntl)
+    emm_block_move_kernel<V, U, SP, DP, true, false><<<grid, kThreads, 0, s>>>(p);
+  else if (nts)
+    emm_block_move_kernel<V, U, SP, DP, false, true><<<grid, kThreads, 0, s>>>(p);
+  else
+    emm_block_move_kernel<V, U, SP, DP, false, false><<<grid, kThreads, 0, s>>>(p);
+}
+
+template <bool SP, bool DP>
+int launch_move(MoveParams &p, int num_layers, int min_align, hipStream_t s,
+                const char *what) {
+  if (p.n == 0 || num_layers == 0 || p.num_kv == 0 || p.chunk_bytes == 0) return EMM_OK;
+  // widest lane access that divides the chunk and every base address
+  int vec = 16;
+  while (vec > 1 && (p.chunk_bytes % vec != 0 || min_align % vec != 0)) vec >>= 1;
+  if (vec == 8) vec = 4; // 8-byte lanes are not instantiated
+  int unroll = 4;
+  bool ntl = true, nts = true;
+  if (vec == 16 && g_move_variant > 0) {
+    const int u = g_move_variant & 0xff;
+    if (u == 1 || u == 2 || u == 4 || u == 8) unroll = u;
+    if (g_move_variant & 0x100) ntl = false;
+    if (g_move_variant & 0x200) nts = false;
+  }
+  // do not make the tile larger than the chunk needs
+  if (vec == 16)
+    while (unroll > 1 && (int64_t)(unroll / 2) * kThreads * vec >= p.chunk_bytes) unroll >>= 1;
+  const int64_t tile_bytes = (int64_t)unroll * kThreads * vec;
+  const int64_t tpc = (p.chunk_bytes + tile_bytes - 1) / tile_bytes;
+  const int64_t gx = p.n * tpc;
+  if (tpc > 0x7fffffffLL || gx > 0x7fffffffLL)
+    return fail(EMM_EINVAL, "%s: n * tiles_per_chunk = %lld exceeds the grid limit", what, (long long)gx);
+  if (num_layers > 65535 || p.num_kv > 65535)
+    return fail(EMM_EINVAL, "%s: num_layers / num_kv exceed the grid limit", what);
+  p.tiles_per_chunk = (uint32_t)tpc;
+  dim3 grid((uint32_t)gx, p.num_kv, (uint32_t)num_layers);
+
+#define EMM_MOVE_CASE(VB, UU)                                                          \
+  if (vec == VB && unroll == UU) {                                                     \
+    launch_move_nt<typename VecOf<VB>::type, UU, SP, DP>(p, grid, ntl, nts, s);        \
+    return check_launch(what);                                                         \
+  }
+  EMM_MOVE_CASE(16, 8)
+  EMM_MOVE_CASE(16, 4)
+  EMM_MOVE_CASE(16, 2)
+  EMM_MOVE_CASE(16, 1)
+  // rare unaligned shapes: narrower lanes, one fixed tile shape
+  EMM_MOVE_CASE(4, 4)
+  EMM_MOVE_CASE(2, 4)
+  EMM_MOVE_CASE(1, 4)
+#undef EMM_MOVE_CASE
+  return fail(EMM_EINVAL, "%s: no kernel for vec=%d unroll=%d", what, vec, unroll);
+}
+
+int common_align(int a, const void *p) {
+  int x = 16;
+  while (x > 1 && !aligned(p, x)) x >>= 1;
+  return a < x ? a : x;
+}
+
+int check_pool_args(const char *what, const void *const *layer_ptrs, int num_layers,
+                    int num_kv, int64_t num_blocks, int64_t chunk_bytes, int64_t n) {
+  if (num_layers < 0 || num_layers > EMM_MAX_LAYERS)
+    return fail(EMM_EINVAL, "%s: num_layers=%d outside [0, %d]", what, num_layers, EMM_MAX_LAYERS);
+  if (num_kv < 0 || num_blocks < 0 || chunk_bytes < 0 || n < 0)
+    return fail(EMM_EINVAL, "%s: negative size (num_kv=%d num_blocks=%lld chunk_bytes=%lld n=%lld)",
+                what, num_kv, (long long)num_blocks, (long long)chunk_bytes, (long long)n);
+  if (num_layers > 0 && !layer_ptrs) return fail(EMM_EINVAL, "%s: layer_ptrs is null", what);
+  for (int l = 0; l < num_layers; ++l)
+    if (!layer_ptrs[l] && n > 0 && num_blocks > 0)
+      return fail(EMM_EINVAL, "%s: layer_ptrs[%d] is null", what, l);
+  return EMM_OK;
+}
+
+// ----------------------------------------------------------------------------
+// fp8-e4m3fn <-> fp32 / 16-bit conversions (bit-exact integer formulations)
+// ----------------------------------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) {
+  return __uint_as_float(h << 16);
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+  _Float16 x;
+  uint16_t b = (uint16_t)h;
+  __builtin_memcpy(&x, &b, 2);
+  return (float)x;
+}
+
+// fp32 -> e4m3fn, round to nearest even, no saturation: magnitudes that round
+// past 448 (>= 465 after RNE, i.e. bits >= 480.0 or the [464, 480) interval
+// rounding up), inf and NaN give sign|0x7F.
+__device__ __forceinline__ uint32_t f32_to_e4m3fn(float f) {
+  const uint32_t u = __float_as_uint(f);
+  const uint32_t sign = (u >> 24) & 0x80u;
+  uint32_t a = u & 0x7fffffffu;
+  uint32_t r;
+  if (a >= 0x43f00000u) { // >= 480, inf, NaN
+    r = 0x7fu;
+  } else if (a < 0x3c800000u) { // below 2^-6: subnormal grid of 2^-9
+    // |f| * 2^9 is exact; rintf rounds to nearest even; 8 encodes 2^-6
+    r = (uint32_t)(int)__builtin_rintf(__uint_as_float(a) * 512.0f);
+  } else {
+    const uint32_t odd = (a >> 20) & 1u;
+    a += 0x7ffffu + odd;    // RNE at bit 20
+    a -= (120u << 23);      // rebias 127 -> 7
+    r = a >> 20;            // may carry into 0x7f (NaN) for [464, 480)
+  }
+  return r | sign;
+}
+
+// e4m3fn byte -> fp32 (exact). NaN bytes give a quiet NaN with the byte's sign.
+__device__ __forceinline__ float e4m3fn_to_f32(uint32_t b) {
+  const uint32_t sign = (b & 0x80u) << 24;
+  const uint32_t e = (b >> 3) & 0xfu;
+  const uint32_t m = b & 7u;
+  uint32_t bits;
+  if (e == 0) {
+    bits = __float_as_uint((float)m * 0.001953125f); // m * 2^-9, exact
+  } else if (e == 15 && m == 7) {
+    bits = 0x7fc00000u;
+  } else {
+    bits = ((e + 120u) << 23) | (m << 20);
+  }
+  return __uint_as_float(bits | sign);
+}
+
+// fp32 -> bf16 bits, round to nearest even; NaN -> 0x7FC0.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  const uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0u;
+  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+// fp32 -> f16 bits, round to nearest even; NaN -> 0x7E00.
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+  const uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7e00u;
+  _Float16 h = (_Float16)f; // v_cvt_f16_f32: RNE
+  uint16_t b;
+  __builtin_memcpy(&b, &h, 2);
+  return b;
+}
+
+template <int SRC_DTYPE>
+__device__ __forceinline__ float half_bits_to_f32(uint32_t h) {
+  if constexpr (SRC_DTYPE == EMM_DTYPE_BF16)
+    return bf16_bits_to_f32(h);
+  else
+    return f16_bits_to_f32(h);
+}
+
+// 8 sixteen-bit values (one u32x4) -> 8 e4m3fn bytes (one u32x2), q = rne(x / scale)
+template <int SRC_DTYPE>
+__device__ __forceinline__ u32x2 quant8(u32x4 in, float scale) {
+  u32x2 out;
+#pragma unroll
+  for (int w = 0; w < 2; ++w) {
+    uint32_t acc = 0;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const uint32_t word = in[w * 2 + k];
+      const float lo = half_bits_to_f32<SRC_DTYPE>(word & 0xffffu) / scale;
+      const float hi = half_bits_to_f32<SRC_DTYPE>(word >> 16) / scale;
+      acc |= (f32_to_e4m3fn(lo) | (f32_to_e4m3fn(hi) << 8)) << (16 * k);
+    }
+    out[w] = acc;
+  }
+  return out;
+}
+
+// 16 e4m3fn bytes (one u32x4) -> 16 sixteen-bit values (two u32x4)
+template <int OUT_DTYPE>
+__device__ __forceinline__ void dequant16(u32x4 in, float scale, u32x4 &o0, u32x4 &o1) {
+  uint32_t o[8];
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const uint32_t b0 = (in[w] >> (16 * k)) & 0xffu;
+      const uint32_t b1 = (in[w] >> (16 * k + 8)) & 0xffu;
+      const float f0 = e4m3fn_to_f32(b0) * scale;
+      const float f1 = e4m3fn_to_f32(b1) * scale;
+      uint32_t h0, h1;
+      if constexpr (OUT_DTYPE == EMM_DTYPE_BF16) {
+        h0 = f32_to_bf16_bits(f0);
+        h1 = f32_to_bf16_bits(f1);
+      } else {
+        h0 = f32_to_f16_bits(f0);
+        h1 = f32_to_f16_bits(f1);
+      }
+      o[w * 2 + k] = h0 | (h1 << 16);
+    }
+  }
+  o0 = u32x4{o[0], o[1], o[2], o[3]};
+  o1 = u32x4{o[4], o[5], o[6], o[7]};
+}
+
+// ----------------------------------------------------------------------------
+// dequant-unpack: fp8 transfer buffer -> 16-bit pool
+// ----------------------------------------------------------------------------
+struct DequantParams {
+  char *dst_layers[EMM_MAX_LAYERS];
+  const char *packed;
+  const int64_t *dst_idx;
+  const float *k_scales;
+  const float *v_scales;
+  int64_t dst_num_blocks;
+  int64_t chunk_elems; // fp8 bytes per chunk == elements
+  int64_t n;
+  uint32_t tiles_per_chunk;
+};
+
+// Tile = U * 256 lanes * 16 fp8 bytes in, twice that out.
+// grid: x = n * tiles_per_chunk, y = 2 (K, V), z = num_layers.
+template <int U, int OUT_DTYPE>
+__global__ __launch_bounds__(kThreads) void emm_unpack_dequant_fp8_kernel(
+    const DequantParams p) {
+  constexpr int64_t TILE = (int64_t)U * kThreads * 16;
+  uint32_t j = blockIdx.x, tile = 0;
+  if (p.tiles_per_chunk != 1) {
+    j = blockIdx.x / p.tiles_per_chunk;
+    tile = blockIdx.x - j * p.tiles_per_chunk;
+  }
+  const uint32_t kv = blockIdx.y, l = blockIdx.z;
+  const int64_t b = p.dst_idx[j];
+  if ((uint64_t)b >= (uint64_t)p.dst_num_blocks) return;
+  const float scale = kv == 0 ? p.k_scales[l] : p.v_scales[l];
+  const int64_t chunk = p.chunk_elems;
+  const int64_t tile_off = (int64_t)tile * TILE;
+  const char *src = p.packed + (((int64_t)l * 2 + kv) * p.n + j) * chunk + tile_off;
+  char *dst = p.dst_layers[l] + (((int64_t)kv * p.dst_num_blocks + b) * chunk + tile_off) * 2;
+  const int64_t limit = chunk - tile_off;
+  u32x4 v[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int64_t off = ((int64_t)u * kThreads + threadIdx.x) * 16;
+    if (off < limit) v[u] = ld<u32x4, true>(src + off);
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int64_t off = ((int64_t)u * kThreads + threadIdx.x) * 16;
+    if (off < limit) {
+      u32x4 o0, o1;
+      dequant16<OUT_DTYPE>(v[u], scale, o0, o1);
+      st<u32x4, true>(dst + off * 2, o0);
+      st<u32x4, true>(dst + off * 2 + 16, o1);
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------
+// reshape_and_cache: row scatter by slot_mapping
+// ----------------------------------------------------------------------------
+struct AppendParams {
+  const char *key[EMM_MAX_LAYERS];
+  const char *value[EMM_MAX_LAYERS];
+  char *key_cache[EMM_MAX_LAYERS];
+  char *value_cache[EMM_MAX_LAYERS];
+  const int64_t *slot_mapping;
+  const float *k_scales; // fp8 only
+  const float *v_scales;
+  int64_t num_tokens;
+  int64_t row_bytes;  // source row bytes (copy) / source row elements (fp8)
+  int64_t key_stride; // bytes (copy) / elements (fp8)
+  int64_t value_stride;
+  int64_t num_slots;
+};
+
+constexpr int kRowsPerWave = 4;
+constexpr int kWavesPerGroup = kThreads / 64;
+
+// One wave moves kRowsPerWave token rows of K or V. grid: x = token groups,
+// y = 2 (K, V), z = layers.
+template <typename V, bool NT>
+__global__ __launch_bounds__(kThreads) void emm_append_kernel(const AppendParams p) {
+  constexpr int64_t VB = sizeof(V);
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const uint32_t kv = blockIdx.y, l = blockIdx.z;
+  const int64_t t0 = ((int64_t)blockIdx.x * kWavesPerGroup + wave) * kRowsPerWave;
+  const char *src_base = kv == 0 ? p.key[l] : p.value[l];
+  char *dst_base = kv == 0 ? p.key_cache[l] : p.value_cache[l];
+  const int64_t stride = kv == 0 ? p.key_stride : p.value_stride;
+
+  int64_t slot[kRowsPerWave];
+#pragma unroll
+  for (int r = 0; r < kRowsPerWave; ++r) {
+    const int64_t t = t0 + r;
+    int64_t s = -1;
+    if (t < p.num_tokens) s = p.slot_mapping[t];
+    // wave-uniform: keep the slot and everything derived from it scalar
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)s);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)s >> 32));
+    s = (int64_t)(((uint64_t)hi << 32) | lo);
+    if ((uint64_t)s >= (uint64_t)p.num_slots) s = -1;
+    slot[r] = s;
+  }
+  for (int64_t off = (int64_t)lane * VB; off < p.row_bytes; off += 64 * VB) {
+    V v[kRowsPerWave];
+#pragma unroll
+    for (int r = 0; r < kRowsPerWave; ++r)
+      if (slot[r] >= 0) v[r] = ld<V, NT>(src_base + (t0 + r) * stride + off);
+#pragma unroll
+    for (int r = 0; r < kRowsPerWave; ++r)
+      if (slot[r] >= 0) st<V, NT>(dst_base + slot[r] * p.row_bytes + off, v[r]);
+  }
+}
+
+// fp8 append: each lane converts 8 contiguous 16-bit elements (16 B) into
+// 8 fp8 bytes (8 B) per step; a wave covers 512 elements per step.
+template <int SRC_DTYPE, int VEC_ELEMS>
+__global__ __launch_bounds__(kThreads) void emm_append_fp8_kernel(const AppendParams p) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const uint32_t kv = blockIdx.y, l = blockIdx.z;
+  const int64_t t0 = ((int64_t)blockIdx.x * kWavesPerGroup + wave) * kRowsPerWave;
+  const char *src_base = kv == 0 ? p.key[l] : p.value[l];
+  char *dst_base = kv == 0 ? p.key_cache[l] : p.value_cache[l];
+  const int64_t stride = kv == 0 ? p.key_stride : p.value_stride;
+  const float scale = kv == 0 ? p.k_scales[l] : p.v_scales[l];
+  const int64_t row = p.row_bytes; // elements
+
+  int64_t slot[kRowsPerWave];
+#pragma unroll
+  for (int r = 0; r < kRowsPerWave; ++r) {
+    const int64_t t = t0 + r;
+    int64_t s = -1;
+    if (t < p.num_tokens) s = p.slot_mapping[t];
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)s);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)s >> 32));
+    s = (int64_t)(((uint64_t)hi << 32) | lo);
+    if ((uint64_t)s >= (uint64_t)p.num_slots) s = -1;
+    slot[r] = s;
+  }
+  if constexpr (VEC_ELEMS == 8) {
+    for (int64_t e = (int64_t)lane * 8; e < row; e += 64 * 8) {
+      u32x4 v[kRowsPerWave];
+#pragma unroll
+      for (int r = 0; r < kRowsPerWave; ++r)
+        if (slot[r] >= 0) v[r] = ld<u32x4, true>(src_base + ((t0 + r) * stride + e) * 2);
+#pragma unroll
+      for (int r = 0; r < kRowsPerWave; ++r)
+        if (slot[r] >= 0)
+          st<u32x2, true>(dst_base + slot[r] * row + e, quant8<SRC_DTYPE>(v[r], scale));
+    }
+  } else {
+    // element-wise path for rows that are not a multiple of 8 elements or
+    // misaligned bases
+    for (int64_t e = lane; e < row; e += 64) {
+#pragma unroll
+      for (int r = 0; r < kRowsPerWave; ++r) {
+        if (slot[r] >= 0) {
+          const uint16_t h = *reinterpret_cast<const uint16_t *>(src_base + ((t0 + r) * stride + e) * 2);
+          const float x = half_bits_to_f32<SRC_DTYPE>(h) / scale;
+          *reinterpret_cast<uint8_t *>(dst_base + slot[r] * row + e) = (uint8_t)f32_to_e4m3fn(x);
+        }
+      }
+    }
+  }
+}
+
+dim3 append_grid(int64_t num_tokens, int num_layers) {
+  const int64_t rows_per_group = (int64_t)kWavesPerGroup * kRowsPerWave;
+  return dim3((uint32_t)((num_tokens + rows_per_group - 1) / rows_per_group), 2, (uint32_t)num_layers);
+}
+
+int check_append_args(const char *what, const void *const *k, const void *const *v,
+                      void *const *kc, void *const *vc, int num_layers,
+                      const int64_t *slot_mapping, int64_t num_tokens, int64_t row,
+                      int64_t ks, int64_t vs, int64_t num_slots) {
+  if (num_layers < 0 || num_layers > EMM_MAX_LAYERS)
+    return fail(EMM_EINVAL, "%s: num_layers=%d outside [0, %d]", what, num_layers, EMM_MAX_LAYERS);
+  if (num_tokens < 0 || row < 0 || num_slots < 0 || ks < 0 || vs < 0)
+    return fail(EMM_EINVAL, "%s: negative size", what);
+  if (num_tokens == 0 || num_layers == 0 || row == 0) return EMM_OK;
+  if (!slot_mapping) return fail(EMM_EINVAL, "%s: slot_mapping is null", what);
+  if (!k || !v || !kc || !vc) return fail(EMM_EINVAL, "%s: pointer table is null", what);
+  for (int l = 0; l < num_layers; ++l)
+    if (!k[l] || !v[l] || !kc[l] || !vc[l])
+      return fail(EMM_EINVAL, "%s: null tensor pointer at layer %d", what, l);
+  if (ks < row || vs < row)
+    return fail(EMM_EINVAL, "%s: token stride smaller than the row", what);
+  if ((num_tokens + 15) / 16 > 0x7fffffffLL) return fail(EMM_EINVAL, "%s: too many tokens", what);
+  return EMM_OK;
+}
+
+int append_copy(const void *const *k, const void *const *v, void *const *kc, void *const *vc,
+                int num_layers, const int64_t *slot_mapping, int64_t num_tokens,
+                int64_t row_bytes, int64_t ks, int64_t vs, int64_t num_slots,
+                hipStream_t s, const char *what) {
+  int rc = check_append_args(what, k, v, kc, vc, num_layers, slot_mapping, num_tokens,
+                             row_bytes, ks, vs, num_slots);
+  if (rc != EMM_OK) return rc;
+  if (num_tokens == 0 || num_layers == 0 || row_bytes == 0) return EMM_OK;
+  AppendParams p;
+  memset(&p, 0, sizeof(p));
+  int al = 16;
+  for (int l = 0; l < num_layers; ++l) {
+    p.key[l] = (const char *)k[l];
+    p.value[l] = (const char *)v[l];
+    p.key_cache[l] = (char *)kc[l];
+    p.value_cache[l] = (char *)vc[l];
+    al = common_align(al, k[l]);
+    al = common_align(al, v[l]);
+    al = common_align(al, kc[l]);
+    al = common_align(al, vc[l]);
+  }
+  p.slot_mapping = slot_mapping;
+  p.num_tokens = num_tokens;
+  p.row_bytes = row_bytes;
+  p.key_stride = ks;
+  p.value_stride = vs;
+  p.num_slots = num_slots;
+  int vec = al;
+  while (vec > 1 && (row_bytes % vec || ks % vec || vs % vec)) vec >>= 1;
+  dim3 grid = append_grid(num_tokens, num_layers);
+  switch (vec) {
+  case 16: emm_append_kernel<u32x4, true><<<grid, kThreads, 0, s>>>(p); break;
+  case 8: emm_append_kernel<u32x2, true><<<grid, kThreads, 0, s>>>(p); break;
+  case 4: emm_append_kernel<uint32_t, true><<<grid, kThreads, 0, s>>>(p); break;
+  case 2: emm_append_kernel<uint16_t, true><<<grid, kThreads, 0, s>>>(p); break;
+  default: emm_append_kernel<uint8_t, true><<<grid, kThreads, 0, s>>>(p); break;
+  }
+  return check_launch(what);
+}
+
+int append_fp8(const void *const *k, const void *const *v, void *const *kc, void *const *vc,
+               int num_layers, const int64_t *slot_mapping, int64_t num_tokens,
+               int64_t row_elems, int64_t ks, int64_t vs, int64_t num_slots,
+               const float *k_scales, const float *v_scales, int src_dtype,
+               hipStream_t s, const char *what) {
+  int rc = check_append_args(what, k, v, kc, vc, num_layers, slot_mapping, num_tokens,
+                             row_elems, ks, vs, num_slots);
+  if (rc != EMM_OK) return rc;
+  if (src_dtype != EMM_DTYPE_BF16 && src_dtype != EMM_DTYPE_F16)
+    return fail(EMM_EINVAL, "%s: unknown src_dtype %d", what, src_dtype);
+  if (num_tokens == 0 || num_layers == 0 || row_elems == 0) return EMM_OK;
+  if (!k_scales || !v_scales) return fail(EMM_EINVAL, "%s: scale pointer is null", what);
+  AppendParams p;
+  memset(&p, 0, sizeof(p));
+  bool wide = (row_elems % 8 == 0) && (ks % 8 == 0) && (vs % 8 == 0);
+  for (int l = 0; l < num_layers; ++l) {
+    p.key[l] = (const char *)k[l];
+    p.value[l] = (const char *)v[l];
+    p.key_cache[l] = (char *)kc[l];
+    p.value_cache[l] = (char *)vc[l];
+    wide = wide && aligned(k[l], 16) && aligned(v[l], 16) && aligned(kc[l], 8) && aligned(vc[l], 8);
+    if (!aligned(k[l], 2) || !aligned(v[l], 2))
+      return fail(EMM_EINVAL, "%s: 16-bit source not 2-byte aligned at layer %d", what, l);
+  }
+  p.slot_mapping = slot_mapping;
+  p.k_scales = k_scales;
+  p.v_scales = v_scales;
+  p.num_tokens = num_tokens;
+  p.row_bytes = row_elems;
+  p.key_stride = ks;
+  p.value_stride = vs;
+  p.num_slots = num_slots;
+  dim3 grid = append_grid(num_tokens, num_layers);
+  if (src_dtype == EMM_DTYPE_BF16) {
+    if (wide) emm_append_fp8_kernel<EMM_DTYPE_BF16, 8><<<grid, kThreads, 0, s>>>(p);
+    else emm_append_fp8_kernel<EMM_DTYPE_BF16, 1><<<grid, kThreads, 0, s>>>(p);
+  } else {
+    if (wide) emm_append_fp8_kernel<EMM_DTYPE_F16, 8><<<grid, kThreads, 0, s>>>(p);
+    else emm_append_fp8_kernel<EMM_DTYPE_F16, 1><<<grid, kThreads, 0, s>>>(p);
+  }
+  return check_launch(what);
+}
+
+// ----------------------------------------------------------------------------
+// concat_rows: ragged segments -> one contiguous buffer
+// ----------------------------------------------------------------------------
+struct ConcatParams {
+  const char *src[EMM_MAX_SEGMENTS];
+  int64_t dst_off[EMM_MAX_SEGMENTS];
+  int64_t nbytes[EMM_MAX_SEGMENTS];
+  uint32_t tile_start[EMM_MAX_SEGMENTS + 1]; // prefix sum of tiles per segment
+  char *dst;
+  int32_t n;
+};
+
+template <typename V, int U>
+__global__ __launch_bounds__(kThreads) void emm_concat_rows_kernel(const ConcatParams p) {
+  constexpr int64_t TILE = (int64_t)U * kThreads * sizeof(V);
+  const uint32_t w = blockIdx.x;
+  // wave-uniform binary search: last segment whose first tile is <= w
+  int lo = 0, hi = p.n - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (p.tile_start[mid] <= w) lo = mid; else hi = mid - 1;
+  }
+  const int64_t off = (int64_t)(w - p.tile_start[lo]) * TILE;
+  copy_tile<V, U, true, true>(p.src[lo] + off, p.dst + p.dst_off[lo] + off, p.nbytes[lo] - off);
+}
+
+hipStream_t as_stream(emm_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+} // namespace
+
+// ============================================================================
+// C ABI
+// ============================================================================
+extern "C" {
+
+const char *emm_last_error(void) { return g_last_error; }
+int emm_abi_version(void) { return EMM_KV_ABI_VERSION; }
+
+int emm_set_move_variant(int variant) {
+  const int old = g_move_variant;
+  g_move_variant = variant;
+  return old;
+}
+
+int emm_kv_pack(const void *const *layer_ptrs, int num_layers, int num_kv,
+                int64_t num_blocks, int64_t chunk_bytes, const int64_t *block_idx,
+                int64_t n, void *packed, emm_stream_t stream) {
+  int rc = check_pool_args("emm_kv_pack", layer_ptrs, num_layers, num_kv, num_blocks, chunk_bytes, n);
+  if (rc != EMM_OK) return rc;
+  if (n == 0 || num_layers == 0 || num_kv == 0 || chunk_bytes == 0) return EMM_OK;
+  if (!block_idx || !packed) return fail(EMM_EINVAL, "emm_kv_pack: null block_idx / packed");
+  MoveParams p;
+  memset(&p, 0, sizeof(p));
+  int al = common_align(16, packed);
+  for (int l = 0; l < num_layers; ++l) {
+    p.src_layers[l] = (const char *)layer_ptrs[l];
+    al = common_align(al, layer_ptrs[l]);
+  }
+  p.dst_linear = (char *)packed;
+  p.src_idx = block_idx;
+  p.idx_stride = 1;
+  p.src_num_blocks = num_blocks;
+  p.chunk_bytes = chunk_bytes;
+  p.n = n;
+  p.num_kv = (uint32_t)num_kv;
+  return launch_move<true, false>(p, num_layers, al, as_stream(stream), "emm_kv_pack");
+}
+
+int emm_kv_unpack(void *const *layer_ptrs, int num_layers, int num_kv,
+                  int64_t num_blocks, int64_t chunk_bytes, const int64_t *block_idx,
+                  int64_t n, const void *packed, emm_stream_t stream) {
+  int rc = check_pool_args("emm_kv_unpack", (const void *const *)layer_ptrs, num_layers, num_kv,
+                           num_blocks, chunk_bytes, n);
+  if (rc != EMM_OK) return rc;
+  if (n == 0 || num_layers == 0 || num_kv == 0 || chunk_bytes == 0) return EMM_OK;
+  if (!block_idx || !packed) return fail(EMM_EINVAL, "emm_kv_unpack: null block_idx / packed");
+  MoveParams p;
+  memset(&p, 0, sizeof(p));
+  int al = common_align(16, packed);
+  for (int l = 0; l < num_layers; ++l) {
+    p.dst_layers[l] = (char *)layer_ptrs[l];
+    al = common_align(al, layer_ptrs[l]);
+  }
+  p.src_linear = (const char *)packed;
+  p.dst_idx = block_idx;
+  p.idx_stride = 1;
+  p.dst_num_blocks = num_blocks;
+  p.chunk_bytes = chunk_bytes;
+  p.n = n;
+  p.num_kv = (uint32_t)num_kv;
+  return launch_move<false, true>(p, num_layers, al, as_stream(stream), "emm_kv_unpack");
+}
+
+int emm_copy_blocks(void *const *layer_ptrs, int num_layers, int num_kv,
+                    int64_t num_blocks, int64_t chunk_bytes,
+                    const int64_t *block_mapping, int64_t num_pairs, emm_stream_t stream) {
+  int rc = check_pool_args("emm_copy_blocks", (const void *const *)layer_ptrs, num_layers, num_kv,
+                           num_blocks, chunk_bytes, num_pairs);
+  if (rc != EMM_OK) return rc;
+  if (num_pairs == 0 || num_layers == 0 || num_kv == 0 || chunk_bytes == 0) return EMM_OK;
+  if (!block_mapping) return fail(EMM_EINVAL, "emm_copy_blocks: null block_mapping");
+  MoveParams p;
+  memset(&p, 0, sizeof(p));
+  int al = 16;
+  for (int l = 0; l < num_layers; ++l) {
+    p.src_layers[l] = (const char *)layer_ptrs[l];
+    p.dst_layers[l] = (char *)layer_ptrs[l];
+    al = common_align(al, layer_ptrs[l]);
+  }
+  p.src_idx = block_mapping;
+  p.dst_idx = block_mapping + 1;
+  p.idx_stride = 2;
+  p.src_num_blocks = num_blocks;
+  p.dst_num_blocks = num_blocks;
+  p.chunk_bytes = chunk_bytes;
+  p.n = num_pairs;
+  p.num_kv = (uint32_t)num_kv;
+  return launch_move<true, true>(p, num_layers, al, as_stream(stream), "emm_copy_blocks");
+}
+
+int emm_kv_migrate(const void *const *src_layer_ptrs, int64_t src_num_blocks,
+                   void *const *dst_layer_ptrs, int64_t dst_num_blocks, int num_layers,
+                   int num_kv, int64_t chunk_bytes, const int64_t *src_idx,
+                   const int64_t *dst_idx, int64_t n, emm_stream_t stream) {
+  int rc = check_pool_args("emm_kv_migrate", src_layer_ptrs, num_layers, num_kv, src_num_blocks,
+                           chunk_bytes, n);
+  if (rc != EMM_OK) return rc;
+  rc = check_pool_args("emm_kv_migrate", (const void *const *)dst_layer_ptrs, num_layers, num_kv,
+                       dst_num_blocks, chunk_bytes, n);
+  if (rc != EMM_OK) return rc;
+  if (n == 0 || num_layers == 0 || num_kv == 0 || chunk_bytes == 0) return EMM_OK;
+  if (!src_idx || !dst_idx) return fail(EMM_EINVAL, "emm_kv_migrate: null index array");
+  MoveParams p;
+  memset(&p, 0, sizeof(p));
+  int al = 16;
+  for (int l = 0; l < num_layers; ++l) {
+    p.src_layers[l] = (const char *)src_layer_ptrs[l];
+    p.dst_layers[l] = (char *)dst_layer_ptrs[l];
+    al = common_align(al, src_layer_ptrs[l]);
+    al = common_align(al, dst_layer_ptrs[l]);
+  }
+  p.src_idx = src_idx;
+  p.dst_idx = dst_idx;
+  p.idx_stride = 1;
+  p.src_num_blocks = src_num_blocks;
+  p.dst_num_blocks = dst_num_blocks;
+  p.chunk_bytes = chunk_bytes;
+  p.n = n;
+  p.num_kv = (uint32_t)num_kv;
+  return launch_move<true, true>(p, num_layers, al, as_stream(stream), "emm_kv_migrate");
+}
+
+int emm_stream_copy(const void *src, void *dst, int64_t nbytes, emm_stream_t stream) {
+  if (nbytes < 0) return fail(EMM_EINVAL, "emm_stream_copy: negative size");
+  if (nbytes == 0) return EMM_OK;
+  if (!src || !dst) return fail(EMM_EINVAL, "emm_stream_copy: null pointer");
+  MoveParams p;
+  memset(&p, 0, sizeof(p));
+  p.src_linear = (const char *)src;
+  p.dst_linear = (char *)dst;
+  p.chunk_bytes = nbytes;
+  p.n = 1;
+  p.num_kv = 1;
+  int al = common_align(common_align(16, src), dst);
+  return launch_move<false, false>(p, 1, al, as_stream(stream), "emm_stream_copy");
+}
+
+int emm_kv_unpack_dequant_fp8(void *const *layer_ptrs, int num_layers, int64_t num_blocks,
+                              int64_t chunk_elems, const int64_t *block_idx, int64_t n,
+                              const void *packed_fp8, const float *k_scales,
+                              const float *v_scales, int out_dtype, emm_stream_t stream) {
+  const char *what = "emm_kv_unpack_dequant_fp8";
+  int rc = check_pool_args(what, (const void *const *)layer_ptrs, num_layers, 2, num_blocks,
+                           chunk_elems, n);
+  if (rc != EMM_OK) return rc;
+  if (out_dtype != EMM_DTYPE_BF16 && out_dtype != EMM_DTYPE_F16)
+    return fail(EMM_EINVAL, "%s: unknown out_dtype %d", what, out_dtype);
+  if (n == 0 || num_layers == 0 || chunk_elems == 0) return EMM_OK;
+  if (!block_idx || !packed_fp8 || !k_scales || !v_scales)
+    return fail(EMM_EINVAL, "%s: null pointer argument", what);
+  if (chunk_elems % 16 != 0 || !aligned(packed_fp8, 16))
+    return fail(EMM_EINVAL, "%s: chunk_elems (%lld) and packed_fp8 must be multiples of 16",
+                what, (long long)chunk_elems);
+  DequantParams p;
+  memset(&p, 0, sizeof(p));
+  for (int l = 0; l < num_layers; ++l) {
+    if (!aligned(layer_ptrs[l], 16))
+      return fail(EMM_EINVAL, "%s: layer_ptrs[%d] not 16-byte aligned", what, l);
+    p.dst_layers[l] = (char *)layer_ptrs[l];
+  }
+  p.packed = (const char *)packed_fp8;
+  p.dst_idx = block_idx;
+  p.k_scales = k_scales;
+  p.v_scales = v_scales;
+  p.dst_num_blocks = num_blocks;
+  p.chunk_elems = chunk_elems;
+  p.n = n;
+  constexpr int U = 2;
+  const int64_t tile = (int64_t)U * kThreads * 16;
+  const int64_t tpc = (chunk_elems + tile - 1) / tile;
+  if (tpc > 0x7fffffffLL || n * tpc > 0x7fffffffLL)
+    return fail(EMM_EINVAL, "%s: grid too large", what);
+  p.tiles_per_chunk = (uint32_t)tpc;
+  dim3 grid((uint32_t)(n * tpc), 2, (uint32_t)num_layers);
+  if (out_dtype == EMM_DTYPE_BF16)
+    emm_unpack_dequant_fp8_kernel<U, EMM_DTYPE_BF16><<<grid, kThreads, 0, as_stream(stream)>>>(p);
+  else
+    emm_unpack_dequant_fp8_kernel<U, EMM_DTYPE_F16><<<grid, kThreads, 0, as_stream(stream)>>>(p);
+  return check_launch(what);
+}
+
+int emm_reshape_and_cache(const void *key, const void *value, void *key_cache,
+                          void *value_cache, const int64_t *slot_mapping,
+                          int64_t num_tokens, int64_t row_bytes, int64_t key_stride_bytes,
+                          int64_t value_stride_bytes, int64_t num_slots, emm_stream_t stream) {
+  return append_copy(&key, &value, &key_cache, &value_cache, 1, slot_mapping, num_tokens,
+                     row_bytes, key_stride_bytes, value_stride_bytes, num_slots,
+                     as_stream(stream), "emm_reshape_and_cache");
+}
+
+int emm_reshape_and_cache_layers(const void *const *key_ptrs, const void *const *value_ptrs,
+                                 void *const *key_cache_ptrs, void *const *value_cache_ptrs,
+                                 int num_layers, const int64_t *slot_mapping,
+                                 int64_t num_tokens, int64_t row_bytes,
+                                 int64_t key_stride_bytes, int64_t value_stride_bytes,
+                                 int64_t num_slots, emm_stream_t stream) {
+  return append_copy(key_ptrs, value_ptrs, key_cache_ptrs, value_cache_ptrs, num_layers,
+                     slot_mapping, num_tokens, row_bytes, key_stride_bytes, value_stride_bytes,
+                     num_slots, as_stream(stream), "emm_reshape_and_cache_layers");
+}
+
+int emm_reshape_and_cache_fp8(const void *key, const void *value, void *key_cache,
+                              void *value_cache, const int64_t *slot_mapping,
+                              int64_t num_tokens, int64_t row_elems, int64_t key_stride_elems,
+                              int64_t value_stride_elems, int64_t num_slots,
+                              const float *k_scale, const float *v_scale, int src_dtype,
+                              emm_stream_t stream) {
+  return append_fp8(&key, &value, &key_cache, &value_cache, 1, slot_mapping, num_tokens,
+                    row_elems, key_stride_elems, value_stride_elems, num_slots, k_scale, v_scale,
+                    src_dtype, as_stream(stream), "emm_reshape_and_cache_fp8");
+}
+
+int emm_reshape_and_cache_fp8_layers(const void *const *key_ptrs, const void *const *value_ptrs,
+                                     void *const *key_cache_ptrs, void *const *value_cache_ptrs,
+                                     int num_layers, const int64_t *slot_mapping,
+                                     int64_t num_tokens, int64_t row_elems,
+                                     int64_t key_stride_elems, int64_t value_stride_elems,
+                                     int64_t num_slots, const float *k_scales,
+                                     const float *v_scales, int src_dtype, emm_stream_t stream) {
+  return append_fp8(key_ptrs, value_ptrs, key_cache_ptrs, value_cache_ptrs, num_layers,
+                    slot_mapping, num_tokens, row_elems, key_stride_elems, value_stride_elems,
+                    num_slots, k_scales, v_scales, src_dtype, as_stream(stream),
+                    "emm_reshape_and_cache_fp8_layers");
+}
+
+int emm_concat_rows(const void *const *srcs, const int64_t *nbytes, int n, void *dst,
+                    int64_t dst_offset_bytes, emm_stream_t stream) {
+  const char *what = "emm_concat_rows";
+  if (n < 0 || n > EMM_MAX_SEGMENTS)
+    return fail(EMM_EINVAL, "%s: n=%d outside [0, %d]", what, n, EMM_MAX_SEGMENTS);
+  if (n == 0) return EMM_OK;
+  if (!srcs || !nbytes || !dst || dst_offset_bytes < 0)
+    return fail(EMM_EINVAL, "%s: null pointer / negative offset", what);
+  ConcatParams p;
+  memset(&p, 0, sizeof(p));
+  constexpr int U = 4;
+  int al = common_align(16, (const char *)dst + dst_offset_bytes);
+  int64_t off = dst_offset_bytes;
+  int m = 0;
+  for (int i = 0; i < n; ++i) {
+    if (nbytes[i] < 0) return fail(EMM_EINVAL, "%s: nbytes[%d] negative", what, i);
+    if (nbytes[i] == 0) continue;
+    if (!srcs[i]) return fail(EMM_EINVAL, "%s: srcs[%d] is null", what, i);
+    p.src[m] = (const char *)srcs[i];
+    p.dst_off[m] = off;
+    p.nbytes[m] = nbytes[i];
+    al = common_align(al, srcs[i]);
+    while (al > 1 && (off % al || nbytes[i] % al)) al >>= 1;
+    off += nbytes[i];
+    ++m;
+  }
+  if (m == 0) return EMM_OK;
+  if (al == 8) al = 4;
+  const int64_t tile = (int64_t)U * kThreads * al;
+  uint64_t tiles = 0;
+  for (int i = 0; i < m; ++i) {
+    p.tile_start[i] = (uint32_t)tiles;
+    tiles += (uint64_t)((p.nbytes[i] + tile - 1) / tile);
+    if (tiles > 0x7fffffffULL) return fail(EMM_EINVAL, "%s: grid too large", what);
+  }
+  p.tile_start[m] = (uint32_t)tiles;
+  p.dst = (char *)dst;
+  p.n = m;
+  dim3 grid((uint32_t)tiles);
+  hipStream_t s = as_stream(stream);
+  switch (al) {
+  case 16: emm_concat_rows_kernel<u32x4, U><<<grid, kThreads, 0, s>>>(p); break;
+  case 4: emm_concat_rows_kernel<uint32_t, U><<<grid, kThreads, 0, s>>>(p); break;
+  case 2: emm_concat_rows_kernel<uint16_t, U><<<grid, kThreads, 0, s>>>(p); break;
+  default: emm_concat_rows_kernel<uint8_t, U><<<grid, kThreads, 0, s>>>(p); break;
+  }
+  return check_launch(what);
+}
+
+} // extern "C"

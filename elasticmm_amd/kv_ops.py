@@ -1,0 +1,390 @@
+"""Tensor-level operators over libemm_kv.so.
+
+Every function launches on torch's current HIP stream of the tensors' device and
+returns without synchronising. torch is used for device memory and streams
+only; all data movement is done by the HIP kernels of the library.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence, Union
+
+import numpy as np
+import torch
+
+from . import _lib
+from ._lib import EMM_DTYPE_BF16, EMM_DTYPE_F16, EMM_MAX_LAYERS, EMM_MAX_SEGMENTS, check, ptr_table
+
+IndexLike = Union[Sequence[int], np.ndarray, torch.Tensor]
+
+
+def _stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require_gpu(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{what}: tensor is on {t.device}; the KV kernels run on the GPU only")
+
+
+def block_index_tensor(block_indices: IndexLike, num_blocks: int, device: torch.device) -> torch.Tensor:
+    """int64 device tensor of block ids.
+
+    A Python list / numpy array is checked on the host with the semantics torch
+    gives ``tensor[:, idx]`` (worker.py:597, :604): ids in [-num_blocks,
+    num_blocks), negatives counted from the end, anything else IndexError. It is
+    then staged through pinned memory and copied asynchronously. A device tensor
+    is used as is (int64, contiguous); the kernels skip negative or too-large
+    entries instead of faulting.
+    """
+    if isinstance(block_indices, torch.Tensor):
+        t = block_indices
+        if t.dtype != torch.long:
+            raise TypeError(f"block index tensor must be int64, got {t.dtype}")
+        if t.is_cuda:
+            return t.contiguous()
+        arr = t.numpy()
+    else:
+        arr = np.asarray(block_indices, dtype=np.int64)
+    arr = arr.reshape(-1)
+    if arr.size:
+        lo, hi = int(arr.min()), int(arr.max())
+        if lo < -num_blocks or hi >= num_blocks:
+            bad = lo if lo < -num_blocks else hi
+            raise IndexError(f"index {bad} is out of bounds for dimension 1 with size {num_blocks}")
+        if lo < 0:
+            arr = np.where(arr < 0, arr + num_blocks, arr)
+    host = torch.from_numpy(np.ascontiguousarray(arr))
+    if device.type == "cuda":
+        return host.pin_memory().to(device, non_blocking=True)
+    return host
+
+
+class PoolView:
+    """A block pool as the kernels see it: per-layer base pointers + geometry.
+
+    ``kv_cache`` is the reference's pool: a list of L tensors
+    ``[num_kv, num_blocks, block_size, num_heads, head_size]`` (worker.py:388-394,
+    :594) or one monolithic tensor ``[L, num_kv, num_blocks, ...]``
+    (nccl_transfer.py:215). Trailing dimensions are free (the vision block pool
+    ``[num_blocks, tokens, dim]`` is viewed with num_kv = 1).
+    """
+
+    def __init__(self, kv_cache: Union[Sequence[torch.Tensor], torch.Tensor], num_kv_dim: bool = True):
+        if isinstance(kv_cache, torch.Tensor):
+            layers = list(kv_cache.unbind(0))
+        else:
+            layers = list(kv_cache)
+        if not layers:
+            raise ValueError("empty KV pool")
+        first = layers[0]
+        for i, t in enumerate(layers):
+            _require_gpu(t, "PoolView")
+            if t.shape != first.shape or t.dtype != first.dtype or t.device != first.device:
+                raise ValueError(f"layer {i} differs from layer 0 in shape / dtype / device")
+            if not t.is_contiguous():
+                raise ValueError(f"layer {i} is not contiguous")
+        self.layers: List[torch.Tensor] = layers
+        self.device = first.device
+        self.dtype = first.dtype
+        self.elem_bytes = first.element_size()
+        if num_kv_dim:
+            self.num_kv = int(first.shape[0])
+            self.num_blocks = int(first.shape[1])
+            self.block_shape = tuple(first.shape[2:])
+        else:
+            self.num_kv = 1
+            self.num_blocks = int(first.shape[0])
+            self.block_shape = tuple(first.shape[1:])
+        self.chunk_elems = int(np.prod(self.block_shape, dtype=np.int64)) if self.block_shape else 1
+        self.chunk_bytes = self.chunk_elems * self.elem_bytes
+        self.ptrs = [t.data_ptr() for t in layers]
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def layer_groups(self):
+        """(first_layer, ctypes pointer table) per group of at most EMM_MAX_LAYERS layers."""
+        for l0 in range(0, self.num_layers, EMM_MAX_LAYERS):
+            yield l0, ptr_table(self.ptrs[l0:l0 + EMM_MAX_LAYERS])
+
+    def packed_shape(self, n: int):
+        return (self.num_layers, self.num_kv, n) + self.block_shape
+
+
+def kv_pack(pool: PoolView, block_indices: IndexLike, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Gather ``n`` blocks of every layer into ``[L, num_kv, n, *block_shape]``."""
+    lib = _lib.load()
+    idx = block_index_tensor(block_indices, pool.num_blocks, pool.device)
+    n = idx.numel()
+    shape = pool.packed_shape(n)
+    if out is None:
+        out = torch.empty(shape, dtype=pool.dtype, device=pool.device)
+    else:
+        if out.device != pool.device or out.dtype != pool.dtype or not out.is_contiguous() \
+                or out.numel() != int(np.prod(shape, dtype=np.int64)):
+            raise ValueError("kv_pack: `out` must be a contiguous pool-dtype tensor of the packed size")
+    stream = _stream_ptr(pool.device)
+    plane = pool.num_kv * n * pool.chunk_bytes
+    for l0, table in pool.layer_groups():
+        check(lib.emm_kv_pack(table, len(table), pool.num_kv, pool.num_blocks, pool.chunk_bytes,
+                              idx.data_ptr(), n, out.data_ptr() + l0 * plane, stream), "emm_kv_pack")
+    return out
+
+
+def kv_unpack(pool: PoolView, block_indices: IndexLike, packed: torch.Tensor) -> None:
+    """Scatter ``packed`` ``[L, num_kv, n, ...]`` into the pool under ``block_indices``."""
+    lib = _lib.load()
+    _require_gpu(packed, "kv_unpack")
+    idx = block_index_tensor(block_indices, pool.num_blocks, pool.device)
+    n = idx.numel()
+    want = pool.num_layers * pool.num_kv * n * pool.chunk_bytes
+    if packed.device != pool.device:
+        raise ValueError("kv_unpack: packed buffer is on another device")
+    if packed.numel() * packed.element_size() != want:
+        raise ValueError(f"kv_unpack: packed buffer holds {packed.numel() * packed.element_size()} bytes, "
+                         f"pool geometry needs {want}")
+    if not packed.is_contiguous():
+        packed = packed.contiguous()
+    stream = _stream_ptr(pool.device)
+    plane = pool.num_kv * n * pool.chunk_bytes
+    for l0, table in pool.layer_groups():
+        check(lib.emm_kv_unpack(table, len(table), pool.num_kv, pool.num_blocks, pool.chunk_bytes,
+                                idx.data_ptr(), n, packed.data_ptr() + l0 * plane, stream), "emm_kv_unpack")
+
+
+def kv_migrate(src: PoolView, src_indices: IndexLike, dst: PoolView, dst_indices: IndexLike) -> None:
+    """``dst[l][:, dst_idx[j]] = src[l][:, src_idx[j]]`` in one launch, no staging buffer."""
+    lib = _lib.load()
+    if (src.num_layers, src.num_kv, src.chunk_bytes, src.device) != (dst.num_layers, dst.num_kv, dst.chunk_bytes, dst.device):
+        raise ValueError("kv_migrate: pools differ in layers / kv / chunk size / device")
+    si = block_index_tensor(src_indices, src.num_blocks, src.device)
+    di = block_index_tensor(dst_indices, dst.num_blocks, dst.device)
+    if si.numel() != di.numel():
+        raise ValueError(f"Block count mismatch: src={si.numel()}, dst={di.numel()}")
+    stream = _stream_ptr(src.device)
+    for (l0, st), (_, dt) in zip(src.layer_groups(), dst.layer_groups()):
+        check(lib.emm_kv_migrate(st, src.num_blocks, dt, dst.num_blocks, len(st), src.num_kv, src.chunk_bytes,
+                                 si.data_ptr(), di.data_ptr(), si.numel(), stream), "emm_kv_migrate")
+
+
+def copy_blocks(pool: PoolView, block_mapping: Union[torch.Tensor, Sequence[Sequence[int]]]) -> None:
+    """All layers: ``pool[:, dst] = pool[:, src]`` for the (src, dst) rows of ``block_mapping``."""
+    lib = _lib.load()
+    if isinstance(block_mapping, torch.Tensor):
+        m = block_mapping
+        if m.dtype != torch.long or m.dim() != 2 or m.shape[1] != 2:
+            raise ValueError("block_mapping must be an int64 tensor of shape [num_pairs, 2]")
+        if not m.is_cuda:
+            m = block_index_tensor(m.reshape(-1), pool.num_blocks, pool.device).view(-1, 2)
+        m = m.contiguous()
+    else:
+        arr = np.asarray(block_mapping, dtype=np.int64).reshape(-1, 2)
+        m = block_index_tensor(arr.reshape(-1), pool.num_blocks, pool.device).view(-1, 2)
+    stream = _stream_ptr(pool.device)
+    for _, table in pool.layer_groups():
+        check(lib.emm_copy_blocks(table, len(table), pool.num_kv, pool.num_blocks, pool.chunk_bytes,
+                                  m.data_ptr(), m.shape[0], stream), "emm_copy_blocks")
+
+
+def _half_code(dt: torch.dtype, what: str) -> int:
+    if dt == torch.bfloat16:
+        return EMM_DTYPE_BF16
+    if dt == torch.float16:
+        return EMM_DTYPE_F16
+    raise TypeError(f"{what}: 16-bit side must be bfloat16 or float16, got {dt}")
+
+
+def _scales_tensor(scales, num_layers: int, device: torch.device) -> torch.Tensor:
+    t = scales if isinstance(scales, torch.Tensor) else torch.tensor(scales, dtype=torch.float32)
+    t = t.to(device=device, dtype=torch.float32).reshape(-1).contiguous()
+    if t.numel() != num_layers:
+        raise ValueError(f"expected {num_layers} per-layer scales, got {t.numel()}")
+    return t
+
+
+def kv_unpack_dequant_fp8(pool: PoolView, block_indices: IndexLike, packed_fp8: torch.Tensor,
+                          k_scales, v_scales) -> None:
+    """Scatter an fp8-e4m3fn transfer buffer ``[L, 2, n, ...]`` into a bf16/f16 pool,
+    ``out = rne16(float(q) * scale)`` with per-layer K and V scales."""
+    lib = _lib.load()
+    _require_gpu(packed_fp8, "kv_unpack_dequant_fp8")
+    if pool.num_kv != 2:
+        raise ValueError("kv_unpack_dequant_fp8 needs a [2, num_blocks, ...] pool")
+    if packed_fp8.element_size() != 1:
+        raise TypeError("packed_fp8 must be a 1-byte tensor (float8_e4m3fn or uint8)")
+    code = _half_code(pool.dtype, "kv_unpack_dequant_fp8")
+    idx = block_index_tensor(block_indices, pool.num_blocks, pool.device)
+    n = idx.numel()
+    if packed_fp8.numel() != pool.num_layers * 2 * n * pool.chunk_elems:
+        raise ValueError("kv_unpack_dequant_fp8: packed buffer size does not match the pool geometry")
+    packed_fp8 = packed_fp8.contiguous()
+    ks = _scales_tensor(k_scales, pool.num_layers, pool.device)
+    vs = _scales_tensor(v_scales, pool.num_layers, pool.device)
+    stream = _stream_ptr(pool.device)
+    plane = 2 * n * pool.chunk_elems
+    for l0, table in pool.layer_groups():
+        check(lib.emm_kv_unpack_dequant_fp8(table, len(table), pool.num_blocks, pool.chunk_elems, idx.data_ptr(), n,
+                                            packed_fp8.data_ptr() + l0 * plane, ks.data_ptr() + 4 * l0,
+                                            vs.data_ptr() + 4 * l0, code, stream), "emm_kv_unpack_dequant_fp8")
+
+
+def _row_geometry(x: torch.Tensor, what: str):
+    """(num_tokens, row_elems, token_stride_elems) of a [T, ...] tensor whose rows are contiguous."""
+    if x.dim() < 1:
+        raise ValueError(f"{what}: expected [num_tokens, ...]")
+    T = int(x.shape[0])
+    row = int(np.prod(x.shape[1:], dtype=np.int64)) if x.dim() > 1 else 1
+    if T > 0 and x.dim() > 1 and not x[0].is_contiguous():
+        raise ValueError(f"{what}: rows must be contiguous (only the token dimension may be strided)")
+    stride = int(x.stride(0)) if T > 1 else row
+    return T, row, stride
+
+
+def _cache_slots(cache: torch.Tensor, row_elems: int, what: str) -> int:
+    if not cache.is_contiguous():
+        raise ValueError(f"{what}: cache plane must be contiguous")
+    if row_elems == 0:
+        return 0
+    if cache.numel() % row_elems:
+        raise ValueError(f"{what}: cache size is not a multiple of the token row")
+    return cache.numel() // row_elems
+
+
+def reshape_and_cache(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
+                      slot_mapping: torch.Tensor, k_scale: Optional[torch.Tensor] = None,
+                      v_scale: Optional[torch.Tensor] = None) -> None:
+    """Append one layer: ``cache.view(slots, row)[slot_mapping[t]] = cvt(x[t])`` for slots >= 0.
+
+    Same-width caches are copied bit for bit; a 1-byte cache with a 16-bit source
+    is quantised to fp8-e4m3fn with ``k_scale`` / ``v_scale`` (one float each)."""
+    lib = _lib.load()
+    for t, nm in ((key, "key"), (value, "value"), (key_cache, "key_cache"), (value_cache, "value_cache"),
+                  (slot_mapping, "slot_mapping")):
+        _require_gpu(t, f"reshape_and_cache({nm})")
+    if slot_mapping.dtype != torch.long:
+        raise TypeError("slot_mapping must be int64")
+    slot_mapping = slot_mapping.contiguous()
+    T, row, ks = _row_geometry(key, "key")
+    Tv, rowv, vs = _row_geometry(value, "value")
+    if (T, row) != (Tv, rowv):
+        raise ValueError("key and value differ in shape")
+    if slot_mapping.numel() < T:
+        raise ValueError("slot_mapping is shorter than the token count")
+    T = min(T, slot_mapping.numel())
+    num_slots = _cache_slots(key_cache, row, "key_cache")
+    if _cache_slots(value_cache, row, "value_cache") != num_slots:
+        raise ValueError("key_cache and value_cache differ in size")
+    stream = _stream_ptr(key.device)
+    eb = key.element_size()
+    if key_cache.element_size() == eb:
+        check(lib.emm_reshape_and_cache(key.data_ptr(), value.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(),
+                                        slot_mapping.data_ptr(), T, row * eb, ks * eb, vs * eb, num_slots, stream),
+              "emm_reshape_and_cache")
+    elif key_cache.element_size() == 1 and eb == 2:
+        if k_scale is None or v_scale is None:
+            raise ValueError("fp8 cache needs k_scale and v_scale")
+        code = _half_code(key.dtype, "reshape_and_cache")
+        k_s = _scales_tensor(k_scale, 1, key.device)
+        v_s = _scales_tensor(v_scale, 1, key.device)
+        check(lib.emm_reshape_and_cache_fp8(key.data_ptr(), value.data_ptr(), key_cache.data_ptr(),
+                                            value_cache.data_ptr(), slot_mapping.data_ptr(), T, row, ks, vs,
+                                            num_slots, k_s.data_ptr(), v_s.data_ptr(), code, stream),
+              "emm_reshape_and_cache_fp8")
+    else:
+        raise TypeError(f"unsupported source/cache element sizes {eb}/{key_cache.element_size()}")
+
+
+def reshape_and_cache_layers(keys: Sequence[torch.Tensor], values: Sequence[torch.Tensor],
+                             key_caches: Sequence[torch.Tensor], value_caches: Sequence[torch.Tensor],
+                             slot_mapping: torch.Tensor, k_scales=None, v_scales=None) -> None:
+    """Append all layers of one step in a single launch (per group of EMM_MAX_LAYERS)."""
+    lib = _lib.load()
+    L = len(keys)
+    if not (len(values) == len(key_caches) == len(value_caches) == L):
+        raise ValueError("per-layer lists differ in length")
+    if L == 0:
+        return
+    _require_gpu(keys[0], "reshape_and_cache_layers")
+    if slot_mapping.dtype != torch.long:
+        raise TypeError("slot_mapping must be int64")
+    slot_mapping = slot_mapping.contiguous()
+    T, row, ks = _row_geometry(keys[0], "key")
+    _, _, vs = _row_geometry(values[0], "value")
+    for l in range(L):
+        if _row_geometry(keys[l], "key") != (T, row, ks) or _row_geometry(values[l], "value") != (T, row, vs):
+            raise ValueError(f"layer {l}: key/value geometry differs from layer 0")
+    if slot_mapping.numel() < T:
+        raise ValueError("slot_mapping is shorter than the token count")
+    num_slots = _cache_slots(key_caches[0], row, "key_cache")
+    for l in range(L):
+        if _cache_slots(key_caches[l], row, "key_cache") != num_slots or \
+                _cache_slots(value_caches[l], row, "value_cache") != num_slots:
+            raise ValueError(f"layer {l}: cache size differs from layer 0")
+    dev = keys[0].device
+    stream = _stream_ptr(dev)
+    eb = keys[0].element_size()
+    ceb = key_caches[0].element_size()
+    fp8 = ceb == 1 and eb == 2
+    if not fp8 and ceb != eb:
+        raise TypeError(f"unsupported source/cache element sizes {eb}/{ceb}")
+    if fp8:
+        code = _half_code(keys[0].dtype, "reshape_and_cache_layers")
+        k_s = _scales_tensor(k_scales, L, dev)
+        v_s = _scales_tensor(v_scales, L, dev)
+    for l0 in range(0, L, EMM_MAX_LAYERS):
+        sl = slice(l0, l0 + EMM_MAX_LAYERS)
+        kt = ptr_table([t.data_ptr() for t in keys[sl]])
+        vt = ptr_table([t.data_ptr() for t in values[sl]])
+        kct = ptr_table([t.data_ptr() for t in key_caches[sl]])
+        vct = ptr_table([t.data_ptr() for t in value_caches[sl]])
+        if fp8:
+            check(lib.emm_reshape_and_cache_fp8_layers(kt, vt, kct, vct, len(kt), slot_mapping.data_ptr(), T, row,
+                                                       ks, vs, num_slots, k_s.data_ptr() + 4 * l0,
+                                                       v_s.data_ptr() + 4 * l0, code, stream),
+                  "emm_reshape_and_cache_fp8_layers")
+        else:
+            check(lib.emm_reshape_and_cache_layers(kt, vt, kct, vct, len(kt), slot_mapping.data_ptr(), T, row * eb,
+                                                   ks * eb, vs * eb, num_slots, stream),
+                  "emm_reshape_and_cache_layers")
+
+
+def concat_rows(tensors: Sequence[torch.Tensor], out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``torch.cat(tensors, dim=0)`` of ragged ``[rows_i, ...]`` tensors in one launch per
+    EMM_MAX_SEGMENTS segments."""
+    lib = _lib.load()
+    tensors = list(tensors)
+    if not tensors:
+        raise ValueError("concat_rows: expected a non-empty list of tensors")
+    first = tensors[0]
+    for t in tensors:
+        _require_gpu(t, "concat_rows")
+        if t.shape[1:] != first.shape[1:] or t.dtype != first.dtype or t.device != first.device:
+            raise ValueError("concat_rows: tensors differ in trailing shape / dtype / device")
+    tensors = [t if t.is_contiguous() else t.contiguous() for t in tensors]
+    rows = sum(int(t.shape[0]) for t in tensors)
+    shape = (rows,) + tuple(first.shape[1:])
+    if out is None:
+        out = torch.empty(shape, dtype=first.dtype, device=first.device)
+    elif tuple(out.shape) != shape or out.dtype != first.dtype or not out.is_contiguous():
+        raise ValueError("concat_rows: `out` has the wrong shape / dtype or is not contiguous")
+    stream = _stream_ptr(first.device)
+    off = 0
+    for i0 in range(0, len(tensors), EMM_MAX_SEGMENTS):
+        seg = tensors[i0:i0 + EMM_MAX_SEGMENTS]
+        srcs = ptr_table([t.data_ptr() for t in seg])
+        sizes = [t.numel() * t.element_size() for t in seg]
+        nbytes = (_lib.c_int64 * len(seg))(*sizes)
+        check(lib.emm_concat_rows(srcs, nbytes, len(seg), out.data_ptr(), off, stream), "emm_concat_rows")
+        off += sum(sizes)
+    return out
+
+
+def stream_copy(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """Plain device copy with the block-move tile engine (benchmark yardstick)."""
+    lib = _lib.load()
+    _require_gpu(src, "stream_copy")
+    nbytes = src.numel() * src.element_size()
+    if dst.numel() * dst.element_size() != nbytes or not src.is_contiguous() or not dst.is_contiguous():
+        raise ValueError("stream_copy: contiguous tensors of equal byte size required")
+    check(lib.emm_stream_copy(src.data_ptr(), dst.data_ptr(), nbytes, _stream_ptr(src.device)), "emm_stream_copy")

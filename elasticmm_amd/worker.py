@@ -1,0 +1,338 @@
+"""KVWorker — the KV data-path surface of the reference's V0Worker on one MI355X.
+
+Method names, argument order, return shapes and error behaviour follow
+``elasticmm/engine/v0/worker.py`` (the class ``V0Worker``), restricted to the
+methods that touch KV / vision-embedding tensors:
+
+  extract_kv_blocks / write_kv_blocks / get_kv_cache_layout   worker.py:578-647
+  p2p_send_kv / p2p_recv_kv                                   worker.py:665-731
+  p2p_coordinated_transfer_kv                                 worker.py:733-871
+  p2p_pull_kv / p2p_serve_kv                                  worker.py:873-937
+  collective_transfer_kv                                      worker.py:939-1005
+  extract_vision_blocks / write_vision_blocks                 worker.py:1007-1036
+  init_kvcache (pool allocation only)                         worker.py:358-418
+
+Model loading, Ray actor plumbing and step_* execution are not part of this
+class. The cross-GPU hop (``torch.distributed.send/recv``) is replaced by a
+``LoopbackLink``: a same-device FIFO that hands the sender's transfer buffer to
+the receiver, which unpacks it into its own, independently allocated pool.
+Where the reference loops over layers with one gather / scatter launch each,
+this class issues one kernel launch for all layers.
+"""
+from __future__ import annotations
+
+import collections
+import math
+import time
+from typing import Any, Deque, Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from . import kv_ops
+from .kv_ops import PoolView
+
+_DTYPES = {
+    "float16": torch.float16, "half": torch.float16, "fp16": torch.float16,
+    "bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
+    "float32": torch.float32, "fp32": torch.float32,
+}
+
+
+class LoopbackLink:
+    """Same-device stand-in for the global NCCL group: per (src, dst, tag) FIFOs of
+    device tensors. ``send`` enqueues a tensor, ``recv`` dequeues it; both sides run
+    on the same HIP stream order, so no extra synchronisation is needed."""
+
+    def __init__(self, world_size: int = 2):
+        self.world_size = world_size
+        self._queues: Dict[Tuple[int, int, int], Deque[torch.Tensor]] = collections.defaultdict(collections.deque)
+
+    def send(self, tensor: torch.Tensor, src: int, dst: int, tag: int = 0) -> None:
+        if not (0 <= dst < self.world_size):
+            raise ValueError(f"Invalid dst rank: {dst} (world_size={self.world_size})")
+        self._queues[(src, dst, tag)].append(tensor)
+
+    def recv(self, src: int, dst: int, tag: int = 0) -> torch.Tensor:
+        q = self._queues[(src, dst, tag)]
+        if not q:
+            raise RuntimeError(f"no message pending from rank {src} to rank {dst} (tag {tag})")
+        return q.popleft()
+
+    def pending(self, src: int, dst: int, tag: int = 0) -> int:
+        return len(self._queues[(src, dst, tag)])
+
+
+class KVWorker:
+    """Owns one block pool on one GPU and moves blocks in and out of it."""
+
+    def __init__(self, worker_id: int = 0, device: str = "cuda:0", block_size: int = 16,
+                 link: Optional[LoopbackLink] = None, global_rank: Optional[int] = None):
+        self.worker_id = worker_id
+        self.device = torch.device(device)
+        self.block_size = block_size
+        self.kv_cache: Optional[List[torch.Tensor]] = None
+        self.ve_cache: Optional[Dict[str, torch.Tensor]] = None
+        self._pool: Optional[PoolView] = None
+        self.link = link
+        self.global_rank = global_rank
+        self.nccl_pg_initialized = link is not None and global_rank is not None
+        self.peers: Dict[int, "KVWorker"] = {}
+
+    # ----- pool -----------------------------------------------------------
+    def init_kvcache(self, num_gpu_blocks: int, num_cpu_blocks: int = 0, *, num_layers: int, num_kv_heads: int,
+                     head_size: int, dtype: torch.dtype = torch.bfloat16, monolithic: bool = True) -> List[int]:
+        """Allocate the pool: L tensors ``[2, num_gpu_blocks, block_size, num_kv_heads, head_size]``
+        (worker.py:388-394). With ``monolithic`` the L tensors are views of one
+        allocation, which keeps the list API and lets the whole pool be one HBM
+        region; otherwise each layer is its own allocation as vLLM's CacheEngine does."""
+        shape = (2, num_gpu_blocks, self.block_size, num_kv_heads, head_size)
+        if monolithic:
+            whole = torch.empty((num_layers,) + shape, dtype=dtype, device=self.device)
+            layers = list(whole.unbind(0))
+        else:
+            layers = [torch.empty(shape, dtype=dtype, device=self.device) for _ in range(num_layers)]
+        self.bind_kv_cache(layers)
+        return []  # placeholder for an IPC handle, as in the reference (worker.py:418)
+
+    def bind_kv_cache(self, kv_cache: Sequence[torch.Tensor]) -> None:
+        """Adopt an existing pool (e.g. the list vLLM's CacheEngine allocated)."""
+        self.kv_cache = list(kv_cache)
+        self._pool = PoolView(self.kv_cache)
+
+    def init_vecache(self, num_gpu_blocks: int = 0, num_cpu_blocks: int = 0) -> List[int]:
+        """Vision embeddings are kept per request id (worker.py:431-437)."""
+        self.ve_cache = {}
+        self.ve_cache_capacity = num_gpu_blocks
+        return []
+
+    @property
+    def pool(self) -> PoolView:
+        if self._pool is None:
+            raise RuntimeError("KV cache not initialized")
+        return self._pool
+
+    # ----- extract / write (worker.py:578-647) ------------------------------
+    def extract_kv_blocks(self, block_indices: List[int]) -> torch.Tensor:
+        """-> ``[num_layers, 2, n, block_size, num_heads, head_size]``, one launch."""
+        if self.kv_cache is None:
+            raise RuntimeError("KV cache not initialized")
+        return kv_ops.kv_pack(self.pool, block_indices)
+
+    def write_kv_blocks(self, block_indices: List[int], kv_data: torch.Tensor) -> None:
+        if self.kv_cache is None:
+            raise RuntimeError("KV cache not initialized")
+        assert kv_data.shape[2] == len(block_indices), \
+            f"Block count mismatch: {kv_data.shape[2]} vs {len(block_indices)}"
+        if kv_data.dtype != self.pool.dtype:
+            kv_data = kv_data.to(self.pool.dtype)
+        if kv_data.device != self.device:
+            kv_data = kv_data.to(self.device)
+        kv_ops.kv_unpack(self.pool, block_indices, kv_data)
+
+    def get_kv_cache_layout(self) -> Dict[str, Any]:
+        if not self.kv_cache:
+            return {}
+        sample_layer = self.kv_cache[0]
+        return {
+            "num_layers": len(self.kv_cache),
+            "block_size": sample_layer.shape[2],
+            "num_heads": sample_layer.shape[3],
+            "head_size": sample_layer.shape[4],
+            "dtype": str(sample_layer.dtype).split(".")[-1],
+        }
+
+    # ----- P2P (worker.py:649-937) over the loopback link -------------------
+    def init_global_nccl(self) -> bool:
+        return bool(self.nccl_pg_initialized)
+
+    def get_global_rank(self) -> int:
+        return self.global_rank if self.global_rank is not None else -1
+
+    def _layer_bytes(self, n: int) -> int:
+        return self.pool.num_kv * n * self.pool.chunk_bytes
+
+    def p2p_send_kv(self, dst_rank: int, block_indices: List[int]) -> Dict[str, Any]:
+        """Pack all layers with one launch, then hand the link one ``[2, n, bs, H, D]``
+        message per layer (views of the one transfer buffer), as the reference sends
+        one message per layer."""
+        if not self.nccl_pg_initialized:
+            return {"error": "Global NCCL not initialized", "bytes": 0, "blocks": 0}
+        try:
+            packed = kv_ops.kv_pack(self.pool, block_indices)
+            total_bytes = 0
+            for l in range(self.pool.num_layers):
+                layer_data = packed[l]
+                self.link.send(layer_data, src=self.global_rank, dst=dst_rank)
+                total_bytes += layer_data.numel() * layer_data.element_size()
+            torch.cuda.synchronize(self.device)
+            return {"bytes": total_bytes, "blocks": len(block_indices)}
+        except Exception as e:  # transport failures are reported, not raised (worker.py:686-691)
+            error_msg = f"NCCL send failed: {type(e).__name__}: {str(e)}"
+            return {"error": error_msg, "bytes": 0, "blocks": 0}
+
+    def _recv_layers(self, src_rank: int, block_indices: List[int], tagged: bool = False,
+                     deadline: Optional[Tuple[float, float]] = None) -> Any:
+        """Receive L per-layer messages and scatter them. Messages that are the
+        consecutive slices of one transfer buffer are scattered with one launch."""
+        pool = self.pool
+        n = len(block_indices)
+        layer_shape = (pool.num_kv, n) + pool.block_shape
+        msgs: List[torch.Tensor] = []
+        for layer_idx in range(pool.num_layers):
+            if deadline is not None and time.time() - deadline[0] > deadline[1]:
+                return layer_idx
+            m = self.link.recv(src=src_rank, dst=self.global_rank, tag=layer_idx if tagged else 0)
+            if tuple(m.shape) != layer_shape:
+                raise RuntimeError(f"layer {layer_idx}: received {tuple(m.shape)}, expected {layer_shape}")
+            msgs.append(m)
+        total_bytes = sum(m.numel() * m.element_size() for m in msgs)
+        step = self._layer_bytes(n)
+        whole = msgs[0]._base if msgs else None
+        fused = (whole is not None and whole.is_contiguous()
+                 and whole.numel() == sum(m.numel() for m in msgs)
+                 and all(m._base is whole and m.is_contiguous()
+                         and m.data_ptr() == whole.data_ptr() + i * step for i, m in enumerate(msgs)))
+        if fused:
+            kv_ops.kv_unpack(pool, block_indices, whole)
+        else:
+            idx = kv_ops.block_index_tensor(block_indices, pool.num_blocks, pool.device)
+            for l, m in enumerate(msgs):
+                kv_ops.kv_unpack(PoolView([pool.layers[l]]), idx, m)
+        return {"bytes": total_bytes}
+
+    def p2p_recv_kv(self, src_rank: int, block_indices: List[int]) -> Dict[str, Any]:
+        if not self.nccl_pg_initialized:
+            return {"error": "Global NCCL not initialized", "bytes": 0, "blocks": 0}
+        try:
+            res = self._recv_layers(src_rank, block_indices)
+            torch.cuda.synchronize(self.device)
+            return {"bytes": res["bytes"], "blocks": len(block_indices)}
+        except Exception as e:
+            error_msg = f"NCCL recv failed: {type(e).__name__}: {str(e)}"
+            return {"error": error_msg, "bytes": 0, "blocks": 0}
+
+    def p2p_coordinated_transfer_kv(self, src_worker_ref: Any, src_rank: int, src_blocks: List[int],
+                                    dst_blocks: List[int], timeout: float = 10.0) -> Dict[str, Any]:
+        """Called on the destination: triggers the source's send, receives and scatters.
+        ``src_worker_ref`` is the source ``KVWorker`` (the reference passes a Ray actor
+        handle and calls ``.p2p_send_kv.remote``)."""
+        if not self.nccl_pg_initialized:
+            raise RuntimeError("Destination worker: Global NCCL not initialized")
+        if len(src_blocks) != len(dst_blocks):
+            raise ValueError(f"Block count mismatch: src={len(src_blocks)}, dst={len(dst_blocks)}")
+        if len(src_blocks) == 0:
+            return {"bytes": 0, "blocks": 0, "error": "No blocks to transfer"}
+        if src_rank < 0 or src_rank >= self.link.world_size:
+            raise ValueError(f"Invalid src_rank: {src_rank} (world_size={self.link.world_size})")
+        start_time = time.time()
+        try:
+            send_result = src_worker_ref.p2p_send_kv(self.global_rank, src_blocks)
+            if "error" in send_result:
+                return {"error": f"Send error: {send_result['error']}", "bytes": 0, "blocks": 0,
+                        "elapsed": time.time() - start_time}
+            res = self._recv_layers(src_rank, dst_blocks, deadline=(start_time, timeout))
+            if isinstance(res, int):
+                return {"error": f"Transfer timeout after {timeout}s at layer {res}/{len(self.kv_cache)}",
+                        "bytes": 0, "blocks": 0, "elapsed": time.time() - start_time}
+            torch.cuda.synchronize(self.device)
+            elapsed = time.time() - start_time
+            total_bytes = res["bytes"]
+            if send_result["bytes"] != total_bytes:
+                print(f"[KVWorker] Warning: Transfer size mismatch: expected {total_bytes}, got {send_result['bytes']}")
+            return {"bytes": total_bytes, "blocks": len(dst_blocks), "elapsed": elapsed,
+                    "method": "coordinated_single_call"}
+        except Exception as e:
+            elapsed = time.time() - start_time
+            error_msg = f"NCCL coordinated transfer failed after {elapsed:.2f}s: {type(e).__name__}: {str(e)}"
+            return {"error": error_msg, "bytes": 0, "blocks": 0, "elapsed": elapsed}
+
+    def p2p_pull_kv(self, src_rank: int, src_blocks: List[int], dst_blocks: List[int]) -> Dict[str, Any]:
+        """Receiver-initiated transfer: send the request (block ids, tag 999), let the
+        source serve it, receive layer messages tagged by layer index."""
+        if not self.nccl_pg_initialized:
+            raise RuntimeError("Global NCCL not initialized")
+        request_tensor = torch.full((1024,), -1, dtype=torch.long)
+        if len(src_blocks) > 1024:
+            raise ValueError("at most 1024 blocks per pull request")
+        request_tensor[:len(src_blocks)] = torch.as_tensor(list(src_blocks), dtype=torch.long)
+        self.link.send(request_tensor.to(self.device), src=self.global_rank, dst=src_rank, tag=999)
+        server = self.peers.get(src_rank)
+        if server is not None:  # the reference's source actor runs p2p_serve_kv concurrently
+            server.p2p_serve_kv(self.global_rank)
+        res = self._recv_layers(src_rank, dst_blocks, tagged=True)
+        torch.cuda.synchronize(self.device)
+        return {"bytes": res["bytes"], "blocks": len(dst_blocks)}
+
+    def p2p_serve_kv(self, requester_rank: int) -> Dict[str, Any]:
+        """Serve a pull request: a fixed 1024-slot int64 request padded with -1
+        (worker.py:920-925). The ids stay on the device; only their count is read back."""
+        if not self.nccl_pg_initialized:
+            raise RuntimeError("Global NCCL not initialized")
+        request_tensor = self.link.recv(src=requester_rank, dst=self.global_rank, tag=999)
+        block_idx = request_tensor[request_tensor >= 0]
+        n = int(block_idx.numel())
+        packed = kv_ops.kv_pack(self.pool, block_idx)
+        total_bytes = 0
+        for layer_idx in range(self.pool.num_layers):
+            layer_data = packed[layer_idx]
+            self.link.send(layer_data, src=self.global_rank, dst=requester_rank, tag=layer_idx)
+            total_bytes += layer_data.numel() * layer_data.element_size()
+        torch.cuda.synchronize(self.device)
+        return {"bytes": total_bytes, "blocks": n}
+
+    def collective_transfer_kv(self, group_name: str, root: int, block_indices: List[int],
+                               tensor_shape: Sequence[int], dtype: str, mode: str) -> Dict[str, Any]:
+        """Flat-buffer form (worker.py:939-1005): the sender packs and publishes one flat
+        tensor; the receiver takes it, views it as ``tensor_shape`` and scatters it."""
+        normalized_dtype = dtype.replace("torch.", "").lower()
+        if normalized_dtype not in _DTYPES:
+            raise ValueError(f"[KVWorker] Unsupported dtype for collective transfer: {dtype}")
+        torch_dtype = _DTYPES[normalized_dtype]
+        tensor_shape = tuple(int(dim) for dim in tensor_shape)
+        if self.link is None:
+            raise RuntimeError("no link attached")
+        tag = hash(group_name) & 0x7FFFFFFF
+        if mode == "send":
+            kv_tensor = self.extract_kv_blocks(block_indices).contiguous()
+            flat_tensor = kv_tensor.view(-1).to(dtype=torch_dtype)
+            for dst in range(self.link.world_size):
+                if dst != root:
+                    self.link.send(flat_tensor, src=root, dst=dst, tag=tag)
+            bytes_transferred = flat_tensor.numel() * flat_tensor.element_size()
+        elif mode == "recv":
+            numel = math.prod(tensor_shape)
+            flat_tensor = self.link.recv(src=root, dst=self.global_rank, tag=tag)
+            if flat_tensor.numel() != numel or flat_tensor.dtype != torch_dtype:
+                raise RuntimeError("broadcast payload does not match tensor_shape / dtype")
+            kv_tensor = flat_tensor.view(tensor_shape)
+            self.write_kv_blocks(block_indices, kv_tensor)
+            bytes_transferred = flat_tensor.numel() * flat_tensor.element_size()
+        else:
+            raise ValueError(f"[KVWorker] Unknown collective transfer mode: {mode}")
+        torch.cuda.synchronize(self.device)
+        return {"bytes": bytes_transferred, "mode": mode}
+
+    # ----- vision embeddings (worker.py:1007-1036, worker_steps.py:252-267) --
+    def extract_vision_blocks(self, request_id: str) -> torch.Tensor:
+        if self.ve_cache is None:
+            raise RuntimeError("Vision embedding cache not initialized")
+        if request_id not in self.ve_cache:
+            raise KeyError(f"Request {request_id} not found in vision cache")
+        return self.ve_cache[request_id]
+
+    def write_vision_blocks(self, request_id: str, ve_data: torch.Tensor) -> None:
+        if self.ve_cache is None:
+            raise RuntimeError("Vision embedding cache not initialized")
+        self.ve_cache[request_id] = ve_data
+
+    def gather_vision_embeddings(self, request_ids: Sequence[str]) -> Optional[torch.Tensor]:
+        """The prefill input built at worker_steps.py:252-267: embeddings of the batch's
+        requests that are cached, concatenated on dim 0 (a single tensor passes through)."""
+        if self.ve_cache is None:
+            return None
+        vision_embeds = [self.ve_cache[r] for r in request_ids if r in self.ve_cache]
+        if not vision_embeds:
+            return None
+        if len(vision_embeds) == 1:
+            return vision_embeds[0]
+        return kv_ops.concat_rows(vision_embeds)

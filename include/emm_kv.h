@@ -1,0 +1,220 @@
+/*
+ * emm_kv.h — C ABI of libemm_kv.so: the KV-cache data-movement path of ElasticMM
+ * (pack / unpack / reshape_and_cache / copy_blocks / vision-row concat) as
+ * hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions (all entry points):
+ *   - returns 0 on success, a negative EMM_E* code on failure; the text of the
+ *     last failure on the calling thread is available from emm_last_error();
+ *   - every launch is asynchronous on `stream` (a hipStream_t passed as void*;
+ *     NULL = the null stream). The library never synchronises;
+ *   - the library takes no ownership: every device pointer must stay alive
+ *     until the stream has run past the call;
+ *   - `layer_ptrs` is a HOST array of `num_layers` DEVICE base pointers, one
+ *     per layer tensor of the block pool (the reference pool is a Python list
+ *     of separately allocated per-layer tensors, elasticmm/engine/v0/worker.py:388-394;
+ *     a monolithic [L,2,NB,...] pool, elasticmm/engine/v0/nccl_transfer.py:215,
+ *     is passed as base + l*layer_stride). The table is copied into the kernel
+ *     argument block at launch, so the host array may be freed on return and
+ *     nothing is allocated on the device. num_layers <= EMM_MAX_LAYERS per
+ *     call (split larger models over several calls);
+ *   - a layer tensor is [num_kv, num_blocks, chunk] contiguous, where
+ *     chunk = block_size * num_kv_heads * head_dim elements is the contiguous
+ *     unit of one block (layout [2, num_blocks, block_size, num_heads, head_size],
+ *     elasticmm/engine/v0/worker.py:594);
+ *   - block indices, slot mappings and block mappings are int64 DEVICE arrays.
+ *     A negative block index marks padding and is skipped (the reference's
+ *     fixed-size request convention, elasticmm/engine/v0/worker.py:924-925); an
+ *     index >= num_blocks is never dereferenced (skipped), the Python layer
+ *     raises IndexError for it before launch when indices arrive as a list;
+ *   - no allocation, no global mutable state; re-entrant from any host thread.
+ */
+#ifndef EMM_KV_H
+#define EMM_KV_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EMM_KV_ABI_VERSION 1
+#define EMM_MAX_LAYERS 96   /* layer pointers carried in one kernel argument block */
+#define EMM_MAX_SEGMENTS 96  /* ragged segments carried by one emm_concat_rows launch */
+
+/* error codes */
+#define EMM_OK 0
+#define EMM_EINVAL (-1)  /* bad argument (null pointer, size, alignment, count) */
+#define EMM_ELAUNCH (-2) /* hipLaunchKernel / hipGetLastError reported an error */
+
+/* element types of the 16-bit side of the fp8 kernels */
+#define EMM_DTYPE_BF16 0
+#define EMM_DTYPE_F16 1
+
+typedef void *emm_stream_t; /* hipStream_t */
+
+/* Text of the last error raised on the calling thread ("" if none). */
+const char *emm_last_error(void);
+/* EMM_KV_ABI_VERSION the library was built with. */
+int emm_abi_version(void);
+
+/*
+ * pack — gather n scattered blocks of every layer (K and V) into one
+ * contiguous transfer buffer `packed` of layout [num_layers, num_kv, n, chunk].
+ * Replaces V0Worker.extract_kv_blocks (elasticmm/engine/v0/worker.py:578-610:
+ * per-layer `layer_kv[:, idx]` followed by torch.stack), the per-layer gather
+ * of p2p_send_kv / p2p_serve_kv (worker.py:676-682, :931-934; call with
+ * num_layers = 1 or slice `packed` per layer) and the 6-D-pool gather of
+ * V0NCCLTransferManager.transfer_kv_cache_blocks (nccl_transfer.py:241-247).
+ * With num_kv = 1 it is the vision-block gather of nccl_transfer.py:329-332.
+ */
+int emm_kv_pack(const void *const *layer_ptrs, int num_layers, int num_kv,
+                int64_t num_blocks, int64_t chunk_bytes,
+                const int64_t *block_idx, int64_t n, void *packed,
+                emm_stream_t stream);
+
+/*
+ * unpack — scatter `packed` [num_layers, num_kv, n, chunk] into the pool under
+ * block table `block_idx` (unique entries). Replaces V0Worker.write_kv_blocks
+ * (worker.py:612-633), the scatter half of p2p_recv_kv /
+ * p2p_coordinated_transfer_kv / p2p_pull_kv (worker.py:715-722, :804-820,
+ * :900-904) and the per-block loop of nccl_transfer.py:287-289 (:363-364 with
+ * num_kv = 1).
+ */
+int emm_kv_unpack(void *const *layer_ptrs, int num_layers, int num_kv,
+                  int64_t num_blocks, int64_t chunk_bytes,
+                  const int64_t *block_idx, int64_t n, const void *packed,
+                  emm_stream_t stream);
+
+/*
+ * copy_blocks — for every layer and every pair p: pool[:, dst_p] = pool[:, src_p].
+ * `block_mapping` is int64 [num_pairs, 2] row-major (src, dst), the argument
+ * shape of vLLM's copy_blocks(kv_caches, block_mapping) that the reference
+ * reaches through CacheEngine (worker.py:380); the in-reference analogue is
+ * the src->dst block lists of migrate_instance (elasticmm/engine/v0/backend.py:674-708).
+ * Destinations must be pairwise distinct and disjoint from the sources.
+ */
+int emm_copy_blocks(void *const *layer_ptrs, int num_layers, int num_kv,
+                    int64_t num_blocks, int64_t chunk_bytes,
+                    const int64_t *block_mapping, int64_t num_pairs,
+                    emm_stream_t stream);
+
+/*
+ * migrate — pack and unpack fused for two pools on one device:
+ * dst_pool[l][:, dst_idx[j]] = src_pool[l][:, src_idx[j]] without the staging
+ * buffer. Same-device form of V0KVTransferManager.transfer_kv_cache
+ * (elasticmm/engine/v0/kv_transfer.py:224-262). Both pools share num_kv and
+ * chunk_bytes; block counts may differ.
+ */
+int emm_kv_migrate(const void *const *src_layer_ptrs, int64_t src_num_blocks,
+                   void *const *dst_layer_ptrs, int64_t dst_num_blocks,
+                   int num_layers, int num_kv, int64_t chunk_bytes,
+                   const int64_t *src_idx, const int64_t *dst_idx, int64_t n,
+                   emm_stream_t stream);
+
+/*
+ * dequant-unpack — scatter an fp8-e4m3fn transfer buffer
+ * [num_layers, 2, n, chunk_elems] (bytes) into a 16-bit pool, converting
+ * out = round_to_nearest_even_16bit(float(q) * scale), scale = k_scales[l] for
+ * kv = 0 and v_scales[l] for kv = 1 (DEVICE float arrays of num_layers). NaN
+ * bytes (0x7F / 0xFF) become the canonical quiet NaN (bf16 0x7FC0, f16 0x7E00).
+ * No counterpart in the reference (its transfer rejects fp8,
+ * worker.py:956-966); defined by the fp8 KV configuration of this build.
+ */
+int emm_kv_unpack_dequant_fp8(void *const *layer_ptrs, int num_layers,
+                              int64_t num_blocks, int64_t chunk_elems,
+                              const int64_t *block_idx, int64_t n,
+                              const void *packed_fp8, const float *k_scales,
+                              const float *v_scales, int out_dtype,
+                              emm_stream_t stream);
+
+/*
+ * reshape_and_cache (flash layout) — append: for token t with
+ * s = slot_mapping[t] >= 0: key_cache[s] = key[t], value_cache[s] = value[t],
+ * rows of row_bytes = num_heads * head_size * elem_bytes; s < 0 (padding) and
+ * s >= num_slots are skipped. The cache is addressed as [num_slots, row] with
+ * num_slots = num_blocks * block_size (blocks contiguous). key/value rows are
+ * `key_stride_bytes` / `value_stride_bytes` apart. Replaces vLLM's
+ * reshape_and_cache_flash as reached from model_runner.execute_model
+ * (elasticmm/engine/v0/worker_steps.py:281, :438) on the pool bound at
+ * worker.py:408-412.
+ */
+int emm_reshape_and_cache(const void *key, const void *value, void *key_cache,
+                          void *value_cache, const int64_t *slot_mapping,
+                          int64_t num_tokens, int64_t row_bytes,
+                          int64_t key_stride_bytes, int64_t value_stride_bytes,
+                          int64_t num_slots, emm_stream_t stream);
+
+/*
+ * Same append for all layers of one step in a single launch: key_ptrs[l] /
+ * value_ptrs[l] are that layer's [num_tokens, row] inputs, the cache pointers
+ * that layer's K and V planes. HOST arrays of num_layers DEVICE pointers.
+ * All layers share slot_mapping (one table per step, worker_steps.py:219-234).
+ */
+int emm_reshape_and_cache_layers(const void *const *key_ptrs,
+                                 const void *const *value_ptrs,
+                                 void *const *key_cache_ptrs,
+                                 void *const *value_cache_ptrs, int num_layers,
+                                 const int64_t *slot_mapping,
+                                 int64_t num_tokens, int64_t row_bytes,
+                                 int64_t key_stride_bytes,
+                                 int64_t value_stride_bytes, int64_t num_slots,
+                                 emm_stream_t stream);
+
+/*
+ * fp8 append — as emm_reshape_and_cache with a 16-bit source (src_dtype) and an
+ * fp8-e4m3fn cache: q = e4m3fn_rne(float(x) / scale) with a correctly rounded
+ * fp32 division, round-to-nearest-even, ties at 464 -> 448 and at 2^-10 -> 0,
+ * |x/scale| >= 465, inf and NaN -> sign|0x7F (no saturation) — the rule of
+ * torch's .to(torch.float8_e4m3fn). k_scale / v_scale are DEVICE pointers to
+ * one float each (per-layer per-tensor scale). Strides in elements.
+ */
+int emm_reshape_and_cache_fp8(const void *key, const void *value,
+                              void *key_cache, void *value_cache,
+                              const int64_t *slot_mapping, int64_t num_tokens,
+                              int64_t row_elems, int64_t key_stride_elems,
+                              int64_t value_stride_elems, int64_t num_slots,
+                              const float *k_scale, const float *v_scale,
+                              int src_dtype, emm_stream_t stream);
+
+/* fp8 append for all layers in one launch; k_scales / v_scales are DEVICE
+ * float arrays of num_layers. */
+int emm_reshape_and_cache_fp8_layers(const void *const *key_ptrs,
+                                     const void *const *value_ptrs,
+                                     void *const *key_cache_ptrs,
+                                     void *const *value_cache_ptrs,
+                                     int num_layers,
+                                     const int64_t *slot_mapping,
+                                     int64_t num_tokens, int64_t row_elems,
+                                     int64_t key_stride_elems,
+                                     int64_t value_stride_elems,
+                                     int64_t num_slots, const float *k_scales,
+                                     const float *v_scales, int src_dtype,
+                                     emm_stream_t stream);
+
+/*
+ * concat_rows — copy n ragged segments back to back into `dst`: segment i is
+ * nbytes[i] bytes at srcs[i]. HOST arrays (n <= EMM_MAX_SEGMENTS per call;
+ * `dst_offset_bytes` lets the caller continue a longer list). Replaces
+ * torch.cat(vision_embeds, dim=0) of elasticmm/engine/v0/worker_steps.py:264-267
+ * on the tensors held by V0Worker.ve_cache (worker.py:1007-1036).
+ */
+int emm_concat_rows(const void *const *srcs, const int64_t *nbytes, int n,
+                    void *dst, int64_t dst_offset_bytes, emm_stream_t stream);
+
+/*
+ * Plain device-to-device copy with the same tile engine as pack/unpack: the
+ * yardstick the block-move kernels are compared with (no indirection).
+ */
+int emm_stream_copy(const void *src, void *dst, int64_t nbytes,
+                    emm_stream_t stream);
+
+/* Tuning hook: 0 = library default; otherwise selects a launch variant of the
+ * block-move kernels (see emm_kv.hip). Process-wide, not thread-safe; meant
+ * for benchmarks. Returns the previous value. */
+int emm_set_move_variant(int variant);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EMM_KV_H */

@@ -1,0 +1,69 @@
+"""The C-ABI library loads and exports exactly what include/emm_kv.h declares (no GPU needed)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from elasticmm_amd import _lib, library_path
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "emm_kv.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(emm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    syms = declared_symbols()
+    for name in ("emm_kv_pack", "emm_kv_unpack", "emm_copy_blocks", "emm_reshape_and_cache",
+                 "emm_reshape_and_cache_fp8", "emm_kv_unpack_dequant_fp8", "emm_concat_rows", "emm_last_error"):
+        assert name in syms
+
+
+def test_library_exports_every_declared_symbol():
+    assert os.path.exists(library_path()), "libemm_kv.so has not been built"
+    lib = ctypes.CDLL(library_path())
+    for name in declared_symbols():
+        assert hasattr(lib, name), f"{name} declared in emm_kv.h but not exported"
+
+
+def test_binding_table_matches_header():
+    assert sorted(_lib.SIGNATURES) == declared_symbols()
+    text = open(HEADER).read()
+    assert int(re.search(r"#define EMM_MAX_LAYERS (\d+)", text).group(1)) == _lib.EMM_MAX_LAYERS
+    assert int(re.search(r"#define EMM_MAX_SEGMENTS (\d+)", text).group(1)) == _lib.EMM_MAX_SEGMENTS
+    assert int(re.search(r"#define EMM_KV_ABI_VERSION (\d+)", text).group(1)) == _lib.EMM_KV_ABI_VERSION
+
+
+def test_load_and_argument_errors_without_gpu():
+    """Argument validation happens before any HIP call, so it can be exercised on a CPU-only host."""
+    lib = _lib.load()
+    assert lib.emm_abi_version() == _lib.EMM_KV_ABI_VERSION
+    table = _lib.ptr_table([0x1000])
+    rc = lib.emm_kv_pack(table, 200, 2, 4, 64, 0x1000, 1, 0x1000, None)
+    assert rc == -1 and b"num_layers" in lib.emm_last_error()
+    rc = lib.emm_kv_pack(table, 1, 2, 4, -64, 0x1000, 1, 0x1000, None)
+    assert rc == -1 and b"negative" in lib.emm_last_error()
+    rc = lib.emm_kv_pack(table, 1, 2, 4, 64, None, 1, 0x1000, None)
+    assert rc == -1 and b"null" in lib.emm_last_error()
+    # empty work is a no-op that never reaches the device
+    assert lib.emm_kv_pack(table, 1, 2, 4, 64, None, 0, None, None) == 0
+    assert lib.emm_concat_rows(None, None, 0, None, 0, None) == 0
+    assert lib.emm_concat_rows(None, None, 1000, None, 0, None) == -1
+    with pytest.raises(_lib.EmmError, match="emm_concat_rows"):
+        _lib.check(-1, "emm_concat_rows")
+    rc = lib.emm_reshape_and_cache(0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 4, 64, 32, 64, 16, None)
+    assert rc == -1 and b"stride" in lib.emm_last_error()
+    rc = lib.emm_kv_unpack_dequant_fp8(table, 1, 4, 24, 0x1000, 1, 0x1000, 0x1000, 0x1000, 0, None)
+    assert rc == -1 and b"multiples of 16" in lib.emm_last_error()
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "library_path", lambda: str(tmp_path / "nope.so"))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        _lib.load()

@@ -1,0 +1,593 @@
+"""GPU parity tests: the HIP path (through the C ABI) against the CPU oracle.
+
+Bit-exact everywhere (byte moves and the fp8 cast alike): pools, transfer buffers
+and caches are compared as raw bit patterns. Small and medium shapes are compared
+with the oracle in full; the BASELINE-size shapes are checked through
+size-independent properties (every moved block equals its source, everything
+else keeps its canary) evaluated on the device with torch indexing as a second,
+independent implementation.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import kv_oracle as orc  # noqa: E402  (test infrastructure)
+from elasticmm_amd import _lib, cache_ops, kv_ops, pool_transfer  # noqa: E402
+from elasticmm_amd.kv_ops import PoolView  # noqa: E402
+from elasticmm_amd.worker import KVWorker, LoopbackLink  # noqa: E402
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    _lib.load()
+    yield
+    torch.cuda.synchronize()
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+def raw(t: torch.Tensor) -> np.ndarray:
+    """Bit pattern of a tensor as a flat uint8 numpy array (host)."""
+    return t.detach().contiguous().cpu().reshape(-1).view(torch.uint8).numpy()
+
+
+def same_bits(a: torch.Tensor, b) -> bool:
+    bb = raw(b) if isinstance(b, torch.Tensor) else np.ascontiguousarray(b).reshape(-1).view(np.uint8)
+    aa = raw(a)
+    return aa.size == bb.size and bool((aa == bb).all())
+
+
+def cpu_pool(L, NB, bs, H, D, dtype, seed, scale=1.0, fill=None):
+    g = torch.Generator().manual_seed(seed)
+    out = []
+    for _ in range(L):
+        if fill is not None:
+            out.append(torch.full((2, NB, bs, H, D), fill, dtype=dtype))
+        else:
+            out.append((torch.randn((2, NB, bs, H, D), generator=g) * scale).to(dtype))
+    return out
+
+
+def to_dev(pool, monolithic=False):
+    if monolithic:
+        return list(torch.stack(pool, 0).to(DEV).unbind(0))
+    return [p.to(DEV) for p in pool]
+
+
+# ------------------------------------------------------------------ config 1
+def test_cfg1_pack_unpack_bitwise():
+    say("cfg1: L4 [2,1024,16,8,128] fp16, 32 blocks, seeds 0/1")
+    L, NB, bs, H, D = 4, 1024, 16, 8, 128
+    src_c = cpu_pool(L, NB, bs, H, D, torch.float16, 0)
+    dst_c = cpu_pool(L, NB, bs, H, D, torch.float16, 0, fill=-3.0)
+    src_idx = torch.randperm(NB, generator=torch.Generator().manual_seed(0))[:32].tolist()
+    dst_idx = torch.randperm(NB, generator=torch.Generator().manual_seed(1))[:32].tolist()
+    src_g, dst_g = to_dev(src_c), to_dev(dst_c)
+    sw, dw = KVWorker(device=DEV), KVWorker(device=DEV)
+    sw.bind_kv_cache(src_g)
+    dw.bind_kv_cache(dst_g)
+    buf = sw.extract_kv_blocks(src_idx)
+    assert buf.shape == (L, 2, 32, bs, H, D) and buf.dtype == torch.float16 and buf.is_contiguous()
+    assert buf.numel() * 2 == 8 << 20
+    want = orc.ref_extract_kv_blocks(src_c, src_idx)
+    assert same_bits(buf, want)
+    assert same_bits(buf, orc.c_kv_pack(src_c, src_idx))
+    dw.write_kv_blocks(dst_idx, buf)
+    orc.ref_write_kv_blocks(dst_c, dst_idx, want)
+    for l in range(L):
+        assert same_bits(dst_g[l], dst_c[l]), f"layer {l}"
+        assert same_bits(src_g[l], src_c[l])
+    assert sw.get_kv_cache_layout() == {"num_layers": 4, "block_size": 16, "num_heads": 8, "head_size": 128,
+                                        "dtype": "float16"}
+
+
+def test_golden_fixture_through_the_gpu(golden_dir):
+    z = np.load(os.path.join(golden_dir, "kv_small.npz"))
+
+    def t16(a, dt=torch.float16):
+        return torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).view(dt).to(DEV)
+
+    src = [t16(a) for a in z["src"]]
+    pool = PoolView(src)
+    packed = kv_ops.kv_pack(pool, z["src_idx"].tolist())
+    assert same_bits(packed, z["packed"])
+    dst = [torch.full_like(p, -7.0) for p in src]
+    kv_ops.kv_unpack(PoolView(dst), z["dst_idx"].tolist(), packed)
+    assert same_bits(torch.stack(dst), z["dst_after"])
+    NB, bs, H, D = z["key_cache_after"].shape
+    kc = torch.full((NB, bs, H, D), 3.0, dtype=torch.float16, device=DEV)
+    vc = torch.full((NB, bs, H, D), 5.0, dtype=torch.float16, device=DEV)
+    cache_ops.reshape_and_cache_flash(t16(z["key"]), t16(z["value"]), kc, vc, torch.from_numpy(z["slots"]).to(DEV))
+    assert same_bits(kc, z["key_cache_after"]) and same_bits(vc, z["value_cache_after"])
+    cb = [p.clone() for p in src]
+    cache_ops.copy_blocks(cb, torch.from_numpy(z["mapping"]).to(DEV))
+    assert same_bits(torch.stack(cb), z["copy_after"])
+    segs = [t16(z[f"seg{i}"], torch.bfloat16) for i in range(3)]
+    assert same_bits(kv_ops.concat_rows(segs), z["cat"])
+
+
+# ------------------------------------------------------------------ shapes / edge cases
+@pytest.mark.parametrize("dtype,bs,H,D,desc", [
+    (torch.bfloat16, 16, 4, 128, "16 KiB chunk, one full tile"),
+    (torch.float16, 16, 8, 128, "32 KiB chunk, two tiles"),
+    (torch.bfloat16, 16, 5, 128, "20 KiB chunk, tail tile"),
+    (torch.bfloat16, 2, 1, 64, "256 B chunk, smaller than a tile"),
+    (torch.float16, 1, 1, 3, "6 B chunk, 2-byte lanes"),
+    (torch.float32, 1, 1, 5, "20 B chunk, 4-byte lanes"),
+    (torch.uint8, 1, 1, 7, "7 B chunk, byte lanes"),
+    (torch.float32, 16, 2, 64, "fp32 pool"),
+])
+@pytest.mark.parametrize("monolithic", [False, True])
+def test_pack_unpack_shapes(dtype, bs, H, D, desc, monolithic):
+    say(f"shape case: {desc} monolithic={monolithic}")
+    L, NB, n = 3, 37, 9
+    g = torch.Generator().manual_seed(21)
+    if dtype == torch.uint8:
+        src_c = [torch.randint(0, 255, (2, NB, bs, H, D), generator=g, dtype=torch.uint8) for _ in range(L)]
+        dst_c = [torch.full((2, NB, bs, H, D), 0xAB, dtype=torch.uint8) for _ in range(L)]
+    else:
+        src_c = cpu_pool(L, NB, bs, H, D, dtype, 21)
+        dst_c = cpu_pool(L, NB, bs, H, D, dtype, 0, fill=-5.0)
+    si = torch.randperm(NB, generator=g)[:n].tolist()
+    di = torch.randperm(NB, generator=g)[:n].tolist()
+    src_g, dst_g = to_dev(src_c, monolithic), to_dev(dst_c, monolithic)
+    buf = kv_ops.kv_pack(PoolView(src_g), si)
+    assert same_bits(buf, orc.c_kv_pack(src_c, si))
+    kv_ops.kv_unpack(PoolView(dst_g), di, buf)
+    orc.c_kv_unpack(dst_c, di, raw(buf))
+    for l in range(L):
+        assert same_bits(dst_g[l], dst_c[l])
+
+
+def test_empty_and_single_block():
+    src_c = cpu_pool(2, 8, 4, 2, 16, torch.bfloat16, 5)
+    src_g = to_dev(src_c)
+    pool = PoolView(src_g)
+    e = kv_ops.kv_pack(pool, [])
+    assert e.shape == (2, 2, 0, 4, 2, 16)
+    kv_ops.kv_unpack(pool, [], e)
+    kv_ops.copy_blocks(pool, torch.zeros((0, 2), dtype=torch.long, device=DEV))
+    one = kv_ops.kv_pack(pool, [7])
+    assert same_bits(one, orc.ref_extract_kv_blocks(src_c, [7]))
+    k = torch.zeros((0, 2, 16), dtype=torch.bfloat16, device=DEV)
+    kv_ops.reshape_and_cache(k, k, src_g[0][0], src_g[0][1], torch.zeros((0,), dtype=torch.long, device=DEV))
+    for l in range(2):
+        assert same_bits(src_g[l], src_c[l])
+
+
+def test_list_indices_follow_torch_rules_on_gpu():
+    src_c = cpu_pool(1, 6, 2, 1, 8, torch.float16, 6)
+    pool = PoolView(to_dev(src_c))
+    got = kv_ops.kv_pack(pool, [-1, 0, -6])
+    assert same_bits(got, orc.ref_extract_kv_blocks(src_c, [-1, 0, -6]))
+    with pytest.raises(IndexError):
+        kv_ops.kv_pack(pool, [6])
+
+
+def test_device_indices_padding_and_out_of_range_are_skipped():
+    src_c = cpu_pool(2, 6, 2, 1, 8, torch.float16, 7)
+    pool = PoolView(to_dev(src_c))
+    idx = torch.tensor([4, -1, 99, 0], dtype=torch.long, device=DEV)
+    out = torch.full((2, 2, 4, 2, 1, 8), 1.25, dtype=torch.float16, device=DEV)
+    kv_ops.kv_pack(pool, idx, out=out)
+    want = torch.full((2, 2, 4, 2, 1, 8), 1.25, dtype=torch.float16)
+    ref = orc.ref_extract_kv_blocks(src_c, [4, 0])
+    want[:, :, 0] = ref[:, :, 0]
+    want[:, :, 3] = ref[:, :, 1]
+    assert same_bits(out, want)
+    dst_c = cpu_pool(2, 6, 2, 1, 8, torch.float16, 0, fill=2.0)
+    dst_g = to_dev(dst_c)
+    kv_ops.kv_unpack(PoolView(dst_g), idx, out)
+    orc.c_kv_unpack(dst_c, [4, -1, 99, 0], raw(out))
+    for l in range(2):
+        assert same_bits(dst_g[l], dst_c[l])
+
+
+def test_more_layers_than_one_argument_block():
+    L = _lib.EMM_MAX_LAYERS + 5
+    src_c = cpu_pool(L, 5, 1, 1, 8, torch.float16, 8)
+    src_g = to_dev(src_c)
+    buf = kv_ops.kv_pack(PoolView(src_g), [3, 1])
+    assert same_bits(buf, orc.ref_extract_kv_blocks(src_c, [3, 1]))
+    dst_g = [torch.zeros_like(p) for p in src_g]
+    kv_ops.kv_unpack(PoolView(dst_g), [0, 4], buf)
+    dst_c = [torch.zeros_like(p) for p in src_c]
+    orc.ref_write_kv_blocks(dst_c, [0, 4], orc.ref_extract_kv_blocks(src_c, [3, 1]))
+    assert same_bits(torch.stack(dst_g), torch.stack(dst_c))
+    kv_ops.kv_migrate(PoolView(src_g), [2], PoolView(dst_g), [1])
+    assert same_bits(torch.stack(dst_g)[:, :, 1], torch.stack(src_c)[:, :, 2])
+
+
+# ------------------------------------------------------------------ copy_blocks / migrate
+def test_copy_blocks_against_oracle():
+    L, NB = 5, 64
+    base = cpu_pool(L, NB, 16, 4, 128, torch.bfloat16, 9, scale=0.5)
+    g = torch.Generator().manual_seed(9)
+    perm = torch.randperm(NB, generator=g)
+    mapping = torch.stack([perm[:20], perm[20:40]], 1).contiguous()
+    dev = to_dev(base)
+    cache_ops.copy_blocks(dev, mapping.to(DEV))
+    want = [p.clone() for p in base]
+    orc.c_copy_blocks(want, mapping.numpy())
+    ref = [p.clone() for p in base]
+    orc.ref_copy_blocks(ref, mapping)
+    for l in range(L):
+        assert same_bits(dev[l], want[l]) and same_bits(dev[l], ref[l])
+        assert same_bits(dev[l][:, perm[:20].to(DEV)], base[l][:, perm[:20]])  # sources unchanged
+    # list-of-pairs form goes through the same path
+    dev2 = to_dev(base)
+    kv_ops.copy_blocks(PoolView(dev2), mapping.tolist())
+    assert same_bits(torch.stack(dev2), torch.stack(want))
+
+
+def test_migrate_equals_pack_then_unpack():
+    L, NBs, NBd = 4, 40, 24
+    src_c = cpu_pool(L, NBs, 16, 4, 128, torch.bfloat16, 10)
+    g = torch.Generator().manual_seed(10)
+    si = torch.randperm(NBs, generator=g)[:12].tolist()
+    di = torch.randperm(NBd, generator=g)[:12].tolist()
+    src_g = to_dev(src_c)
+    a = [torch.full((2, NBd, 16, 4, 128), 1.0, dtype=torch.bfloat16, device=DEV) for _ in range(L)]
+    b = [t.clone() for t in a]
+    kv_ops.kv_migrate(PoolView(src_g), si, PoolView(a), di)
+    kv_ops.kv_unpack(PoolView(b), di, kv_ops.kv_pack(PoolView(src_g), si))
+    assert same_bits(torch.stack(a), torch.stack(b))
+    with pytest.raises(ValueError, match="Block count mismatch"):
+        kv_ops.kv_migrate(PoolView(src_g), si, PoolView(a), di[:-1])
+
+
+# ------------------------------------------------------------------ legacy pools
+def test_monolithic_6d_pool_and_vision_pool():
+    L, NB, bs, H, D = 3, 20, 16, 2, 64
+    g = torch.Generator().manual_seed(11)
+    pool6 = torch.randn((L, 2, NB, bs, H, D), generator=g).to(torch.float16)
+    si, di = [7, 0, 19, 3], [1, 2, 18, 5]
+    flat = pool_transfer.gather_kv_blocks(pool6.to(DEV), si)
+    assert flat.dim() == 1 and same_bits(flat, orc.ref_pool6d_gather(pool6, si))
+    dst_c = torch.zeros_like(pool6)
+    dst_g = dst_c.to(DEV)
+    kv_data = pool_transfer.scatter_kv_blocks(dst_g, di, flat)
+    assert kv_data.shape == (L, 2, 4, bs, H, D)
+    orc.ref_pool6d_scatter(dst_c, di, orc.ref_pool6d_gather(pool6, si))
+    assert same_bits(dst_g, dst_c)
+    ve = torch.randn((12, 9, 48), generator=g).to(torch.bfloat16)
+    vf = pool_transfer.gather_vision_blocks(ve.to(DEV), [5, 11, 0])
+    assert same_bits(vf, orc.ref_vision_gather(ve, [5, 11, 0]))
+    ve_dst_c = torch.zeros_like(ve)
+    ve_dst_g = ve_dst_c.to(DEV)
+    pool_transfer.scatter_vision_blocks(ve_dst_g, [2, 3, 4], vf)
+    orc.ref_vision_scatter(ve_dst_c, [2, 3, 4], orc.ref_vision_gather(ve, [5, 11, 0]))
+    assert same_bits(ve_dst_g, ve_dst_c)
+
+
+# ------------------------------------------------------------------ append
+def make_slots(num_slots, T, seed, pad_frac=0.05):
+    g = torch.Generator().manual_seed(seed)
+    slots = torch.randperm(num_slots, generator=g)[:T].clone()
+    pad = torch.rand(T, generator=g) < pad_frac
+    slots[pad] = -1
+    return slots
+
+
+def test_cfg3_append_reduced_pool():
+    say("cfg3 shape: T=8448 [T,4,128] bf16, 5% padded slots; pool reduced to 2048 blocks, 2 layers")
+    NB, bs, H, D, T, L = 2048, 16, 4, 128, 8448, 2
+    slots = make_slots(NB * bs, T, 3)
+    assert (slots < 0).sum() > 300
+    g = torch.Generator().manual_seed(3)
+    pool_c = cpu_pool(L, NB, bs, H, D, torch.bfloat16, 0, fill=7.0)
+    pool_g = to_dev(pool_c)
+    slots_g = slots.to(DEV)
+    for l in range(L):
+        key = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+        value = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+        cache_ops.reshape_and_cache_flash(key.to(DEV), value.to(DEV), pool_g[l][0], pool_g[l][1], slots_g, "auto")
+        orc.c_reshape_and_cache(key, value, pool_c[l][0], pool_c[l][1], slots)
+        assert same_bits(pool_g[l], pool_c[l]), f"layer {l}"
+    ref = cpu_pool(1, NB, bs, H, D, torch.bfloat16, 0, fill=7.0)[0]
+    orc.ref_reshape_and_cache_flash(key, value, ref[0], ref[1], slots)
+    assert same_bits(pool_g[L - 1], ref)
+
+
+def test_append_strided_tokens_odd_rows_and_layers_variant():
+    NB, bs, H, D, T, L = 16, 4, 3, 40, 37, 3  # 240-byte rows (16-B lanes), T not a multiple of 16
+    g = torch.Generator().manual_seed(13)
+    qkv = torch.randn((L, T, 3 * H * D), generator=g).to(torch.float16)
+    slots = make_slots(NB * bs, T, 13, pad_frac=0.2)
+    pool_c = cpu_pool(L, NB, bs, H, D, torch.float16, 0, fill=1.0)
+    pool_g = to_dev(pool_c)
+    qkv_g = qkv.to(DEV)
+    keys = [qkv_g[l, :, H * D:2 * H * D].view(T, H, D) for l in range(L)]       # strided views
+    values = [qkv_g[l, :, 2 * H * D:].view(T, H, D) for l in range(L)]
+    assert not keys[0].is_contiguous()
+    cache_ops.reshape_and_cache_flash_layers(keys, values, pool_g, slots.to(DEV))
+    for l in range(L):
+        k = qkv[l, :, H * D:2 * H * D].reshape(T, H, D).contiguous()
+        v = qkv[l, :, 2 * H * D:].reshape(T, H, D).contiguous()
+        orc.c_reshape_and_cache(k, v, pool_c[l][0], pool_c[l][1], slots)
+        assert same_bits(pool_g[l], pool_c[l])
+    # per-layer call on a strided view, narrow rows (6 bytes -> 2-byte lanes)
+    kc = torch.zeros((4, 2, 1, 3), dtype=torch.float16, device=DEV)
+    vc = torch.zeros_like(kc)
+    x = torch.randn((5, 2, 3), generator=g).to(torch.float16)
+    xs = x.to(DEV)[:, 1:2, :]
+    sl = torch.tensor([7, -1, 0, 3, 5])
+    cache_ops.reshape_and_cache_flash(xs, xs, kc, vc, sl.to(DEV))
+    kcc = torch.zeros((4, 2, 1, 3), dtype=torch.float16)
+    vcc = torch.zeros_like(kcc)
+    orc.c_reshape_and_cache(x[:, 1:2, :].contiguous(), x[:, 1:2, :].contiguous(), kcc, vcc, sl)
+    assert same_bits(kc, kcc) and same_bits(vc, vcc)
+
+
+def test_append_out_of_range_slot_is_skipped():
+    kc = torch.full((2, 2, 1, 8), 4.0, dtype=torch.bfloat16, device=DEV)
+    vc = kc.clone()
+    x = torch.ones((3, 1, 8), dtype=torch.bfloat16, device=DEV)
+    cache_ops.reshape_and_cache_flash(x, x, kc, vc, torch.tensor([1, 4, -1], device=DEV))
+    want = torch.full((4, 8), 4.0)
+    want[1] = 1.0
+    assert torch.equal(kc.float().cpu().view(4, 8), want)
+
+
+# ------------------------------------------------------------------ fp8
+def test_fp8_append_exhaustive_bf16_and_f16(golden_dir):
+    """Every 16-bit input x several scales through the append kernel: 64 tokens x 1024
+    elements is exactly the 65 536 bit patterns."""
+    kat = json.load(open(os.path.join(golden_dir, "fp8_kat.json")))
+    import hashlib
+    for dtype, name in ((torch.bfloat16, "bf16"), (torch.float16, "f16")):
+        allx = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype)
+        key = allx.view(64, 8, 128)
+        value = allx.flip(0).contiguous().view(64, 8, 128)
+        slots = torch.arange(64)
+        for s in kat["scales"]:
+            say(f"fp8 exhaustive {name} scale {s}")
+            kc = torch.zeros((4, 16, 8, 128), dtype=torch.uint8, device=DEV)
+            vc = torch.zeros_like(kc)
+            sc = torch.tensor([s], dtype=torch.float32, device=DEV)
+            cache_ops.reshape_and_cache_flash(key.to(DEV), value.to(DEV), kc.view(torch.float8_e4m3fn),
+                                              vc.view(torch.float8_e4m3fn), slots.to(DEV), "fp8", sc, sc)
+            got = raw(kc)
+            want = orc.c_quant_fp8(allx, s).reshape(-1)
+            bad = np.nonzero(got != want)[0]
+            assert bad.size == 0, f"{name} scale {s}: {bad.size} mismatches, first bits {bad[:8]} got {got[bad[:8]]} want {want[bad[:8]]}"
+            assert hashlib.sha256(got.tobytes()).hexdigest() == kat["sweep_sha256"][f"{name}@{s}"]
+            assert (raw(vc) == orc.c_quant_fp8(allx.flip(0).contiguous(), s).reshape(-1)).all()
+
+
+def test_fp8_known_answers_on_gpu():
+    xs = [448, 464, 465, 480, -1000, 2 ** -9, 2 ** -10, 2 ** -10 * 1.0001, 17, 18, 19, float("inf")]
+    want = [126, 126, 127, 127, 255, 1, 0, 1, 88, 89, 90, 127]
+    x = torch.zeros((1, 1, 16), dtype=torch.bfloat16)
+    x[0, 0, :12] = torch.tensor(xs, dtype=torch.float32).to(torch.bfloat16)
+    # 465 and 2^-10*1.0001 are not bf16 values: use f32-exact neighbours that are
+    x[0, 0, 2] = 466.0
+    x[0, 0, 7] = 2 ** -10 * 1.0078125
+    kc = torch.zeros((1, 1, 1, 16), dtype=torch.uint8, device=DEV)
+    vc = torch.zeros_like(kc)
+    one = torch.ones(1, device=DEV)
+    cache_ops.reshape_and_cache_flash(x.to(DEV), x.to(DEV), kc, vc, torch.zeros(1, dtype=torch.long, device=DEV),
+                                      "fp8", one, one)
+    assert raw(kc)[:12].tolist() == want
+
+
+def test_cfg4_fp8_append_pack_dequant_reduced():
+    say("cfg4 shape reduced: 6 layers [2,256,16,8,128] fp8, scales U[0.01,0.1], T=1500")
+    L, NB, bs, H, D, T = 6, 256, 16, 8, 128, 1500
+    g = torch.Generator().manual_seed(4)
+    ks = (torch.rand(L, generator=g) * 0.09 + 0.01).float()
+    vs = (torch.rand(L, generator=g) * 0.09 + 0.01).float()
+    slots = make_slots(NB * bs, T, 4)
+    pool_c = [torch.full((2, NB, bs, H, D), 0x5A, dtype=torch.uint8) for _ in range(L)]
+    pool_g = to_dev(pool_c)
+    keys, values = [], []
+    for l in range(L):
+        k = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+        v = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+        keys.append(k.to(DEV))
+        values.append(v.to(DEV))
+        orc.c_reshape_and_cache_fp8(k, v, pool_c[l][0], pool_c[l][1], slots, float(ks[l]), float(vs[l]))
+    # layer 0 through the per-layer entry point, all through the fused one on a second pool
+    pool_g2 = [p.clone() for p in pool_g]
+    for l in range(L):
+        cache_ops.reshape_and_cache_flash(keys[l], values[l], pool_g[l][0], pool_g[l][1], slots.to(DEV), "fp8",
+                                          ks[l:l + 1].to(DEV), vs[l:l + 1].to(DEV))
+    cache_ops.reshape_and_cache_flash_layers(keys, values, pool_g2, slots.to(DEV), "fp8", ks, vs)
+    for l in range(L):
+        assert same_bits(pool_g[l], pool_c[l]), f"layer {l}"
+        assert same_bits(pool_g2[l], pool_c[l]), f"fused layer {l}"
+    # pack / unpack move fp8 bytes
+    si = torch.randperm(NB, generator=g)[:40].tolist()
+    di = torch.randperm(NB, generator=g)[:40].tolist()
+    packed = kv_ops.kv_pack(PoolView(pool_g), si)
+    assert packed.dtype == torch.uint8 and same_bits(packed, orc.c_kv_pack(pool_c, si))
+    dst8 = [torch.zeros_like(p) for p in pool_g]
+    kv_ops.kv_unpack(PoolView(dst8), di, packed)
+    dst8_c = [torch.zeros_like(p) for p in pool_c]
+    orc.c_kv_unpack(dst8_c, di, raw(packed))
+    assert same_bits(torch.stack(dst8), torch.stack(dst8_c))
+    # dequantising unpack into bf16 and f16 pools
+    for dt in (torch.bfloat16, torch.float16):
+        dq_g = [torch.full((2, NB, bs, H, D), 9.0, dtype=dt, device=DEV) for _ in range(L)]
+        dq_c = [torch.full((2, NB, bs, H, D), 9.0, dtype=dt) for _ in range(L)]
+        kv_ops.kv_unpack_dequant_fp8(PoolView(dq_g), di, packed, ks, vs)
+        orc.c_unpack_dequant_fp8(dq_c, di, raw(packed), ks.numpy(), vs.numpy())
+        assert same_bits(torch.stack(dq_g), torch.stack(dq_c)), str(dt)
+
+
+def test_fp8_dequant_all_bytes_all_scales(golden_dir):
+    kat = json.load(open(os.path.join(golden_dir, "fp8_kat.json")))
+    scales = kat["scales"]
+    L = len(scales)
+    # one block of 256 bytes per layer holding every byte value; K uses scale s, V uses s/3
+    allq = torch.arange(256, dtype=torch.int32).to(torch.uint8)
+    packed = allq.view(1, 1, 1, 256).expand(L, 2, 1, 256).contiguous().to(DEV)
+    ks = torch.tensor(scales, dtype=torch.float32)
+    vs = ks / 3
+    for dt in (torch.bfloat16, torch.float16):
+        pool = [torch.zeros((2, 2, 1, 2, 128), dtype=dt, device=DEV) for _ in range(L)]
+        kv_ops.kv_unpack_dequant_fp8(PoolView(pool), [1], packed, ks, vs)
+        for l, s in enumerate(scales):
+            got = pool[l].cpu().view(torch.int16).numpy().view(np.uint16)
+            assert (got[0, 1].reshape(-1) == orc.c_dequant_fp8(allq.numpy(), float(ks[l]), dt)).all()
+            assert (got[1, 1].reshape(-1) == orc.c_dequant_fp8(allq.numpy(), float(vs[l]), dt)).all()
+            assert not got[:, 0].any()
+            if dt == torch.bfloat16 and f"bf16@{s}" in kat["dequant"]:
+                assert got[0, 1].reshape(-1).tolist() == kat["dequant"][f"bf16@{s}"]
+
+
+# ------------------------------------------------------------------ vision concat
+def test_concat_rows_ragged():
+    say("vision concat: 20 tensors [U{64..2304}, 3584] bf16 + edge cases")
+    g = torch.Generator().manual_seed(5)
+    rows = torch.randint(64, 2305, (20,), generator=g).tolist()
+    segs = [torch.randn((r, 3584), generator=g).to(torch.bfloat16) for r in rows]
+    got = kv_ops.concat_rows([s.to(DEV) for s in segs])
+    assert got.shape == (sum(rows), 3584)
+    assert same_bits(got, orc.ref_concat_rows(segs))
+    # more segments than one launch carries, with empty and odd-sized ones
+    many = [torch.randn((int(r), 3), generator=g).to(torch.float16) for r in torch.randint(0, 9, (230,), generator=g)]
+    got = kv_ops.concat_rows([s.to(DEV) for s in many])
+    assert same_bits(got, torch.cat(many, 0))
+    assert same_bits(got, orc.c_concat_rows(many))
+    w = KVWorker(device=DEV)
+    w.init_vecache()
+    for i, s in enumerate(segs[:3]):
+        w.write_vision_blocks(f"r{i}", s.to(DEV))
+    assert same_bits(w.gather_vision_embeddings(["r0", "zz", "r2"]), torch.cat([segs[0], segs[2]], 0))
+    assert w.gather_vision_embeddings(["r1"]) is w.extract_vision_blocks("r1")
+
+
+# ------------------------------------------------------------------ worker protocol
+def make_pair(L=3, NB=32, bs=16, H=2, D=64, dtype=torch.bfloat16):
+    link = LoopbackLink(world_size=2)
+    src = KVWorker(0, DEV, bs, link, 0)
+    dst = KVWorker(1, DEV, bs, link, 1)
+    src.init_kvcache(NB, num_layers=L, num_kv_heads=H, head_size=D, dtype=dtype, monolithic=False)
+    dst.init_kvcache(NB, num_layers=L, num_kv_heads=H, head_size=D, dtype=dtype, monolithic=True)
+    g = torch.Generator().manual_seed(14)
+    for t in src.kv_cache:
+        t.copy_(torch.randn(t.shape, generator=g).to(dtype))
+    for t in dst.kv_cache:
+        t.fill_(-2.0)
+    src.peers[1] = dst
+    dst.peers[0] = src
+    return src, dst
+
+
+def check_moved(src, dst, si, di):
+    src_c = [t.cpu() for t in src.kv_cache]
+    want = [torch.full_like(t, -2.0) for t in src_c]
+    orc.ref_write_kv_blocks(want, di, orc.ref_extract_kv_blocks(src_c, si))
+    for l in range(len(want)):
+        assert same_bits(dst.kv_cache[l], want[l])
+
+
+def test_worker_p2p_send_recv():
+    src, dst = make_pair()
+    si, di = [5, 9, 0, 31], [1, 2, 3, 30]
+    s = src.p2p_send_kv(1, si)
+    per_layer = 2 * 4 * 16 * 2 * 64 * 2
+    assert s == {"bytes": 3 * per_layer, "blocks": 4}
+    r = dst.p2p_recv_kv(0, di)
+    assert r == {"bytes": 3 * per_layer, "blocks": 4}
+    check_moved(src, dst, si, di)
+    # nothing pending -> error dict, not an exception
+    r = dst.p2p_recv_kv(0, di)
+    assert r["bytes"] == 0 and r["blocks"] == 0 and r["error"].startswith("NCCL recv failed: RuntimeError")
+    bad = src.p2p_send_kv(1, [999])
+    assert bad["bytes"] == 0 and bad["error"].startswith("NCCL send failed: IndexError")
+
+
+def test_worker_coordinated_pull_and_collective():
+    src, dst = make_pair()
+    si, di = [7, 8, 30], [0, 15, 16]
+    res = dst.p2p_coordinated_transfer_kv(src, 0, si, di)
+    assert res["method"] == "coordinated_single_call" and res["blocks"] == 3 and res["bytes"] == 3 * 2 * 3 * 16 * 2 * 64 * 2
+    check_moved(src, dst, si, di)
+    res = dst.p2p_coordinated_transfer_kv(src, 0, si, di, timeout=-1.0)
+    assert res["error"].startswith("Transfer timeout after -1.0s at layer 0/3")
+
+    src, dst = make_pair()
+    res = dst.p2p_pull_kv(0, si, di)
+    assert res == {"bytes": 3 * 2 * 3 * 16 * 2 * 64 * 2, "blocks": 3}
+    check_moved(src, dst, si, di)
+
+    src, dst = make_pair()
+    shape = (3, 2, 3, 16, 2, 64)
+    a = src.collective_transfer_kv("g0", 0, si, shape, "torch.bfloat16", "send")
+    b = dst.collective_transfer_kv("g0", 0, di, shape, "bf16", "recv")
+    assert a == {"bytes": int(np.prod(shape)) * 2, "mode": "send"} and b["mode"] == "recv" and b["bytes"] == a["bytes"]
+    check_moved(src, dst, si, di)
+    with pytest.raises(ValueError, match="Unknown collective transfer mode"):
+        src.collective_transfer_kv("g0", 0, si, shape, "bf16", "both")
+    with pytest.raises(AssertionError, match="Block count mismatch"):
+        dst.write_kv_blocks([1, 2], torch.zeros(shape, dtype=torch.bfloat16, device=DEV))
+
+
+# ------------------------------------------------------------------ BASELINE-size properties
+def test_cfg2_full_size_migration_properties():
+    """Qwen2-7B KV shape at full size: 28 x [2,60000,16,4,128] bf16 twice (2 x 51.3 GiB).
+    Checked with torch's own device indexing as the second implementation."""
+    L, NB, bs, H, D = 28, 60000, 16, 4, 128
+    free, _ = torch.cuda.mem_get_info()
+    need = 2 * L * 2 * NB * bs * H * D * 2 + (12 << 30)
+    if free < need:
+        pytest.skip(f"needs {need >> 30} GiB of free HBM, have {free >> 30}")
+    say("cfg2 full size: allocating two 51.3 GiB pools")
+    src = torch.empty((L, 2, NB, bs, H, D), dtype=torch.bfloat16, device=DEV)
+    g = torch.Generator(device=DEV).manual_seed(2)
+    for l in range(L):
+        src[l].normal_(0.0, 0.5, generator=g)
+    dst = torch.empty_like(src)
+    dst.fill_(-1.0)
+    gc = torch.Generator().manual_seed(2)
+    nblk = [(int(p) + 1024 + 15) // 16 for p in torch.randint(512, 4097, (32,), generator=gc)]
+    sperm = torch.randperm(NB, generator=gc)
+    dperm = torch.randperm(NB, generator=gc)
+    sp, dp = PoolView(src), PoolView(dst)
+    off = 0
+    tables = []
+    for n in nblk:
+        si, di = sperm[off:off + n].to(DEV), dperm[off:off + n].to(DEV)
+        tables.append((si, di))
+        off += n
+        buf = kv_ops.kv_pack(sp, si)
+        kv_ops.kv_unpack(dp, di, buf)
+    torch.cuda.synchronize()
+    say(f"cfg2 full size: moved {off} blocks, checking")
+    moved = torch.zeros(NB, dtype=torch.bool, device=DEV)
+    for r, (si, di) in enumerate(tables):
+        moved[di] = True
+        for l in range(0, L, 3) if r % 4 else range(L):
+            assert torch.equal(dst[l][:, di], src[l][:, si]), f"request {r} layer {l}"
+    rest = (~moved).nonzero().squeeze(1)
+    for l in range(L):
+        assert bool((dst[l][:, rest] == -1.0).all()), f"layer {l}: an untouched block changed"
+    # batched form: one launch for all 32 requests
+    dst.fill_(-1.0)
+    all_si = torch.cat([t[0] for t in tables])
+    all_di = torch.cat([t[1] for t in tables])
+    kv_ops.kv_unpack(dp, all_di, kv_ops.kv_pack(sp, all_si))
+    for l in (0, 13, 27):
+        assert torch.equal(dst[l][:, all_di], src[l][:, all_si])
+    # copy_blocks inside the source pool: half of the used blocks to free blocks
+    P = off // 2
+    mapping = torch.stack([sperm[:P], sperm[off:off + P]], 1).to(DEV)
+    before = src[5][:, mapping[:, 0]].clone()
+    kv_ops.copy_blocks(sp, mapping)
+    for l in (0, 5, 27):
+        assert torch.equal(src[l][:, mapping[:, 1]], src[l][:, mapping[:, 0]])
+    assert torch.equal(src[5][:, mapping[:, 0]], before)
+    del src, dst
+    torch.cuda.empty_cache()
