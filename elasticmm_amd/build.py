@@ -21,6 +21,9 @@ HIPCC_FLAGS = [
     "-std=c++17",
     "-fPIC",
     "-shared",
+    # bit-exact arithmetic: no fused multiply-add / fused multiply-convert (the fp8 rule is
+    # "round the fp32 product, then round to 16 bits", two roundings)
+    "-ffp-contract=off",
     # keep the compiler from forming packed-fp32 ops out of float code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]

@@ -316,6 +316,11 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
 
 // fp32 -> f16 bits, round to nearest even; NaN -> 0x7E00.
 __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+  // The product must be rounded to fp32 before it is rounded to f16. Without this
+  // barrier the compiler folds "convert(a * b)" into one mixed-precision
+  // multiply-convert with a single rounding, which differs in the last bit for
+  // some inputs.
+  asm volatile("" : "+v"(f));
   const uint32_t u = __float_as_uint(f);
   if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7e00u;
   _Float16 h = (_Float16)f; // v_cvt_f16_f32: RNE

@@ -42,9 +42,18 @@ def raw(t: torch.Tensor) -> np.ndarray:
 
 
 def same_bits(a: torch.Tensor, b) -> bool:
+    """True if a and b hold the same bytes; otherwise fails with a short summary of the
+    first differences (never prints the tensors)."""
     bb = raw(b) if isinstance(b, torch.Tensor) else np.ascontiguousarray(b).reshape(-1).view(np.uint8)
     aa = raw(a)
-    return aa.size == bb.size and bool((aa == bb).all())
+    if aa.size != bb.size:
+        pytest.fail(f"size differs: {aa.size} vs {bb.size} bytes", pytrace=False)
+    bad = np.nonzero(aa != bb)[0]
+    if bad.size:
+        first = bad[:8]
+        pytest.fail(f"{bad.size} of {aa.size} bytes differ; first at byte offsets {first.tolist()}: "
+                    f"got {aa[first].tolist()} want {bb[first].tolist()}", pytrace=True)
+    return True
 
 
 def cpu_pool(L, NB, bs, H, D, dtype, seed, scale=1.0, fill=None):
@@ -570,24 +579,29 @@ def test_cfg2_full_size_migration_properties():
     for r, (si, di) in enumerate(tables):
         moved[di] = True
         for l in range(0, L, 3) if r % 4 else range(L):
-            assert torch.equal(dst[l][:, di], src[l][:, si]), f"request {r} layer {l}"
+            ok = bool(torch.equal(dst[l][:, di], src[l][:, si]))
+            assert ok, f"request {r} layer {l}"
     rest = (~moved).nonzero().squeeze(1)
     for l in range(L):
-        assert bool((dst[l][:, rest] == -1.0).all()), f"layer {l}: an untouched block changed"
+        ok = bool((dst[l][:, rest] == -1.0).all())
+        assert ok, f"layer {l}: an untouched block changed"
     # batched form: one launch for all 32 requests
     dst.fill_(-1.0)
     all_si = torch.cat([t[0] for t in tables])
     all_di = torch.cat([t[1] for t in tables])
     kv_ops.kv_unpack(dp, all_di, kv_ops.kv_pack(sp, all_si))
     for l in (0, 13, 27):
-        assert torch.equal(dst[l][:, all_di], src[l][:, all_si])
+        ok = bool(torch.equal(dst[l][:, all_di], src[l][:, all_si]))
+        assert ok, f"batched: layer {l}"
     # copy_blocks inside the source pool: half of the used blocks to free blocks
     P = off // 2
     mapping = torch.stack([sperm[:P], sperm[off:off + P]], 1).to(DEV)
     before = src[5][:, mapping[:, 0]].clone()
     kv_ops.copy_blocks(sp, mapping)
     for l in (0, 5, 27):
-        assert torch.equal(src[l][:, mapping[:, 1]], src[l][:, mapping[:, 0]])
-    assert torch.equal(src[5][:, mapping[:, 0]], before)
+        ok = bool(torch.equal(src[l][:, mapping[:, 1]], src[l][:, mapping[:, 0]]))
+        assert ok, f"copy_blocks: layer {l}"
+    ok = bool(torch.equal(src[5][:, mapping[:, 0]], before))
+    assert ok, "copy_blocks changed a source block"
     del src, dst
     torch.cuda.empty_cache()
