@@ -6,9 +6,9 @@ Workload (default, ``qwen2_7b_migrate``): the Qwen2-7B KV shape — 28 layers of
 requests with prompt lengths U{512..4096} plus a 1024-token image prefix
 (96..320 blocks each). One *step* moves every request of the batch: pack from the
 source pool under its block table into a contiguous transfer buffer
-(``KVWorker.extract_kv_blocks``), then unpack into a second, independently
-allocated pool under a different table (``KVWorker.write_kv_blocks``), request
-by request as the reference does. Everything is resident in HBM before the timed
+(``KVWorker.extract_kv_blocks``, one call per request as the reference does), then
+unpack every buffer into a second, independently allocated pool under a different
+table (``KVWorker.write_kv_blocks``, one call per request). Everything is resident in HBM before the timed
 region (pools, block tables); values are synthetic N(0, 0.5).
 
 Prints ONE JSON line. ``value`` is whole-job GB/s = algorithmic bytes (read +
@@ -42,6 +42,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements (append, batched, copy)")
     ap.add_argument("--variant", type=int, default=0, help="block-move launch variant (tuning)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one plain 1 GiB copy with the same tile engine (a kernel of known traffic, "
+                         "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     return ap.parse_args()
 
 
@@ -62,34 +65,35 @@ def make_requests(num_requests, num_blocks, seed):
     return tables, total
 
 
-def cpu_baseline(tables, L, bs, H, D, dtype, budget_s=20.0):
-    """The reference's torch path on the host cores, on a reduced pool (bytes moved depend
-    on the blocks per request, not on the pool size) and the first requests of the batch."""
+def cpu_baseline(tables, L, bs, H, D, dtype, budget_s=15.0):
+    """The reference's torch path on the host cores: the same batch (same block counts per
+    request) on pools reduced to just hold it — bytes moved depend on the blocks per request,
+    not on the pool size. Passes repeat until about `budget_s` seconds of CPU work are done."""
     from oracle import kv_oracle as orc
 
-    sample = tables[:8]
-    nb = sum(len(s) for s, _ in sample)
-    NBc = max(nb, 2048)
+    nb = sum(len(s) for s, _ in tables)
+    NBc = nb + 512
     torch.manual_seed(0)
-    src = [torch.randn((2, NBc, bs, H, D)).mul_(0.5).to(dtype) for _ in range(L)]
+    src = [torch.empty((2, NBc, bs, H, D), dtype=dtype).normal_(0.0, 0.5) for _ in range(L)]
     dst = [torch.zeros((2, NBc, bs, H, D), dtype=dtype) for _ in range(L)]
-    # remap the sample's tables into the reduced pool, keeping them scattered and disjoint
     g = torch.Generator().manual_seed(7)
     sp, dp = torch.randperm(NBc, generator=g), torch.randperm(NBc, generator=g)
     off, tabs = 0, []
-    for s, _ in sample:
+    for s, _ in tables:
         tabs.append((sp[off:off + len(s)].tolist(), dp[off:off + len(s)].tolist()))
         off += len(s)
     chunk = bs * H * D * src[0].element_size()
     bytes_per_pass = 4 * nb * L * 2 * chunk
     times = []
     t_start = time.perf_counter()
-    while len(times) < 5 and (time.perf_counter() - t_start < budget_s or len(times) < 2):
+    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 50):
         t0 = time.perf_counter()
-        for si, di in tabs:
-            buf = orc.ref_extract_kv_blocks(src, si)
+        bufs = [orc.ref_extract_kv_blocks(src, si) for si, _ in tabs]
+        for (_, di), buf in zip(tabs, bufs):
             orc.ref_write_kv_blocks(dst, di, buf)
+        del bufs
         times.append(time.perf_counter() - t0)
+    total = time.perf_counter() - t_start
     times.sort()
     med = times[len(times) // 2]
     return {
@@ -97,9 +101,9 @@ def cpu_baseline(tables, L, bs, H, D, dtype, budget_s=20.0):
         "unit": "GB/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"first {len(sample)} of the batch's requests ({nb} blocks, {bytes_per_pass / 1e9:.2f} GB algorithmic "
-                  f"per pass) on pools reduced to {NBc} blocks; torch index + stack / indexed assignment on CPU; "
-                  f"median of {len(times)} passes ({med:.2f} s each)",
+        "sample": f"the whole batch ({len(tabs)} requests, {nb} blocks, {bytes_per_pass / 1e9:.2f} GB algorithmic per "
+                  f"pass) on host pools reduced to {NBc} blocks; the reference's torch indexing + stack / indexed "
+                  f"assignment on CPU tensors; median of {len(times)} passes over {total:.1f} s ({med:.2f} s each)",
     }
 
 
@@ -142,17 +146,23 @@ def main():
     bytes_per_step = 4 * payload                 # pack: read + write, unpack: read + write
 
     def step(events=None):
-        for si, di in dev_tables:
-            if events is not None:
-                e0, e1, e2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
-                e0.record()
-            buf = src_w.extract_kv_blocks(si)
-            if events is not None:
-                e1.record()
-            dst_w.write_kv_blocks(di, buf)
-            if events is not None:
-                e2.record()
-                events.append((e0, e1, e2, si.numel()))
+        # pack every request on the source side, then unpack every request on the destination
+        # side: 6 GB of transfer buffers lie between a buffer's pack and its unpack, so the
+        # unpack reads come from HBM (not from the 256 MB Infinity Cache) as they would on a
+        # receiving GPU.
+        # HIP events bracket each phase (3 per step, on the launch stream), not each launch: an
+        # event record between every two kernels costs several microseconds of idle GPU.
+        if events is not None:
+            e0, e1, e2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+            e0.record()
+        bufs = [src_w.extract_kv_blocks(si) for si, _ in dev_tables]
+        if events is not None:
+            e1.record()
+        for k, (_, di) in enumerate(dev_tables):
+            dst_w.write_kv_blocks(di, bufs[k])
+        if events is not None:
+            e2.record()
+            events.append((e0, e1, e2))
 
     for _ in range(args.warmup):
         step()
@@ -167,11 +177,12 @@ def main():
     ms_per_step = wall / args.steps * 1e3
     value = bytes_per_step * args.steps / wall / 1e9
 
-    # per-launch kernel time of the block-move kernel (pack and unpack instances)
-    pack_ms = sum(e0.elapsed_time(e1) for e0, e1, _, _ in events)
-    unpack_ms = sum(e1.elapsed_time(e2) for _, e1, e2, _ in events)
-    launches = 2 * len(events)
-    kern_bytes = sum(2 * 2 * n * L * 2 * chunk for *_, n in events)  # per request: pack 2x + unpack 2x payload
+    # kernel time of the block-move kernel (pack and unpack instances) from the phase events:
+    # each phase is 32 back-to-back launches of that kernel and nothing else
+    pack_ms = sum(e0.elapsed_time(e1) for e0, e1, _ in events)
+    unpack_ms = sum(e1.elapsed_time(e2) for _, e1, e2 in events)
+    launches = 2 * len(dev_tables) * len(events)
+    kern_bytes = 2 * 2 * payload * len(events)  # per step: pack 2 x payload + unpack 2 x payload
     achieved = kern_bytes / ((pack_ms + unpack_ms) * 1e-3) / 1e9
     roofline = {
         "bound": "hbm",
@@ -187,6 +198,13 @@ def main():
         "pack_GBps": round(kern_bytes / 2 / (pack_ms * 1e-3) / 1e9, 1),
         "unpack_GBps": round(kern_bytes / 2 / (unpack_ms * 1e-3) / 1e9, 1),
     }
+
+    if args.calibrate_copy:
+        a = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+        b = torch.empty_like(a)
+        kv_ops.stream_copy(a, b)
+        torch.cuda.synchronize()
+        del a, b
 
     # spot check inside the bench: the last request really arrived
     si, di = dev_tables[-1]
@@ -212,7 +230,7 @@ def main():
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "config": {
             "workload": "qwen2_7b_migrate: 28 layers x [2,%d,16,4,128] bf16 x 2 pools, %d requests (%d blocks, "
-                        "%.2f GB payload), per-request pack -> unpack under a different block table"
+                        "%.2f GB payload), 32 per-request packs, then 32 per-request unpacks under different block tables"
                         % (NB, len(tables), total_blocks, payload / 1e9),
             "num_layers": L, "num_blocks": NB, "block_size": bs, "kv_heads": H, "head_dim": D,
             "requests": len(tables), "blocks_moved": total_blocks, "algorithmic_bytes_per_step": bytes_per_step,
@@ -260,6 +278,12 @@ def secondary(src_w, dst_w, dev_tables, payload, L, bs, H, D, NB, dev):
     out["batched_unpack_GBps"] = round(2 * payload / (med * 1e-3) / 1e9, 1)
     med, mn = timed(lambda: kv_ops.kv_migrate(sp, all_si, dp, all_di), 10)
     out["fused_migrate_GBps"] = round(2 * payload / (med * 1e-3) / 1e9, 1)
+    def interleaved():
+        for si, di in dev_tables:
+            dst_w.write_kv_blocks(di, src_w.extract_kv_blocks(si))
+
+    med, mn = timed(interleaved, 5)
+    out["per_request_pack_then_unpack_interleaved_GBps"] = round(4 * payload / (med * 1e-3) / 1e9, 1)
     # yardsticks: plain copies of the same byte count
     flat = buf.view(-1)
     other = torch.empty_like(flat)

@@ -57,182 +57,277 @@ template <> struct VecOf<4> { typedef uint32_t type; };
 template <> struct VecOf<2> { typedef uint16_t type; };
 template <> struct VecOf<1> { typedef uint8_t type; };
 
+// Cache policies of the streaming accessors. Loads are always non-temporal.
+//   0  store nt                (compiler builtin)
+//   1  store sc0 sc1           (system-scope write-through)
+//   2  store sc0 sc1 nt
+//   3  plain load / plain store
+// The sc0/sc1 forms exist only as instruction modifiers, so 16-byte stores under
+// policies 1 and 2 are emitted with a one-line asm statement (a vector store).
+// Every pointer these kernels dereference is device (global) memory. Saying so in
+// the pointer type keeps the accesses global_load / global_store even where a
+// pointer has passed through an opaque asm statement (a generic pointer would
+// become a slower flat access).
+#define EMM_GLOBAL __attribute__((address_space(1)))
+
 template <typename V, bool NT>
 __device__ __forceinline__ V ld(const char *p) {
+  const EMM_GLOBAL V *g = (const EMM_GLOBAL V *)(p);
   if constexpr (NT)
-    return __builtin_nontemporal_load(reinterpret_cast<const V *>(p));
+    return __builtin_nontemporal_load(g);
   else
-    return *reinterpret_cast<const V *>(p);
+    return *g;
 }
 
 template <typename V, bool NT>
 __device__ __forceinline__ void st(char *p, V v) {
+  EMM_GLOBAL V *g = (EMM_GLOBAL V *)(p);
   if constexpr (NT)
-    __builtin_nontemporal_store(v, reinterpret_cast<V *>(p));
+    __builtin_nontemporal_store(v, g);
   else
-    *reinterpret_cast<V *>(p) = v;
+    *g = v;
 }
 
-constexpr int kThreads = 256; // 4 wavefronts of 64 lanes
+template <typename V, int POLICY>
+__device__ __forceinline__ V ld_stream(const char *p) {
+  return ld<V, POLICY != 3>(p);
+}
 
-// Copy one tile of U * kThreads vectors: vector (u * kThreads + tid) of the
-// tile. All U loads are in flight before the first store. `limit` is the number
-// of bytes valid from `src`/`dst` on (tail tiles are predicated per lane).
-template <typename V, int U, bool NTL, bool NTS>
-__device__ __forceinline__ void copy_tile(const char *__restrict__ src,
-                                          char *__restrict__ dst,
-                                          int64_t limit) {
+template <typename V, int POLICY>
+__device__ __forceinline__ void st_stream(char *p, V v) {
+  if constexpr (sizeof(V) == 16 && POLICY == 1) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+  } else if constexpr (sizeof(V) == 16 && POLICY == 2) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt" ::"v"(p), "v"(v) : "memory");
+  } else {
+    st<V, POLICY != 3>(p, v);
+  }
+}
+
+// A value that is the same in every lane, moved to scalar registers.
+__device__ __forceinline__ int64_t uniform64(int64_t x) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)x);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)x >> 32));
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
+constexpr int kThreads = 256; // 4 wavefronts of 64 lanes (append / dequant / concat kernels)
+
+// A tile is U * T vectors; lane `tid` owns vectors (u * T + tid). All U loads of a
+// tile are in flight before the first store. `limit` is the number of bytes valid
+// from the tile start on (tail tiles are predicated per lane): lanes past the end
+// re-read vector 0 (always valid, limit > 0) so the loads stay unconditional;
+// only the stores are predicated.
+template <typename V, int T, int U, int POLICY>
+__device__ __forceinline__ void load_tile(V (&v)[U], const char *__restrict__ src, int64_t limit) {
   constexpr int64_t VB = sizeof(V);
   const int64_t lane_off = (int64_t)threadIdx.x * VB;
-  V v[U];
-  if (limit >= (int64_t)U * kThreads * VB) {
+  if (limit >= (int64_t)U * T * VB) {
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      v[u] = ld<V, NTL>(src + lane_off + (int64_t)u * kThreads * VB);
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-      st<V, NTS>(dst + lane_off + (int64_t)u * kThreads * VB, v[u]);
+      v[u] = ld_stream<V, POLICY>(src + lane_off + (int64_t)u * T * VB);
   } else {
-    // tail tile: lanes past the end re-read vector 0 (always valid, limit > 0)
-    // so the loads stay unconditional and in flight together; only the stores
-    // are predicated
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int64_t off = lane_off + (int64_t)u * kThreads * VB;
-      v[u] = ld<V, NTL>(src + (off < limit ? off : 0));
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int64_t off = lane_off + (int64_t)u * kThreads * VB;
-      if (off < limit) st<V, NTS>(dst + off, v[u]);
+      const int64_t off = lane_off + (int64_t)u * T * VB;
+      v[u] = ld_stream<V, POLICY>(src + (off < limit ? off : 0));
     }
   }
+}
+
+template <typename V, int T, int U, int POLICY>
+__device__ __forceinline__ void store_tile(const V (&v)[U], char *__restrict__ dst, int64_t limit) {
+  constexpr int64_t VB = sizeof(V);
+  const int64_t lane_off = (int64_t)threadIdx.x * VB;
+  if (limit >= (int64_t)U * T * VB) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      st_stream<V, POLICY>(dst + lane_off + (int64_t)u * T * VB, v[u]);
+  } else {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t off = lane_off + (int64_t)u * T * VB;
+      if (off < limit) st_stream<V, POLICY>(dst + off, v[u]);
+    }
+  }
+}
+
+template <typename V, int T, int U, int POLICY>
+__device__ __forceinline__ void copy_tile(const char *__restrict__ src, char *__restrict__ dst,
+                                          int64_t limit) {
+  V v[U];
+  load_tile<V, T, U, POLICY>(v, src, limit);
+  store_tile<V, T, U, POLICY>(v, dst, limit);
 }
 
 // ----------------------------------------------------------------------------
 // block move: pack / unpack / copy_blocks / migrate / plain copy
 // ----------------------------------------------------------------------------
-// One side of a move is either a block pool (per-layer base pointers, block
-// chosen through an int64 index array) or a linear transfer buffer.
+// One side of a move is either a block pool (one base pointer per (layer, K|V)
+// plane, block chosen through an int64 index array) or a linear transfer
+// buffer [planes, n, chunk].
+constexpr int kMaxPlanes = 2 * EMM_MAX_LAYERS;
+constexpr int kMaxGridY = 65535;
+constexpr int kRun = 16; // blocks per plane visit in the pool-to-pool order
+
 struct MoveParams {
-  const char *src_layers[EMM_MAX_LAYERS]; // pool source: per-layer bases
-  char *dst_layers[EMM_MAX_LAYERS];       // pool destination: per-layer bases
-  const char *src_linear;                 // linear source base
-  char *dst_linear;                       // linear destination base
-  const int64_t *src_idx;                 // block ids on the source side
-  const int64_t *dst_idx;                 // block ids on the destination side
-  int64_t idx_stride;                     // elements between consecutive ids
+  const char *src_planes[kMaxPlanes]; // pool source: base of each (layer, kv) plane
+  char *dst_planes[kMaxPlanes];       // pool destination
+  const char *src_linear;             // linear source base
+  char *dst_linear;                   // linear destination base
+  const int64_t *src_idx;             // block ids on the source side
+  const int64_t *dst_idx;             // block ids on the destination side
+  int64_t idx_stride;                 // elements between consecutive ids
   int64_t src_num_blocks;
   int64_t dst_num_blocks;
   int64_t chunk_bytes;
-  int64_t n;                // blocks moved per (layer, kv) plane
-  uint32_t tiles_per_chunk; // ceil(chunk_bytes / tile_bytes)
-  uint32_t num_kv;
+  int64_t n;      // blocks per plane of the linear buffer
+  int64_t j0;     // first block of this launch
+  int64_t j_end;  // one past the last block of this launch
+  int64_t plane0; // first plane of this launch (linear side)
 };
 
-// grid: x = n * tiles_per_chunk, y = num_kv, z = num_layers. The x-major
-// dispatch order walks the transfer buffer linearly.
-template <typename V, int U, bool SRC_POOL, bool DST_POOL, bool NTL, bool NTS>
-__global__ __launch_bounds__(kThreads) void emm_block_move_kernel(
-    const MoveParams p) {
-  constexpr int64_t TILE = (int64_t)U * kThreads * sizeof(V);
-  uint32_t j = blockIdx.x, tile = 0;
-  if (p.tiles_per_chunk != 1) {
-    j = blockIdx.x / p.tiles_per_chunk;
-    tile = blockIdx.x - j * p.tiles_per_chunk;
-  }
-  const uint32_t kv = blockIdx.y;
-  const uint32_t l = blockIdx.z;
-  const int64_t chunk = p.chunk_bytes;
-  const int64_t tile_off = (int64_t)tile * TILE;
-  const int64_t linear_off =
-      (((int64_t)l * p.num_kv + kv) * p.n + j) * chunk + tile_off;
-
-  const char *src;
-  if constexpr (SRC_POOL) {
-    const int64_t b = p.src_idx[(int64_t)j * p.idx_stride];
-    if ((uint64_t)b >= (uint64_t)p.src_num_blocks) return; // padding / invalid
-    src = p.src_layers[l] + ((int64_t)kv * p.src_num_blocks + b) * chunk + tile_off;
+// grid: x = tiles of one chunk, y = blocks (at most kMaxGridY per launch),
+// z = planes. Dispatch order (x fastest, then y, then z) walks the transfer
+// buffer linearly; no integer division is needed to find a workgroup's tile.
+//
+// When both sides are pools (copy_blocks, migrate) the order is different: runs
+// of kRun consecutive blocks per plane, planes next, runs last (y = plane * kRun
+// + position in the run, z = run), so that the workgroups in flight at any moment
+// touch every plane of the pool instead of one plane's window, while a table of
+// consecutive block ids still gives sequential runs. Measured on MI355X this is
+// about 12 % faster for scattered pool-to-pool moves; with a linear side it is
+// slower (the linear buffer would be read as one stream per plane).
+template <typename V, int T, int U, bool SRC_POOL, bool DST_POOL, int POLICY>
+__global__ __launch_bounds__(T) void emm_block_move_kernel(const MoveParams p) {
+  constexpr int64_t TILE = (int64_t)U * T * sizeof(V);
+  constexpr bool PLANE_FASTEST = SRC_POOL && DST_POOL;
+  uint32_t pl;
+  int64_t j;
+  if constexpr (PLANE_FASTEST) {
+    // y = plane * kRun + position in a run of kRun consecutive blocks, z = run
+    pl = blockIdx.y / kRun;
+    // every plane starts at its own run: planes whose bases differ by a highly
+    // aligned stride then do not hit the same memory channels at the same time
+    uint32_t run = blockIdx.z + pl * (gridDim.z / (gridDim.y / kRun));
+    if (run >= gridDim.z) run -= gridDim.z;
+    j = p.j0 + (int64_t)run * kRun + (blockIdx.y % kRun);
+    if (j >= p.j_end) return;
   } else {
-    src = p.src_linear + linear_off;
+    pl = blockIdx.z;
+    j = p.j0 + blockIdx.y;
+  }
+  const int64_t chunk = p.chunk_bytes;
+  const int64_t tile_off = (int64_t)blockIdx.x * TILE;
+  const int64_t linear_off = ((p.plane0 + pl) * p.n + j) * chunk + tile_off;
+
+  const int64_t limit = chunk - tile_off;
+  // The scalar work of a workgroup is a chain of dependent fetches (arguments ->
+  // block ids -> data). The empty asm statements below pin values in scalar
+  // registers at the point where they stand, which keeps the chain at its
+  // minimum: (1) plane bases arrive with the first batch of argument loads,
+  // (2) both block ids are fetched together and waited for once, and (3) loads
+  // from a linear source, which depend on no id, are issued before that wait.
+  const char *src_plane = nullptr;
+  char *dst_plane = nullptr;
+  if constexpr (SRC_POOL) {
+    src_plane = p.src_planes[pl];
+    asm volatile("" : "+s"(src_plane));
+  }
+  if constexpr (DST_POOL) {
+    dst_plane = p.dst_planes[pl];
+    asm volatile("" : "+s"(dst_plane));
+  }
+  int64_t sb = 0, db = 0;
+  if constexpr (SRC_POOL) sb = p.src_idx[j * p.idx_stride];
+  if constexpr (DST_POOL) db = p.dst_idx[j * p.idx_stride];
+  V v[U];
+  if constexpr (!SRC_POOL) load_tile<V, T, U, POLICY>(v, p.src_linear + linear_off, limit);
+  sb = uniform64(sb);
+  db = uniform64(db);
+  asm volatile("" : "+s"(sb), "+s"(db) : : "memory");
+  if constexpr (SRC_POOL) {
+    if ((uint64_t)sb >= (uint64_t)p.src_num_blocks) return; // padding / invalid
+    load_tile<V, T, U, POLICY>(v, src_plane + sb * chunk + tile_off, limit);
   }
   char *dst;
   if constexpr (DST_POOL) {
-    const int64_t b = p.dst_idx[(int64_t)j * p.idx_stride];
-    if ((uint64_t)b >= (uint64_t)p.dst_num_blocks) return;
-    dst = p.dst_layers[l] + ((int64_t)kv * p.dst_num_blocks + b) * chunk + tile_off;
+    if ((uint64_t)db >= (uint64_t)p.dst_num_blocks) return;
+    dst = dst_plane + db * chunk + tile_off;
   } else {
     dst = p.dst_linear + linear_off;
   }
-  copy_tile<V, U, NTL, NTS>(src, dst, chunk - tile_off);
+  store_tile<V, T, U, POLICY>(v, dst, limit);
 }
 
+// Launch variant of the 16-byte path: bits 0-3 vectors per lane (1, 2, 4),
+// bits 4-7 workgroup size code (0: 256, 1: 64), bits 8-11 cache policy + 1.
+// 0 selects the default.
 int g_move_variant = 0;
-
-struct MoveCfg {
-  int vec;  // bytes per lane access
-  int unroll;
-  bool ntl, nts;
-};
 
 bool aligned(const void *p, int a) { return ((uintptr_t)p & (uintptr_t)(a - 1)) == 0; }
 
-template <typename V, int U, bool SP, bool DP>
-void launch_move_nt(const MoveParams &p, dim3 grid, bool ntl, bool nts, hipStream_t s) {
-  if (ntl && nts)
-    emm_block_move_kernel<V, U, SP, DP, true, true><<<grid, kThreads, 0, s>>>(p);
-  else if (ntl)
-    emm_block_move_kernel<V, U, SP, DP, true, false><<<grid, kThreads, 0, s>>>(p);
-  else if (nts)
-    emm_block_move_kernel<V, U, SP, DP, false, true><<<grid, kThreads, 0, s>>>(p);
-  else
-    emm_block_move_kernel<V, U, SP, DP, false, false><<<grid, kThreads, 0, s>>>(p);
+template <typename V, int T, int U, bool SP, bool DP>
+void launch_move_policy(const MoveParams &p, dim3 grid, int policy, hipStream_t s) {
+  switch (policy) {
+  case 1: emm_block_move_kernel<V, T, U, SP, DP, 1><<<grid, T, 0, s>>>(p); break;
+  case 2: emm_block_move_kernel<V, T, U, SP, DP, 2><<<grid, T, 0, s>>>(p); break;
+  case 3: emm_block_move_kernel<V, T, U, SP, DP, 3><<<grid, T, 0, s>>>(p); break;
+  default: emm_block_move_kernel<V, T, U, SP, DP, 0><<<grid, T, 0, s>>>(p); break;
+  }
 }
 
 template <bool SP, bool DP>
-int launch_move(MoveParams &p, int num_layers, int min_align, hipStream_t s,
-                const char *what) {
-  if (p.n == 0 || num_layers == 0 || p.num_kv == 0 || p.chunk_bytes == 0) return EMM_OK;
+int launch_move(MoveParams &p, int planes, int min_align, hipStream_t s, const char *what) {
+  if (p.n == 0 || planes == 0 || p.chunk_bytes == 0) return EMM_OK;
   // widest lane access that divides the chunk and every base address
   int vec = 16;
   while (vec > 1 && (p.chunk_bytes % vec != 0 || min_align % vec != 0)) vec >>= 1;
   if (vec == 8) vec = 4; // 8-byte lanes are not instantiated
-  int unroll = 4;
-  bool ntl = true, nts = true;
+  int threads = 256, unroll = 1, policy = 1;
   if (vec == 16 && g_move_variant > 0) {
-    const int u = g_move_variant & 0xff;
-    if (u == 1 || u == 2 || u == 4 || u == 8) unroll = u;
-    if (g_move_variant & 0x100) ntl = false;
-    if (g_move_variant & 0x200) nts = false;
+    const int u = g_move_variant & 0xf;
+    if (u == 1 || u == 2 || u == 4) unroll = u;
+    if (((g_move_variant >> 4) & 0xf) == 1) threads = 64;
+    const int pc = (g_move_variant >> 8) & 0xf;
+    if (pc >= 1 && pc <= 4) policy = pc - 1;
   }
-  // do not make the tile larger than the chunk needs
-  if (vec == 16)
-    while (unroll > 1 && (int64_t)(unroll / 2) * kThreads * vec >= p.chunk_bytes) unroll >>= 1;
-  const int64_t tile_bytes = (int64_t)unroll * kThreads * vec;
+  if (vec != 16) { threads = 256; unroll = 4; policy = 0; }
+  const int64_t tile_bytes = (int64_t)unroll * threads * vec;
   const int64_t tpc = (p.chunk_bytes + tile_bytes - 1) / tile_bytes;
-  const int64_t gx = p.n * tpc;
-  if (tpc > 0x7fffffffLL || gx > 0x7fffffffLL)
-    return fail(EMM_EINVAL, "%s: n * tiles_per_chunk = %lld exceeds the grid limit", what, (long long)gx);
-  if (num_layers > 65535 || p.num_kv > 65535)
-    return fail(EMM_EINVAL, "%s: num_layers / num_kv exceed the grid limit", what);
-  p.tiles_per_chunk = (uint32_t)tpc;
-  dim3 grid((uint32_t)gx, p.num_kv, (uint32_t)num_layers);
+  if (tpc > 0x7fffffffLL)
+    return fail(EMM_EINVAL, "%s: chunk of %lld bytes needs too many tiles", what, (long long)p.chunk_bytes);
 
-#define EMM_MOVE_CASE(VB, UU)                                                          \
-  if (vec == VB && unroll == UU) {                                                     \
-    launch_move_nt<typename VecOf<VB>::type, UU, SP, DP>(p, grid, ntl, nts, s);        \
-    return check_launch(what);                                                         \
+  const int64_t j_begin = p.j0, j_end = p.j0 + p.n;
+  for (int64_t j0 = j_begin; j0 < j_end; j0 += kMaxGridY) {
+    const int64_t ny = (j_end - j0 < kMaxGridY) ? (j_end - j0) : kMaxGridY;
+    MoveParams q = p;
+    q.j0 = j0;
+    q.j_end = j0 + ny;
+    dim3 grid((uint32_t)tpc, (uint32_t)ny, (uint32_t)planes);
+    if (SP && DP) grid = dim3((uint32_t)tpc, (uint32_t)(planes * kRun), (uint32_t)((ny + kRun - 1) / kRun));
+    bool done = false;
+#define EMM_MOVE_CASE(VB, TT, UU)                                                           \
+  if (!done && vec == VB && threads == TT && unroll == UU) {                                \
+    launch_move_policy<typename VecOf<VB>::type, TT, UU, SP, DP>(q, grid, policy, s);       \
+    done = true;                                                                            \
   }
-  EMM_MOVE_CASE(16, 8)
-  EMM_MOVE_CASE(16, 4)
-  EMM_MOVE_CASE(16, 2)
-  EMM_MOVE_CASE(16, 1)
-  // rare unaligned shapes: narrower lanes, one fixed tile shape
-  EMM_MOVE_CASE(4, 4)
-  EMM_MOVE_CASE(2, 4)
-  EMM_MOVE_CASE(1, 4)
+    EMM_MOVE_CASE(16, 256, 1)
+    EMM_MOVE_CASE(16, 256, 2)
+    EMM_MOVE_CASE(16, 256, 4)
+    EMM_MOVE_CASE(16, 64, 1)
+    EMM_MOVE_CASE(16, 64, 2)
+    EMM_MOVE_CASE(16, 64, 4)
+    // rare unaligned shapes: narrower lanes, one fixed tile shape
+    EMM_MOVE_CASE(4, 256, 4)
+    EMM_MOVE_CASE(2, 256, 4)
+    EMM_MOVE_CASE(1, 256, 4)
 #undef EMM_MOVE_CASE
-  return fail(EMM_EINVAL, "%s: no kernel for vec=%d unroll=%d", what, vec, unroll);
+    if (!done) return fail(EMM_EINVAL, "%s: no kernel for vec=%d threads=%d unroll=%d", what, vec, threads, unroll);
+    const int rc = check_launch(what);
+    if (rc != EMM_OK) return rc;
+  }
+  return EMM_OK;
 }
 
 int common_align(int a, const void *p) {
@@ -252,6 +347,47 @@ int check_pool_args(const char *what, const void *const *layer_ptrs, int num_lay
   for (int l = 0; l < num_layers; ++l)
     if (!layer_ptrs[l] && n > 0 && num_blocks > 0)
       return fail(EMM_EINVAL, "%s: layer_ptrs[%d] is null", what, l);
+  return EMM_OK;
+}
+
+// Build the plane tables for groups of at most kMaxPlanes (layer, kv) planes and
+// launch. A null layer table means that side is the linear buffer.
+template <bool SP, bool DP>
+int move_planes(const void *const *src_layers, int64_t src_nb, void *const *dst_layers,
+                int64_t dst_nb, int num_layers, int num_kv, int64_t chunk,
+                const int64_t *src_idx, const int64_t *dst_idx, int64_t idx_stride, int64_t n,
+                const void *src_linear, void *dst_linear, hipStream_t s, const char *what) {
+  int al = 16;
+  if (!SP) al = common_align(al, src_linear);
+  if (!DP) al = common_align(al, dst_linear);
+  for (int l = 0; l < num_layers; ++l) {
+    if (SP) al = common_align(al, src_layers[l]);
+    if (DP) al = common_align(al, dst_layers[l]);
+  }
+  const int64_t planes = (int64_t)num_layers * num_kv;
+  for (int64_t pl0 = 0; pl0 < planes; pl0 += kMaxPlanes) {
+    const int cnt = (int)((planes - pl0 < kMaxPlanes) ? (planes - pl0) : kMaxPlanes);
+    MoveParams p;
+    memset(&p, 0, sizeof(p));
+    for (int i = 0; i < cnt; ++i) {
+      const int64_t l = (pl0 + i) / num_kv, kv = (pl0 + i) % num_kv;
+      if (SP) p.src_planes[i] = (const char *)src_layers[l] + kv * src_nb * chunk;
+      if (DP) p.dst_planes[i] = (char *)dst_layers[l] + kv * dst_nb * chunk;
+    }
+    p.src_linear = (const char *)src_linear;
+    p.dst_linear = (char *)dst_linear;
+    p.src_idx = src_idx;
+    p.dst_idx = dst_idx;
+    p.idx_stride = idx_stride;
+    p.src_num_blocks = src_nb;
+    p.dst_num_blocks = dst_nb;
+    p.chunk_bytes = chunk;
+    p.n = n;
+    p.j0 = 0;
+    p.plane0 = pl0;
+    const int rc = launch_move<SP, DP>(p, cnt, al, s, what);
+    if (rc != EMM_OK) return rc;
+  }
   return EMM_OK;
 }
 
@@ -678,7 +814,7 @@ __global__ __launch_bounds__(kThreads) void emm_concat_rows_kernel(const ConcatP
     if (p.tile_start[mid] <= w) lo = mid; else hi = mid - 1;
   }
   const int64_t off = (int64_t)(w - p.tile_start[lo]) * TILE;
-  copy_tile<V, U, true, true>(p.src[lo] + off, p.dst + p.dst_off[lo] + off, p.nbytes[lo] - off);
+  copy_tile<V, kThreads, U, 0>(p.src[lo] + off, p.dst + p.dst_off[lo] + off, p.nbytes[lo] - off);
 }
 
 hipStream_t as_stream(emm_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
@@ -706,21 +842,9 @@ int emm_kv_pack(const void *const *layer_ptrs, int num_layers, int num_kv,
   if (rc != EMM_OK) return rc;
   if (n == 0 || num_layers == 0 || num_kv == 0 || chunk_bytes == 0) return EMM_OK;
   if (!block_idx || !packed) return fail(EMM_EINVAL, "emm_kv_pack: null block_idx / packed");
-  MoveParams p;
-  memset(&p, 0, sizeof(p));
-  int al = common_align(16, packed);
-  for (int l = 0; l < num_layers; ++l) {
-    p.src_layers[l] = (const char *)layer_ptrs[l];
-    al = common_align(al, layer_ptrs[l]);
-  }
-  p.dst_linear = (char *)packed;
-  p.src_idx = block_idx;
-  p.idx_stride = 1;
-  p.src_num_blocks = num_blocks;
-  p.chunk_bytes = chunk_bytes;
-  p.n = n;
-  p.num_kv = (uint32_t)num_kv;
-  return launch_move<true, false>(p, num_layers, al, as_stream(stream), "emm_kv_pack");
+  return move_planes<true, false>(layer_ptrs, num_blocks, nullptr, 0, num_layers, num_kv, chunk_bytes,
+                                  block_idx, nullptr, 1, n, nullptr, packed, as_stream(stream),
+                                  "emm_kv_pack");
 }
 
 int emm_kv_unpack(void *const *layer_ptrs, int num_layers, int num_kv,
@@ -731,21 +855,9 @@ int emm_kv_unpack(void *const *layer_ptrs, int num_layers, int num_kv,
   if (rc != EMM_OK) return rc;
   if (n == 0 || num_layers == 0 || num_kv == 0 || chunk_bytes == 0) return EMM_OK;
   if (!block_idx || !packed) return fail(EMM_EINVAL, "emm_kv_unpack: null block_idx / packed");
-  MoveParams p;
-  memset(&p, 0, sizeof(p));
-  int al = common_align(16, packed);
-  for (int l = 0; l < num_layers; ++l) {
-    p.dst_layers[l] = (char *)layer_ptrs[l];
-    al = common_align(al, layer_ptrs[l]);
-  }
-  p.src_linear = (const char *)packed;
-  p.dst_idx = block_idx;
-  p.idx_stride = 1;
-  p.dst_num_blocks = num_blocks;
-  p.chunk_bytes = chunk_bytes;
-  p.n = n;
-  p.num_kv = (uint32_t)num_kv;
-  return launch_move<false, true>(p, num_layers, al, as_stream(stream), "emm_kv_unpack");
+  return move_planes<false, true>(nullptr, 0, layer_ptrs, num_blocks, num_layers, num_kv, chunk_bytes,
+                                  nullptr, block_idx, 1, n, packed, nullptr, as_stream(stream),
+                                  "emm_kv_unpack");
 }
 
 int emm_copy_blocks(void *const *layer_ptrs, int num_layers, int num_kv,
@@ -756,23 +868,9 @@ int emm_copy_blocks(void *const *layer_ptrs, int num_layers, int num_kv,
   if (rc != EMM_OK) return rc;
   if (num_pairs == 0 || num_layers == 0 || num_kv == 0 || chunk_bytes == 0) return EMM_OK;
   if (!block_mapping) return fail(EMM_EINVAL, "emm_copy_blocks: null block_mapping");
-  MoveParams p;
-  memset(&p, 0, sizeof(p));
-  int al = 16;
-  for (int l = 0; l < num_layers; ++l) {
-    p.src_layers[l] = (const char *)layer_ptrs[l];
-    p.dst_layers[l] = (char *)layer_ptrs[l];
-    al = common_align(al, layer_ptrs[l]);
-  }
-  p.src_idx = block_mapping;
-  p.dst_idx = block_mapping + 1;
-  p.idx_stride = 2;
-  p.src_num_blocks = num_blocks;
-  p.dst_num_blocks = num_blocks;
-  p.chunk_bytes = chunk_bytes;
-  p.n = num_pairs;
-  p.num_kv = (uint32_t)num_kv;
-  return launch_move<true, true>(p, num_layers, al, as_stream(stream), "emm_copy_blocks");
+  return move_planes<true, true>((const void *const *)layer_ptrs, num_blocks, layer_ptrs, num_blocks,
+                                 num_layers, num_kv, chunk_bytes, block_mapping, block_mapping + 1, 2,
+                                 num_pairs, nullptr, nullptr, as_stream(stream), "emm_copy_blocks");
 }
 
 int emm_kv_migrate(const void *const *src_layer_ptrs, int64_t src_num_blocks,
@@ -787,39 +885,17 @@ int emm_kv_migrate(const void *const *src_layer_ptrs, int64_t src_num_blocks,
   if (rc != EMM_OK) return rc;
   if (n == 0 || num_layers == 0 || num_kv == 0 || chunk_bytes == 0) return EMM_OK;
   if (!src_idx || !dst_idx) return fail(EMM_EINVAL, "emm_kv_migrate: null index array");
-  MoveParams p;
-  memset(&p, 0, sizeof(p));
-  int al = 16;
-  for (int l = 0; l < num_layers; ++l) {
-    p.src_layers[l] = (const char *)src_layer_ptrs[l];
-    p.dst_layers[l] = (char *)dst_layer_ptrs[l];
-    al = common_align(al, src_layer_ptrs[l]);
-    al = common_align(al, dst_layer_ptrs[l]);
-  }
-  p.src_idx = src_idx;
-  p.dst_idx = dst_idx;
-  p.idx_stride = 1;
-  p.src_num_blocks = src_num_blocks;
-  p.dst_num_blocks = dst_num_blocks;
-  p.chunk_bytes = chunk_bytes;
-  p.n = n;
-  p.num_kv = (uint32_t)num_kv;
-  return launch_move<true, true>(p, num_layers, al, as_stream(stream), "emm_kv_migrate");
+  return move_planes<true, true>(src_layer_ptrs, src_num_blocks, dst_layer_ptrs, dst_num_blocks,
+                                 num_layers, num_kv, chunk_bytes, src_idx, dst_idx, 1, n, nullptr,
+                                 nullptr, as_stream(stream), "emm_kv_migrate");
 }
 
 int emm_stream_copy(const void *src, void *dst, int64_t nbytes, emm_stream_t stream) {
   if (nbytes < 0) return fail(EMM_EINVAL, "emm_stream_copy: negative size");
   if (nbytes == 0) return EMM_OK;
   if (!src || !dst) return fail(EMM_EINVAL, "emm_stream_copy: null pointer");
-  MoveParams p;
-  memset(&p, 0, sizeof(p));
-  p.src_linear = (const char *)src;
-  p.dst_linear = (char *)dst;
-  p.chunk_bytes = nbytes;
-  p.n = 1;
-  p.num_kv = 1;
-  int al = common_align(common_align(16, src), dst);
-  return launch_move<false, false>(p, 1, al, as_stream(stream), "emm_stream_copy");
+  return move_planes<false, false>(nullptr, 0, nullptr, 0, 1, 1, nbytes, nullptr, nullptr, 1, 1, src,
+                                   dst, as_stream(stream), "emm_stream_copy");
 }
 
 int emm_kv_unpack_dequant_fp8(void *const *layer_ptrs, int num_layers, int64_t num_blocks,
