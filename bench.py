@@ -42,6 +42,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements (append, batched, copy)")
     ap.add_argument("--variant", type=int, default=0, help="block-move launch variant (tuning)")
+    ap.add_argument("--extended", action="store_true",
+                    help="after the headline, free its pools and measure the fp8 70B-class shape and the ~200 GB "
+                         "rebalancing shape at full size (adds about a minute)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB copy with the same tile engine (a kernel of known traffic, "
                          "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -217,6 +220,13 @@ def main():
     if not args.no_extra:
         extra = secondary(src_w, dst_w, dev_tables, payload, L, bs, H, D, NB, dev)
 
+    if args.extended:
+        src_w.kv_cache = dst_w.kv_cache = None
+        src_w._pool = dst_w._pool = None
+        dev_tables = None
+        torch.cuda.empty_cache()
+        extra["extended"] = extended(dev)
+
     result = {
         "metric": "KV pack+unpack GB/s",
         "value": round(value, 1),
@@ -304,29 +314,155 @@ def secondary(src_w, dst_w, dev_tables, payload, L, bs, H, D, NB, dev):
         mapping = torch.stack([all_si[:P], free[:P]], 1).contiguous()
         med, mn = timed(lambda: kv_ops.copy_blocks(sp, mapping), 10)
         out["copy_blocks_GBps"] = round(2 * P * L * 2 * chunk / (med * 1e-3) / 1e9, 1)
-    # append (reshape_and_cache): 256 decode tokens + one 8192-token prefill chunk, 5% padded
-    T = 8448
+    out["append"] = append_bench(src_w.kv_cache, NB, bs, H, D, torch.bfloat16, None, None, dev)
+    return out
+
+
+def append_bench(kv, NB, bs, H, D, cache_dtype_name, k_scales, v_scales, dev, T=8448):
+    """reshape_and_cache for one step: 256 decode tokens + one 8192-token prefill chunk, slots random
+    over the pool, 5 % padded (-1). Three ways of issuing it: the vLLM-shaped call once per layer
+    (eager Python), the same L launches replayed from a HIP graph, and one launch for all layers from
+    a prepared plan. tokens/s = valid tokens / time of all layers."""
+    from elasticmm_amd import cache_ops
+
+    L = len(kv)
+    fp8 = kv[0].element_size() == 1
+    mode = "fp8" if fp8 else "auto"
     g = torch.Generator(device=dev).manual_seed(3)
     slots = torch.randperm(NB * bs, device=dev, generator=g)[:T].clone()
     slots[torch.rand(T, device=dev, generator=g) < 0.05] = -1
     valid = int((slots >= 0).sum())
     keys = [torch.randn((T, H, D), device=dev, generator=g).to(torch.bfloat16) for _ in range(L)]
     values = [torch.randn((T, H, D), device=dev, generator=g).to(torch.bfloat16) for _ in range(L)]
-    kv = src_w.kv_cache
-    row = H * D * 2
-    step_bytes = L * (valid * 2 * row * 2 + 8 * T)
+    row = H * D
+    step_bytes = L * (valid * 2 * row * (2 + kv[0].element_size()) + 8 * T)
+    ks = [None] * L if not fp8 else [k_scales[l:l + 1] for l in range(L)]
+    vs = [None] * L if not fp8 else [v_scales[l:l + 1] for l in range(L)]
 
     def per_layer():
         for l in range(L):
-            cache_ops.reshape_and_cache_flash(keys[l], values[l], kv[l][0], kv[l][1], slots, "auto")
+            cache_ops.reshape_and_cache_flash(keys[l], values[l], kv[l][0], kv[l][1], slots, mode, ks[l], vs[l])
 
-    med, mn = timed(per_layer, 20)
-    out["append_per_layer_launches"] = {"tokens_per_s": round(valid / (med * 1e-3)), "ms_per_step": round(med, 4),
-                                        "GBps": round(step_bytes / (med * 1e-3) / 1e9, 1)}
-    med, mn = timed(lambda: cache_ops.reshape_and_cache_flash_layers(keys, values, kv, slots, "auto"), 20)
-    out["append_one_launch"] = {"tokens_per_s": round(valid / (med * 1e-3)), "ms_per_step": round(med, 4),
-                                "GBps": round(step_bytes / (med * 1e-3) / 1e9, 1)}
-    out["append_tokens"] = {"T": T, "valid": valid, "layers": L}
+    def entry(ms):
+        return {"tokens_per_s": round(valid / (ms * 1e-3)), "ms_per_step": round(ms, 4),
+                "GBps": round(step_bytes / (ms * 1e-3) / 1e9, 1)}
+
+    res = {"T": T, "valid": valid, "layers": L, "algorithmic_bytes_per_step": step_bytes}
+    med, _ = timed(per_layer, 20)
+    res["per_layer_calls_eager"] = entry(med)
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        per_layer()
+    torch.cuda.current_stream().wait_stream(side)
+    with torch.cuda.graph(graph):
+        per_layer()
+    med, _ = timed(graph.replay, 20)
+    res["per_layer_calls_hip_graph"] = entry(med)
+    plan = cache_ops.layered_append(keys, values, kv, mode, k_scales, v_scales)
+    med, _ = timed(lambda: plan(slots), 20)
+    res["one_launch_all_layers"] = entry(med)
+    return res
+
+
+def extended(dev):
+    """The two other BASELINE shapes at full size (run with --extended; needs the whole GPU):
+    the fp8-e4m3 70B-class per-GPU shape and the elastic rebalancing of a ~200 GB pool."""
+    from elasticmm_amd import kv_ops
+    from elasticmm_amd.kv_ops import PoolView
+
+    out = {}
+    # ---- fp8: 80 layers x [2, NB, 16, 8, 128] e4m3, 64 requests of U{1024..8192} tokens
+    L, bs, H, D, NB = 80, 16, 8, 128, 20000
+    chunk = bs * H * D
+    g = torch.Generator().manual_seed(4)
+    lens = torch.randint(1024, 8193, (64,), generator=g)
+    nblk = [(int(t) + 15) // 16 for t in lens]
+    total = sum(nblk)
+    perm_s = torch.randperm(NB, generator=g)[:total].to(dev)
+    perm_d = torch.randperm(NB, generator=g)[:total].to(dev)
+    k_scales = (torch.rand(L, generator=g) * 0.09 + 0.01).to(dev)
+    v_scales = (torch.rand(L, generator=g) * 0.09 + 0.01).to(dev)
+    src = torch.empty((L, 2, NB, bs, H, D), dtype=torch.uint8, device=dev)
+    src.random_(0, 0x78)  # finite positive e4m3 bytes
+    dst = torch.zeros_like(src)
+    sp, dp = PoolView(src), PoolView(dst)
+    off, ts_pack, ts_unpack, payload = 0, 0.0, 0.0, 0
+    for n in nblk:  # per-request staging buffers (the whole batch would be 45 GiB)
+        si, di = perm_s[off:off + n], perm_d[off:off + n]
+        buf = torch.empty(sp.packed_shape(n), dtype=torch.uint8, device=dev)
+        med, _ = timed(lambda: kv_ops.kv_pack(sp, si, out=buf), 3, warmup=1)
+        ts_pack += med
+        med, _ = timed(lambda: kv_ops.kv_unpack(dp, di, buf), 3, warmup=1)
+        ts_unpack += med
+        payload += n * L * 2 * chunk
+        off += n
+        del buf
+    out["fp8_70b_shape"] = {"layers": L, "pool_blocks": NB, "requests": 64, "blocks": total,
+                            "payload_GB": round(payload / 1e9, 2),
+                            "pack_GBps": round(2 * payload / (ts_pack * 1e-3) / 1e9, 1),
+                            "unpack_GBps": round(2 * payload / (ts_unpack * 1e-3) / 1e9, 1)}
+    out["fp8_70b_shape"]["append"] = append_bench(list(src.unbind(0)), NB, bs, H, D, "fp8", k_scales, v_scales, dev)
+    del dst, dp
+    torch.cuda.empty_cache()
+    # dequantising unpack into a bf16 pool (first 16 requests)
+    dq = torch.zeros((L, 2, NB, bs, H, D), dtype=torch.bfloat16, device=dev)
+    dqp = PoolView(dq)
+    off, t_dq, pay = 0, 0.0, 0
+    for n in nblk[:16]:
+        buf = kv_ops.kv_pack(sp, perm_s[off:off + n])
+        di = perm_d[off:off + n]
+        med, _ = timed(lambda: kv_ops.kv_unpack_dequant_fp8(dqp, di, buf, k_scales, v_scales), 3, warmup=1)
+        t_dq += med
+        pay += n * L * 2 * chunk
+        off += n
+        del buf
+    out["fp8_70b_shape"]["dequant_unpack_GBps"] = round(3 * pay / (t_dq * 1e-3) / 1e9, 1)
+    del src, sp, dq, dqp
+    torch.cuda.empty_cache()
+
+    # ---- rebalancing: ~200 GB bf16 pool in the Qwen2-7B layout, move 50 % of the live half
+    L, bs, H, D = 28, 16, 4, 128
+    chunk = bs * H * D * 2
+    NB = 218000
+    pool = torch.empty((L, 2, NB, bs, H, D), dtype=torch.bfloat16, device=dev)
+    for l in range(L):
+        pool[l].normal_(0.0, 0.5)
+    pv = PoolView(pool)
+    g = torch.Generator().manual_seed(5)
+    perm = torch.randperm(NB, generator=g)
+    live = perm[:NB // 2]
+    free = perm[NB // 2:]
+    P = live.numel() // 2
+    mapping = torch.stack([live[:P], free[:P]], 1).contiguous().to(dev)
+    med, mn = timed(lambda: kv_ops.copy_blocks(pv, mapping), 5, warmup=1)
+    ok = bool(torch.equal(pool[3][:, mapping[:1000, 1]], pool[3][:, mapping[:1000, 0]]))
+    out["rebalance_200GB"] = {"pool_GB": round(pool.numel() * 2 / 1e9, 1), "pairs": P,
+                              "algorithmic_GB": round(2 * P * L * 2 * chunk / 1e9, 1), "ms": round(med, 3),
+                              "copy_blocks_GBps": round(2 * P * L * 2 * chunk / (med * 1e-3) / 1e9, 1),
+                              "spot_check": ok}
+    # vision-embedding gather interleaved on the same stream
+    imgs = torch.randint(64, 2305, (128,), generator=g).tolist()
+    embeds = [torch.randn((p_, 3584), device=dev).to(torch.bfloat16) for p_ in imgs]
+    vis_bytes = 2 * sum(imgs) * 3584 * 2
+    outbuf = torch.empty((sum(imgs), 3584), dtype=torch.bfloat16, device=dev)
+    med, _ = timed(lambda: kv_ops.concat_rows(embeds, out=outbuf), 10)
+    out["rebalance_200GB"]["vision_concat"] = {"images": 128, "rows": sum(imgs), "ms": round(med, 4),
+                                               "GBps": round(vis_bytes / (med * 1e-3) / 1e9, 1)}
+    med_t, _ = timed(lambda: torch.cat(embeds, 0, out=outbuf), 10)
+    out["rebalance_200GB"]["vision_concat"]["torch_cat_GBps"] = round(vis_bytes / (med_t * 1e-3) / 1e9, 1)
+    quarter = mapping[:P // 8]
+
+    def interleaved():
+        for k in range(8):
+            kv_ops.copy_blocks(pv, mapping[k * (P // 8):(k + 1) * (P // 8)])
+            kv_ops.concat_rows(embeds[k * 16:(k + 1) * 16], out=outbuf[:sum(imgs[k * 16:(k + 1) * 16])])
+
+    med, _ = timed(interleaved, 3, warmup=1)
+    tot = 2 * (P // 8) * 8 * L * 2 * chunk + vis_bytes
+    out["rebalance_200GB"]["interleaved_copy_and_concat_GBps"] = round(tot / (med * 1e-3) / 1e9, 1)
+    del quarter
     return out
 
 

@@ -50,6 +50,19 @@ def reshape_and_cache_flash_layers(keys: Sequence[torch.Tensor], values: Sequenc
         raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
 
 
+def layered_append(keys: Sequence[torch.Tensor], values: Sequence[torch.Tensor], kv_caches: Sequence[torch.Tensor],
+                   kv_cache_dtype: str = "auto", k_scales=None, v_scales=None) -> kv_ops.LayeredAppend:
+    """A prepared whole-step append over fixed key / value staging tensors: validate once,
+    then ``plan(slot_mapping)`` is one C call (and can be captured in a HIP graph)."""
+    key_caches = [c[0] for c in kv_caches]
+    value_caches = [c[1] for c in kv_caches]
+    if kv_cache_dtype == "auto":
+        return kv_ops.LayeredAppend(keys, values, key_caches, value_caches)
+    if kv_cache_dtype in ("fp8", "fp8_e4m3"):
+        return kv_ops.LayeredAppend(keys, values, key_caches, value_caches, k_scales, v_scales)
+    raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
+
+
 def copy_blocks(kv_caches: List[torch.Tensor], block_mapping: torch.Tensor) -> None:
     """``kv_caches``: list of ``[2, num_blocks, block_size, H, D]``; ``block_mapping``: int64
     ``[num_pairs, 2]`` of (src, dst). One launch covers every layer, K and V."""

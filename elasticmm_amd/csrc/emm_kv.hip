@@ -405,9 +405,29 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
   return (float)x;
 }
 
-// fp32 -> e4m3fn, round to nearest even, no saturation: magnitudes that round
-// past 448 (>= 465 after RNE, i.e. bits >= 480.0 or the [464, 480) interval
-// rounding up), inf and NaN give sign|0x7F.
+// fp32 -> e4m3fn with the rule of torch's cast: round to nearest even, no
+// saturation; what rounds past 448 (464 is the tie that still gives 448), +-inf
+// and NaN give sign|0x7F. gfx950's v_cvt_pk_fp8_f32 (OCP e4m3, overflow mode off)
+// implements exactly this for every non-NaN fp32 input — checked against the
+// integer formulation below over all 2^32 bit patterns on the device — and
+// returns 0xFF for every NaN, so NaN inputs are first replaced by the infinity of
+// their sign.
+__device__ __forceinline__ float nan_to_signed_inf(float f) {
+  const uint32_t u = __float_as_uint(f);
+  uint32_t a = u & 0x7fffffffu;
+  a = a < 0x7f800000u ? a : 0x7f800000u;
+  return __uint_as_float(a | (u & 0x80000000u));
+}
+
+// four fp32 -> four e4m3fn bytes in one dword (byte k = value k)
+__device__ __forceinline__ uint32_t f32x4_to_e4m3fn(float q0, float q1, float q2, float q3) {
+  int r = 0;
+  r = __builtin_amdgcn_cvt_pk_fp8_f32(nan_to_signed_inf(q0), nan_to_signed_inf(q1), r, false);
+  r = __builtin_amdgcn_cvt_pk_fp8_f32(nan_to_signed_inf(q2), nan_to_signed_inf(q3), r, true);
+  return (uint32_t)r;
+}
+
+// The same rule in integer arithmetic, one value at a time (element-wise path).
 __device__ __forceinline__ uint32_t f32_to_e4m3fn(float f) {
   const uint32_t u = __float_as_uint(f);
   const uint32_t sign = (u >> 24) & 0x80u;
@@ -425,22 +445,6 @@ __device__ __forceinline__ uint32_t f32_to_e4m3fn(float f) {
     r = a >> 20;            // may carry into 0x7f (NaN) for [464, 480)
   }
   return r | sign;
-}
-
-// e4m3fn byte -> fp32 (exact). NaN bytes give a quiet NaN with the byte's sign.
-__device__ __forceinline__ float e4m3fn_to_f32(uint32_t b) {
-  const uint32_t sign = (b & 0x80u) << 24;
-  const uint32_t e = (b >> 3) & 0xfu;
-  const uint32_t m = b & 7u;
-  uint32_t bits;
-  if (e == 0) {
-    bits = __float_as_uint((float)m * 0.001953125f); // m * 2^-9, exact
-  } else if (e == 15 && m == 7) {
-    bits = 0x7fc00000u;
-  } else {
-    bits = ((e + 120u) << 23) | (m << 20);
-  }
-  return __uint_as_float(bits | sign);
 }
 
 // fp32 -> bf16 bits, round to nearest even; NaN -> 0x7FC0.
@@ -479,41 +483,38 @@ __device__ __forceinline__ u32x2 quant8(u32x4 in, float scale) {
   u32x2 out;
 #pragma unroll
   for (int w = 0; w < 2; ++w) {
-    uint32_t acc = 0;
-#pragma unroll
-    for (int k = 0; k < 2; ++k) {
-      const uint32_t word = in[w * 2 + k];
-      const float lo = half_bits_to_f32<SRC_DTYPE>(word & 0xffffu) / scale;
-      const float hi = half_bits_to_f32<SRC_DTYPE>(word >> 16) / scale;
-      acc |= (f32_to_e4m3fn(lo) | (f32_to_e4m3fn(hi) << 8)) << (16 * k);
-    }
-    out[w] = acc;
+    const uint32_t w0 = in[w * 2], w1 = in[w * 2 + 1];
+    out[w] = f32x4_to_e4m3fn(half_bits_to_f32<SRC_DTYPE>(w0 & 0xffffu) / scale,
+                             half_bits_to_f32<SRC_DTYPE>(w0 >> 16) / scale,
+                             half_bits_to_f32<SRC_DTYPE>(w1 & 0xffffu) / scale,
+                             half_bits_to_f32<SRC_DTYPE>(w1 >> 16) / scale);
   }
   return out;
 }
 
-// 16 e4m3fn bytes (one u32x4) -> 16 sixteen-bit values (two u32x4)
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+// 16 e4m3fn bytes (one u32x4) -> 16 sixteen-bit values (two u32x4). The byte ->
+// fp32 step is v_cvt_pk_f32_fp8 (exact; its NaN carries the wrong sign, which the
+// 16-bit rounding below replaces by the canonical quiet NaN anyway).
 template <int OUT_DTYPE>
 __device__ __forceinline__ void dequant16(u32x4 in, float scale, u32x4 &o0, u32x4 &o1) {
   uint32_t o[8];
 #pragma unroll
   for (int w = 0; w < 4; ++w) {
+    const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)in[w], false); // bytes 0, 1
+    const f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)in[w], true);  // bytes 2, 3
+    const float f[4] = {lo[0] * scale, lo[1] * scale, hi[0] * scale, hi[1] * scale};
+    uint32_t h[4];
 #pragma unroll
-    for (int k = 0; k < 2; ++k) {
-      const uint32_t b0 = (in[w] >> (16 * k)) & 0xffu;
-      const uint32_t b1 = (in[w] >> (16 * k + 8)) & 0xffu;
-      const float f0 = e4m3fn_to_f32(b0) * scale;
-      const float f1 = e4m3fn_to_f32(b1) * scale;
-      uint32_t h0, h1;
-      if constexpr (OUT_DTYPE == EMM_DTYPE_BF16) {
-        h0 = f32_to_bf16_bits(f0);
-        h1 = f32_to_bf16_bits(f1);
-      } else {
-        h0 = f32_to_f16_bits(f0);
-        h1 = f32_to_f16_bits(f1);
-      }
-      o[w * 2 + k] = h0 | (h1 << 16);
+    for (int k = 0; k < 4; ++k) {
+      if constexpr (OUT_DTYPE == EMM_DTYPE_BF16)
+        h[k] = f32_to_bf16_bits(f[k]);
+      else
+        h[k] = f32_to_f16_bits(f[k]);
     }
+    o[w * 2] = h[0] | (h[1] << 16);
+    o[w * 2 + 1] = h[2] | (h[3] << 16);
   }
   o0 = u32x4{o[0], o[1], o[2], o[3]};
   o1 = u32x4{o[4], o[5], o[6], o[7]};
@@ -590,101 +591,149 @@ struct AppendParams {
   int64_t num_slots;
 };
 
-constexpr int kRowsPerWave = 4;
 constexpr int kWavesPerGroup = kThreads / 64;
 
-// One wave moves kRowsPerWave token rows of K or V. grid: x = token groups,
-// y = 2 (K, V), z = layers.
-template <typename V, bool NT>
+// Rows per wave of the append kernels: 0 = default. Set through the tuning hook.
+int g_append_rows = 0;
+
+// Fetch the slots of R consecutive tokens. The loads are only issued here (one
+// address for all lanes); resolve_slots() waits for them, moves the values to
+// scalar registers and turns padding (< 0) and out-of-range slots into -1.
+template <int R>
+__device__ __forceinline__ void fetch_slots(int64_t (&s)[R], const int64_t *slot_mapping, int64_t t0,
+                                            int64_t num_tokens) {
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t t = t0 + r;
+    s[r] = -1;
+    if (t < num_tokens) s[r] = ld<int64_t, false>((const char *)(slot_mapping + t));
+  }
+}
+
+template <int R>
+__device__ __forceinline__ void resolve_slots(int64_t (&s)[R], int64_t num_slots) {
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    s[r] = uniform64(s[r]);
+    if ((uint64_t)s[r] >= (uint64_t)num_slots) s[r] = -1;
+  }
+}
+
+// One wave moves R token rows of K or V: grid x = groups of 4 * R tokens,
+// y = 2 (K, V), z = layers. The source rows do not depend on the slots, so their
+// first loads are issued before the slots are waited for (rows of padded tokens
+// are read and dropped).
+template <typename V, int R, int POLICY>
 __global__ __launch_bounds__(kThreads) void emm_append_kernel(const AppendParams p) {
   constexpr int64_t VB = sizeof(V);
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const uint32_t kv = blockIdx.y, l = blockIdx.z;
-  const int64_t t0 = ((int64_t)blockIdx.x * kWavesPerGroup + wave) * kRowsPerWave;
+  const int64_t t0 = ((int64_t)blockIdx.x * kWavesPerGroup + wave) * R;
+  if (t0 >= p.num_tokens) return;
   const char *src_base = kv == 0 ? p.key[l] : p.value[l];
   char *dst_base = kv == 0 ? p.key_cache[l] : p.value_cache[l];
   const int64_t stride = kv == 0 ? p.key_stride : p.value_stride;
+  const int64_t row_bytes = p.row_bytes;
 
-  int64_t slot[kRowsPerWave];
+  int64_t slot[R];
+  fetch_slots<R>(slot, p.slot_mapping, t0, p.num_tokens);
+  int64_t off = (int64_t)lane * VB;
+  V v[R];
 #pragma unroll
-  for (int r = 0; r < kRowsPerWave; ++r) {
-    const int64_t t = t0 + r;
-    int64_t s = -1;
-    if (t < p.num_tokens) s = p.slot_mapping[t];
-    // wave-uniform: keep the slot and everything derived from it scalar
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)s);
-    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)s >> 32));
-    s = (int64_t)(((uint64_t)hi << 32) | lo);
-    if ((uint64_t)s >= (uint64_t)p.num_slots) s = -1;
-    slot[r] = s;
-  }
-  for (int64_t off = (int64_t)lane * VB; off < p.row_bytes; off += 64 * VB) {
-    V v[kRowsPerWave];
+  for (int r = 0; r < R; ++r)
+    if (t0 + r < p.num_tokens && off < row_bytes)
+      v[r] = ld_stream<V, POLICY>(src_base + (t0 + r) * stride + off);
+  resolve_slots<R>(slot, p.num_slots);
 #pragma unroll
-    for (int r = 0; r < kRowsPerWave; ++r)
-      if (slot[r] >= 0) v[r] = ld<V, NT>(src_base + (t0 + r) * stride + off);
+  for (int r = 0; r < R; ++r)
+    if (slot[r] >= 0 && off < row_bytes) st_stream<V, POLICY>(dst_base + slot[r] * row_bytes + off, v[r]);
+  for (off += 64 * VB; off < row_bytes; off += 64 * VB) {
 #pragma unroll
-    for (int r = 0; r < kRowsPerWave; ++r)
-      if (slot[r] >= 0) st<V, NT>(dst_base + slot[r] * p.row_bytes + off, v[r]);
+    for (int r = 0; r < R; ++r)
+      if (slot[r] >= 0) v[r] = ld_stream<V, POLICY>(src_base + (t0 + r) * stride + off);
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (slot[r] >= 0) st_stream<V, POLICY>(dst_base + slot[r] * row_bytes + off, v[r]);
   }
 }
 
-// fp8 append: each lane converts 8 contiguous 16-bit elements (16 B) into
-// 8 fp8 bytes (8 B) per step; a wave covers 512 elements per step.
-template <int SRC_DTYPE, int VEC_ELEMS>
+// fp8 append. VEC_ELEMS = 16: each lane converts 16 contiguous 16-bit elements
+// (two 16-byte loads) into one 16-byte store, a wave covers 1024 elements per
+// step; VEC_ELEMS = 8: 16 bytes in, 8 bytes out; VEC_ELEMS = 1: element-wise
+// path for odd row sizes or misaligned bases.
+template <int SRC_DTYPE, int VEC_ELEMS, int R>
 __global__ __launch_bounds__(kThreads) void emm_append_fp8_kernel(const AppendParams p) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const uint32_t kv = blockIdx.y, l = blockIdx.z;
-  const int64_t t0 = ((int64_t)blockIdx.x * kWavesPerGroup + wave) * kRowsPerWave;
+  const int64_t t0 = ((int64_t)blockIdx.x * kWavesPerGroup + wave) * R;
+  if (t0 >= p.num_tokens) return;
   const char *src_base = kv == 0 ? p.key[l] : p.value[l];
   char *dst_base = kv == 0 ? p.key_cache[l] : p.value_cache[l];
   const int64_t stride = kv == 0 ? p.key_stride : p.value_stride;
   const float scale = kv == 0 ? p.k_scales[l] : p.v_scales[l];
   const int64_t row = p.row_bytes; // elements
 
-  int64_t slot[kRowsPerWave];
+  int64_t slot[R];
+  fetch_slots<R>(slot, p.slot_mapping, t0, p.num_tokens);
+  if constexpr (VEC_ELEMS == 16) {
+    int64_t e = (int64_t)lane * 16;
+    u32x4 a[R], b[R];
 #pragma unroll
-  for (int r = 0; r < kRowsPerWave; ++r) {
-    const int64_t t = t0 + r;
-    int64_t s = -1;
-    if (t < p.num_tokens) s = p.slot_mapping[t];
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)s);
-    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)s >> 32));
-    s = (int64_t)(((uint64_t)hi << 32) | lo);
-    if ((uint64_t)s >= (uint64_t)p.num_slots) s = -1;
-    slot[r] = s;
-  }
-  if constexpr (VEC_ELEMS == 8) {
+    for (int r = 0; r < R; ++r)
+      if (t0 + r < p.num_tokens && e < row) {
+        const char *sp = src_base + ((t0 + r) * stride + e) * 2;
+        a[r] = ld<u32x4, true>(sp);
+        b[r] = ld<u32x4, true>(sp + 16);
+      }
+    resolve_slots<R>(slot, p.num_slots);
+    while (e < row) {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if (slot[r] >= 0) {
+          const u32x2 lo = quant8<SRC_DTYPE>(a[r], scale), hi = quant8<SRC_DTYPE>(b[r], scale);
+          st_stream<u32x4, 1>(dst_base + slot[r] * row + e, u32x4{lo[0], lo[1], hi[0], hi[1]});
+        }
+      e += 64 * 16;
+      if (e < row) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+          if (slot[r] >= 0) {
+            const char *sp = src_base + ((t0 + r) * stride + e) * 2;
+            a[r] = ld<u32x4, true>(sp);
+            b[r] = ld<u32x4, true>(sp + 16);
+          }
+      }
+    }
+  } else if constexpr (VEC_ELEMS == 8) {
+    resolve_slots<R>(slot, p.num_slots);
     for (int64_t e = (int64_t)lane * 8; e < row; e += 64 * 8) {
-      u32x4 v[kRowsPerWave];
+      u32x4 v[R];
 #pragma unroll
-      for (int r = 0; r < kRowsPerWave; ++r)
+      for (int r = 0; r < R; ++r)
         if (slot[r] >= 0) v[r] = ld<u32x4, true>(src_base + ((t0 + r) * stride + e) * 2);
 #pragma unroll
-      for (int r = 0; r < kRowsPerWave; ++r)
-        if (slot[r] >= 0)
-          st<u32x2, true>(dst_base + slot[r] * row + e, quant8<SRC_DTYPE>(v[r], scale));
+      for (int r = 0; r < R; ++r)
+        if (slot[r] >= 0) st<u32x2, true>(dst_base + slot[r] * row + e, quant8<SRC_DTYPE>(v[r], scale));
     }
   } else {
-    // element-wise path for rows that are not a multiple of 8 elements or
-    // misaligned bases
+    resolve_slots<R>(slot, p.num_slots);
     for (int64_t e = lane; e < row; e += 64) {
 #pragma unroll
-      for (int r = 0; r < kRowsPerWave; ++r) {
+      for (int r = 0; r < R; ++r) {
         if (slot[r] >= 0) {
-          const uint16_t h = *reinterpret_cast<const uint16_t *>(src_base + ((t0 + r) * stride + e) * 2);
+          const uint16_t h = ld<uint16_t, false>(src_base + ((t0 + r) * stride + e) * 2);
           const float x = half_bits_to_f32<SRC_DTYPE>(h) / scale;
-          *reinterpret_cast<uint8_t *>(dst_base + slot[r] * row + e) = (uint8_t)f32_to_e4m3fn(x);
+          st<uint8_t, false>(dst_base + slot[r] * row + e, (uint8_t)f32_to_e4m3fn(x));
         }
       }
     }
   }
 }
 
-dim3 append_grid(int64_t num_tokens, int num_layers) {
-  const int64_t rows_per_group = (int64_t)kWavesPerGroup * kRowsPerWave;
+dim3 append_grid(int64_t num_tokens, int num_layers, int rows_per_wave) {
+  const int64_t rows_per_group = (int64_t)kWavesPerGroup * rows_per_wave;
   return dim3((uint32_t)((num_tokens + rows_per_group - 1) / rows_per_group), 2, (uint32_t)num_layers);
 }
 
@@ -737,13 +786,21 @@ int append_copy(const void *const *k, const void *const *v, void *const *kc, voi
   p.num_slots = num_slots;
   int vec = al;
   while (vec > 1 && (row_bytes % vec || ks % vec || vs % vec)) vec >>= 1;
-  dim3 grid = append_grid(num_tokens, num_layers);
-  switch (vec) {
-  case 16: emm_append_kernel<u32x4, true><<<grid, kThreads, 0, s>>>(p); break;
-  case 8: emm_append_kernel<u32x2, true><<<grid, kThreads, 0, s>>>(p); break;
-  case 4: emm_append_kernel<uint32_t, true><<<grid, kThreads, 0, s>>>(p); break;
-  case 2: emm_append_kernel<uint16_t, true><<<grid, kThreads, 0, s>>>(p); break;
-  default: emm_append_kernel<uint8_t, true><<<grid, kThreads, 0, s>>>(p); break;
+  const int rows = (g_append_rows == 1 || g_append_rows == 2 || g_append_rows == 4) ? g_append_rows : 1;
+  dim3 grid = append_grid(num_tokens, num_layers, vec == 16 ? rows : 4);
+  if (vec == 16) {
+    switch (rows) {
+    case 4: emm_append_kernel<u32x4, 4, 1><<<grid, kThreads, 0, s>>>(p); break;
+    case 2: emm_append_kernel<u32x4, 2, 1><<<grid, kThreads, 0, s>>>(p); break;
+    default: emm_append_kernel<u32x4, 1, 1><<<grid, kThreads, 0, s>>>(p); break;
+    }
+  } else {
+    switch (vec) {
+    case 8: emm_append_kernel<u32x2, 4, 0><<<grid, kThreads, 0, s>>>(p); break;
+    case 4: emm_append_kernel<uint32_t, 4, 0><<<grid, kThreads, 0, s>>>(p); break;
+    case 2: emm_append_kernel<uint16_t, 4, 0><<<grid, kThreads, 0, s>>>(p); break;
+    default: emm_append_kernel<uint8_t, 4, 0><<<grid, kThreads, 0, s>>>(p); break;
+    }
   }
   return check_launch(what);
 }
@@ -762,15 +819,18 @@ int append_fp8(const void *const *k, const void *const *v, void *const *kc, void
   if (!k_scales || !v_scales) return fail(EMM_EINVAL, "%s: scale pointer is null", what);
   AppendParams p;
   memset(&p, 0, sizeof(p));
-  bool wide = (row_elems % 8 == 0) && (ks % 8 == 0) && (vs % 8 == 0);
+  int width = 16;
+  if (row_elems % 16 || ks % 8 || vs % 8) width = (row_elems % 8 || ks % 8 || vs % 8) ? 1 : 8;
   for (int l = 0; l < num_layers; ++l) {
     p.key[l] = (const char *)k[l];
     p.value[l] = (const char *)v[l];
     p.key_cache[l] = (char *)kc[l];
     p.value_cache[l] = (char *)vc[l];
-    wide = wide && aligned(k[l], 16) && aligned(v[l], 16) && aligned(kc[l], 8) && aligned(vc[l], 8);
     if (!aligned(k[l], 2) || !aligned(v[l], 2))
       return fail(EMM_EINVAL, "%s: 16-bit source not 2-byte aligned at layer %d", what, l);
+    if (!aligned(k[l], 16) || !aligned(v[l], 16)) width = 1;
+    if (width == 16 && (!aligned(kc[l], 16) || !aligned(vc[l], 16))) width = 8;
+    if (width == 8 && (!aligned(kc[l], 8) || !aligned(vc[l], 8))) width = 1;
   }
   p.slot_mapping = slot_mapping;
   p.k_scales = k_scales;
@@ -780,14 +840,20 @@ int append_fp8(const void *const *k, const void *const *v, void *const *kc, void
   p.key_stride = ks;
   p.value_stride = vs;
   p.num_slots = num_slots;
-  dim3 grid = append_grid(num_tokens, num_layers);
-  if (src_dtype == EMM_DTYPE_BF16) {
-    if (wide) emm_append_fp8_kernel<EMM_DTYPE_BF16, 8><<<grid, kThreads, 0, s>>>(p);
-    else emm_append_fp8_kernel<EMM_DTYPE_BF16, 1><<<grid, kThreads, 0, s>>>(p);
-  } else {
-    if (wide) emm_append_fp8_kernel<EMM_DTYPE_F16, 8><<<grid, kThreads, 0, s>>>(p);
-    else emm_append_fp8_kernel<EMM_DTYPE_F16, 1><<<grid, kThreads, 0, s>>>(p);
-  }
+  // rows per wave: the conversion is arithmetic-heavy, two rows per wave keep more loads in
+  // flight per lane in a large launch; a small launch needs the extra workgroups of one row
+  int rows = (num_tokens * num_layers >= 100000) ? 2 : 1;
+  if (g_append_rows == 1 || g_append_rows == 2 || g_append_rows == 4) rows = g_append_rows;
+  dim3 grid = append_grid(num_tokens, num_layers, width == 16 ? rows : 4);
+#define EMM_FP8_LAUNCH(DT)                                                                  \
+  if (width == 16) {                                                                        \
+    if (rows == 4) emm_append_fp8_kernel<DT, 16, 4><<<grid, kThreads, 0, s>>>(p);           \
+    else if (rows == 2) emm_append_fp8_kernel<DT, 16, 2><<<grid, kThreads, 0, s>>>(p);      \
+    else emm_append_fp8_kernel<DT, 16, 1><<<grid, kThreads, 0, s>>>(p);                     \
+  } else if (width == 8) emm_append_fp8_kernel<DT, 8, 4><<<grid, kThreads, 0, s>>>(p);      \
+  else emm_append_fp8_kernel<DT, 1, 4><<<grid, kThreads, 0, s>>>(p);
+  if (src_dtype == EMM_DTYPE_BF16) { EMM_FP8_LAUNCH(EMM_DTYPE_BF16) } else { EMM_FP8_LAUNCH(EMM_DTYPE_F16) }
+#undef EMM_FP8_LAUNCH
   return check_launch(what);
 }
 
@@ -830,8 +896,9 @@ const char *emm_last_error(void) { return g_last_error; }
 int emm_abi_version(void) { return EMM_KV_ABI_VERSION; }
 
 int emm_set_move_variant(int variant) {
-  const int old = g_move_variant;
-  g_move_variant = variant;
+  const int old = g_move_variant | (g_append_rows << 12);
+  g_move_variant = variant & 0xfff;
+  g_append_rows = (variant >> 12) & 0xf; // rows per wave of the append kernels
   return old;
 }
 

@@ -17,7 +17,13 @@ from ._lib import EMM_DTYPE_BF16, EMM_DTYPE_F16, EMM_MAX_LAYERS, EMM_MAX_SEGMENT
 IndexLike = Union[Sequence[int], np.ndarray, torch.Tensor]
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream_ptr(device: torch.device) -> int:
+    """hipStream_t of torch's current stream on `device`, as an integer."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
     return torch.cuda.current_stream(device).cuda_stream
 
 
@@ -231,14 +237,23 @@ def kv_unpack_dequant_fp8(pool: PoolView, block_indices: IndexLike, packed_fp8: 
 
 def _row_geometry(x: torch.Tensor, what: str):
     """(num_tokens, row_elems, token_stride_elems) of a [T, ...] tensor whose rows are contiguous."""
-    if x.dim() < 1:
+    nd = x.dim()
+    if nd < 1:
         raise ValueError(f"{what}: expected [num_tokens, ...]")
-    T = int(x.shape[0])
-    row = int(np.prod(x.shape[1:], dtype=np.int64)) if x.dim() > 1 else 1
-    if T > 0 and x.dim() > 1 and not x[0].is_contiguous():
-        raise ValueError(f"{what}: rows must be contiguous (only the token dimension may be strided)")
-    stride = int(x.stride(0)) if T > 1 else row
-    return T, row, stride
+    T = x.shape[0]
+    if nd == 1:
+        return T, 1, (x.stride(0) if T > 1 else 1)
+    row = 1
+    for d in x.shape[1:]:
+        row *= d
+    if T > 0:
+        # rows must be dense: walk the trailing dimensions from the innermost outwards
+        expect = 1
+        for d in range(nd - 1, 0, -1):
+            if x.shape[d] != 1 and x.stride(d) != expect:
+                raise ValueError(f"{what}: rows must be contiguous (only the token dimension may be strided)")
+            expect *= x.shape[d]
+    return T, row, (x.stride(0) if T > 1 else row)
 
 
 def _cache_slots(cache: torch.Tensor, row_elems: int, what: str) -> int:
@@ -246,9 +261,10 @@ def _cache_slots(cache: torch.Tensor, row_elems: int, what: str) -> int:
         raise ValueError(f"{what}: cache plane must be contiguous")
     if row_elems == 0:
         return 0
-    if cache.numel() % row_elems:
+    n = cache.numel()
+    if n % row_elems:
         raise ValueError(f"{what}: cache size is not a multiple of the token row")
-    return cache.numel() // row_elems
+    return n // row_elems
 
 
 def reshape_and_cache(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
@@ -259,29 +275,29 @@ def reshape_and_cache(key: torch.Tensor, value: torch.Tensor, key_cache: torch.T
     Same-width caches are copied bit for bit; a 1-byte cache with a 16-bit source
     is quantised to fp8-e4m3fn with ``k_scale`` / ``v_scale`` (one float each)."""
     lib = _lib.load()
-    for t, nm in ((key, "key"), (value, "value"), (key_cache, "key_cache"), (value_cache, "value_cache"),
-                  (slot_mapping, "slot_mapping")):
-        _require_gpu(t, f"reshape_and_cache({nm})")
+    if not (key.is_cuda and value.is_cuda and key_cache.is_cuda and value_cache.is_cuda and slot_mapping.is_cuda):
+        raise RuntimeError("reshape_and_cache: every tensor must be on the GPU; the KV kernels run on the GPU only")
     if slot_mapping.dtype != torch.long:
         raise TypeError("slot_mapping must be int64")
-    slot_mapping = slot_mapping.contiguous()
+    if not slot_mapping.is_contiguous():
+        slot_mapping = slot_mapping.contiguous()
     T, row, ks = _row_geometry(key, "key")
     Tv, rowv, vs = _row_geometry(value, "value")
-    if (T, row) != (Tv, rowv):
+    if T != Tv or row != rowv:
         raise ValueError("key and value differ in shape")
     if slot_mapping.numel() < T:
         raise ValueError("slot_mapping is shorter than the token count")
-    T = min(T, slot_mapping.numel())
     num_slots = _cache_slots(key_cache, row, "key_cache")
     if _cache_slots(value_cache, row, "value_cache") != num_slots:
         raise ValueError("key_cache and value_cache differ in size")
     stream = _stream_ptr(key.device)
     eb = key.element_size()
-    if key_cache.element_size() == eb:
+    ceb = key_cache.element_size()
+    if ceb == eb:
         check(lib.emm_reshape_and_cache(key.data_ptr(), value.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(),
                                         slot_mapping.data_ptr(), T, row * eb, ks * eb, vs * eb, num_slots, stream),
               "emm_reshape_and_cache")
-    elif key_cache.element_size() == 1 and eb == 2:
+    elif ceb == 1 and eb == 2:
         if k_scale is None or v_scale is None:
             raise ValueError("fp8 cache needs k_scale and v_scale")
         code = _half_code(key.dtype, "reshape_and_cache")
@@ -292,61 +308,91 @@ def reshape_and_cache(key: torch.Tensor, value: torch.Tensor, key_cache: torch.T
                                             num_slots, k_s.data_ptr(), v_s.data_ptr(), code, stream),
               "emm_reshape_and_cache_fp8")
     else:
-        raise TypeError(f"unsupported source/cache element sizes {eb}/{key_cache.element_size()}")
+        raise TypeError(f"unsupported source/cache element sizes {eb}/{ceb}")
+
+
+class LayeredAppend:
+    """All layers of one step appended with a single launch (per group of EMM_MAX_LAYERS).
+
+    The per-layer tensors are validated and their pointer tables built once; calling the
+    object with a ``slot_mapping`` then costs one C call. The tensors are kept alive by the
+    object, which suits a serving loop that reuses its key / value staging buffers (or
+    replays a captured HIP graph)."""
+
+    def __init__(self, keys: Sequence[torch.Tensor], values: Sequence[torch.Tensor],
+                 key_caches: Sequence[torch.Tensor], value_caches: Sequence[torch.Tensor],
+                 k_scales=None, v_scales=None):
+        self.lib = _lib.load()
+        L = len(keys)
+        if not (len(values) == len(key_caches) == len(value_caches) == L):
+            raise ValueError("per-layer lists differ in length")
+        self.num_layers = L
+        self._keep = (list(keys), list(values), list(key_caches), list(value_caches))
+        if L == 0:
+            return
+        for t in (*keys, *values, *key_caches, *value_caches):
+            _require_gpu(t, "LayeredAppend")
+        T, row, ks = _row_geometry(keys[0], "key")
+        _, _, vs = _row_geometry(values[0], "value")
+        for l in range(L):
+            if _row_geometry(keys[l], "key") != (T, row, ks) or _row_geometry(values[l], "value") != (T, row, vs):
+                raise ValueError(f"layer {l}: key/value geometry differs from layer 0")
+        num_slots = _cache_slots(key_caches[0], row, "key_cache")
+        for l in range(L):
+            if _cache_slots(key_caches[l], row, "key_cache") != num_slots or \
+                    _cache_slots(value_caches[l], row, "value_cache") != num_slots:
+                raise ValueError(f"layer {l}: cache size differs from layer 0")
+        self.device = keys[0].device
+        self.T, self.row, self.ks, self.vs, self.num_slots = T, row, ks, vs, num_slots
+        eb = keys[0].element_size()
+        ceb = key_caches[0].element_size()
+        self.fp8 = ceb == 1 and eb == 2
+        if not self.fp8 and ceb != eb:
+            raise TypeError(f"unsupported source/cache element sizes {eb}/{ceb}")
+        self.eb = eb
+        if self.fp8:
+            if k_scales is None or v_scales is None:
+                raise ValueError("fp8 cache needs k_scales and v_scales")
+            self.code = _half_code(keys[0].dtype, "LayeredAppend")
+            self.k_s = _scales_tensor(k_scales, L, self.device)
+            self.v_s = _scales_tensor(v_scales, L, self.device)
+        self.groups = []
+        for l0 in range(0, L, EMM_MAX_LAYERS):
+            sl = slice(l0, l0 + EMM_MAX_LAYERS)
+            self.groups.append((l0, ptr_table([t.data_ptr() for t in keys[sl]]),
+                                ptr_table([t.data_ptr() for t in values[sl]]),
+                                ptr_table([t.data_ptr() for t in key_caches[sl]]),
+                                ptr_table([t.data_ptr() for t in value_caches[sl]])))
+
+    def __call__(self, slot_mapping: torch.Tensor) -> None:
+        if self.num_layers == 0:
+            return
+        if slot_mapping.dtype != torch.long or not slot_mapping.is_cuda:
+            raise TypeError("slot_mapping must be an int64 GPU tensor")
+        if not slot_mapping.is_contiguous():
+            slot_mapping = slot_mapping.contiguous()
+        if slot_mapping.numel() < self.T:
+            raise ValueError("slot_mapping is shorter than the token count")
+        stream = _stream_ptr(self.device)
+        lib = self.lib
+        for l0, kt, vt, kct, vct in self.groups:
+            if self.fp8:
+                check(lib.emm_reshape_and_cache_fp8_layers(kt, vt, kct, vct, len(kt), slot_mapping.data_ptr(), self.T,
+                                                           self.row, self.ks, self.vs, self.num_slots,
+                                                           self.k_s.data_ptr() + 4 * l0, self.v_s.data_ptr() + 4 * l0,
+                                                           self.code, stream), "emm_reshape_and_cache_fp8_layers")
+            else:
+                eb = self.eb
+                check(lib.emm_reshape_and_cache_layers(kt, vt, kct, vct, len(kt), slot_mapping.data_ptr(), self.T,
+                                                       self.row * eb, self.ks * eb, self.vs * eb, self.num_slots,
+                                                       stream), "emm_reshape_and_cache_layers")
 
 
 def reshape_and_cache_layers(keys: Sequence[torch.Tensor], values: Sequence[torch.Tensor],
                              key_caches: Sequence[torch.Tensor], value_caches: Sequence[torch.Tensor],
                              slot_mapping: torch.Tensor, k_scales=None, v_scales=None) -> None:
     """Append all layers of one step in a single launch (per group of EMM_MAX_LAYERS)."""
-    lib = _lib.load()
-    L = len(keys)
-    if not (len(values) == len(key_caches) == len(value_caches) == L):
-        raise ValueError("per-layer lists differ in length")
-    if L == 0:
-        return
-    _require_gpu(keys[0], "reshape_and_cache_layers")
-    if slot_mapping.dtype != torch.long:
-        raise TypeError("slot_mapping must be int64")
-    slot_mapping = slot_mapping.contiguous()
-    T, row, ks = _row_geometry(keys[0], "key")
-    _, _, vs = _row_geometry(values[0], "value")
-    for l in range(L):
-        if _row_geometry(keys[l], "key") != (T, row, ks) or _row_geometry(values[l], "value") != (T, row, vs):
-            raise ValueError(f"layer {l}: key/value geometry differs from layer 0")
-    if slot_mapping.numel() < T:
-        raise ValueError("slot_mapping is shorter than the token count")
-    num_slots = _cache_slots(key_caches[0], row, "key_cache")
-    for l in range(L):
-        if _cache_slots(key_caches[l], row, "key_cache") != num_slots or \
-                _cache_slots(value_caches[l], row, "value_cache") != num_slots:
-            raise ValueError(f"layer {l}: cache size differs from layer 0")
-    dev = keys[0].device
-    stream = _stream_ptr(dev)
-    eb = keys[0].element_size()
-    ceb = key_caches[0].element_size()
-    fp8 = ceb == 1 and eb == 2
-    if not fp8 and ceb != eb:
-        raise TypeError(f"unsupported source/cache element sizes {eb}/{ceb}")
-    if fp8:
-        code = _half_code(keys[0].dtype, "reshape_and_cache_layers")
-        k_s = _scales_tensor(k_scales, L, dev)
-        v_s = _scales_tensor(v_scales, L, dev)
-    for l0 in range(0, L, EMM_MAX_LAYERS):
-        sl = slice(l0, l0 + EMM_MAX_LAYERS)
-        kt = ptr_table([t.data_ptr() for t in keys[sl]])
-        vt = ptr_table([t.data_ptr() for t in values[sl]])
-        kct = ptr_table([t.data_ptr() for t in key_caches[sl]])
-        vct = ptr_table([t.data_ptr() for t in value_caches[sl]])
-        if fp8:
-            check(lib.emm_reshape_and_cache_fp8_layers(kt, vt, kct, vct, len(kt), slot_mapping.data_ptr(), T, row,
-                                                       ks, vs, num_slots, k_s.data_ptr() + 4 * l0,
-                                                       v_s.data_ptr() + 4 * l0, code, stream),
-                  "emm_reshape_and_cache_fp8_layers")
-        else:
-            check(lib.emm_reshape_and_cache_layers(kt, vt, kct, vct, len(kt), slot_mapping.data_ptr(), T, row * eb,
-                                                   ks * eb, vs * eb, num_slots, stream),
-                  "emm_reshape_and_cache_layers")
+    LayeredAppend(keys, values, key_caches, value_caches, k_scales, v_scales)(slot_mapping)
 
 
 def concat_rows(tensors: Sequence[torch.Tensor], out: Optional[torch.Tensor] = None) -> torch.Tensor:
