@@ -95,10 +95,15 @@ __device__ __forceinline__ V ld_stream(const char *p) {
 
 template <typename V, int POLICY>
 __device__ __forceinline__ void st_stream(char *p, V v) {
-  if constexpr (sizeof(V) == 16 && POLICY == 1) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+  // A store of more than 8 bytes reads its data registers after it has issued; the
+  // next instruction must not overwrite them. The compiler inserts that wait state
+  // for its own stores but cannot see inside an asm statement, hence the s_nop.
+  if constexpr (sizeof(V) == 8 && (POLICY == 1 || POLICY == 2)) {
+    asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
+  } else if constexpr (sizeof(V) == 16 && POLICY == 1) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
   } else if constexpr (sizeof(V) == 16 && POLICY == 2) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt" ::"v"(p), "v"(v) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
   } else {
     st<V, POLICY != 3>(p, v);
   }
@@ -447,28 +452,6 @@ __device__ __forceinline__ uint32_t f32_to_e4m3fn(float f) {
   return r | sign;
 }
 
-// fp32 -> bf16 bits, round to nearest even; NaN -> 0x7FC0.
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-  const uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0u;
-  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-}
-
-// fp32 -> f16 bits, round to nearest even; NaN -> 0x7E00.
-__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
-  // The product must be rounded to fp32 before it is rounded to f16. Without this
-  // barrier the compiler folds "convert(a * b)" into one mixed-precision
-  // multiply-convert with a single rounding, which differs in the last bit for
-  // some inputs.
-  asm volatile("" : "+v"(f));
-  const uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7e00u;
-  _Float16 h = (_Float16)f; // v_cvt_f16_f32: RNE
-  uint16_t b;
-  __builtin_memcpy(&b, &h, 2);
-  return b;
-}
-
 template <int SRC_DTYPE>
 __device__ __forceinline__ float half_bits_to_f32(uint32_t h) {
   if constexpr (SRC_DTYPE == EMM_DTYPE_BF16)
@@ -493,31 +476,53 @@ __device__ __forceinline__ u32x2 quant8(u32x4 in, float scale) {
 }
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
-// 16 e4m3fn bytes (one u32x4) -> 16 sixteen-bit values (two u32x4). The byte ->
-// fp32 step is v_cvt_pk_f32_fp8 (exact; its NaN carries the wrong sign, which the
-// 16-bit rounding below replaces by the canonical quiet NaN anyway).
+// two fp32 -> two 16-bit values in one dword, round to nearest even. The hardware
+// conversions (v_cvt_pk_bf16_f32, v_cvt_f16_f32) equal the integer formulation for
+// every non-NaN input (checked over all 2^32 bit patterns on the device); NaNs are
+// replaced by the canonical quiet NaN by the caller.
 template <int OUT_DTYPE>
-__device__ __forceinline__ void dequant16(u32x4 in, float scale, u32x4 &o0, u32x4 &o1) {
-  uint32_t o[8];
+__device__ __forceinline__ uint32_t pack16(float a, float b) {
+  // The products must be rounded to fp32 before they are rounded to 16 bits: the
+  // barrier stops the compiler from fusing multiply and convert into one
+  // mixed-precision instruction with a single rounding.
+  asm volatile("" : "+v"(a), "+v"(b));
+  uint32_t r;
+  if constexpr (OUT_DTYPE == EMM_DTYPE_BF16) {
+    const bf16x2 h = __builtin_convertvector(f32x2{a, b}, bf16x2);
+    __builtin_memcpy(&r, &h, 4);
+  } else {
+    const f16x2 h = __builtin_convertvector(f32x2{a, b}, f16x2);
+    __builtin_memcpy(&r, &h, 4);
+  }
+  return r;
+}
+
+// 8 e4m3fn bytes (one u32x2) -> 8 sixteen-bit values (one u32x4):
+// out = rne16(float(q) * scale); NaN bytes (0x7F / 0xFF) -> canonical quiet NaN.
+// The byte -> fp32 step is v_cvt_pk_f32_fp8 (exact).
+template <int OUT_DTYPE>
+__device__ __forceinline__ u32x4 dequant8(u32x2 in, float scale) {
+  constexpr uint32_t kNaN = OUT_DTYPE == EMM_DTYPE_BF16 ? 0x7fc0u : 0x7e00u;
+  uint32_t o[4];
 #pragma unroll
-  for (int w = 0; w < 4; ++w) {
+  for (int w = 0; w < 2; ++w) {
     const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)in[w], false); // bytes 0, 1
     const f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)in[w], true);  // bytes 2, 3
-    const float f[4] = {lo[0] * scale, lo[1] * scale, hi[0] * scale, hi[1] * scale};
-    uint32_t h[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      if constexpr (OUT_DTYPE == EMM_DTYPE_BF16)
-        h[k] = f32_to_bf16_bits(f[k]);
-      else
-        h[k] = f32_to_f16_bits(f[k]);
+    o[w * 2] = pack16<OUT_DTYPE>(lo[0] * scale, lo[1] * scale);
+    o[w * 2 + 1] = pack16<OUT_DTYPE>(hi[0] * scale, hi[1] * scale);
+    // a byte is NaN iff its low 7 bits are all ones: rare, patched out of line
+    const uint32_t nan = ((in[w] & 0x7f7f7f7fu) + 0x01010101u) & 0x80808080u;
+    if (nan) {
+      if (nan & 0x00000080u) o[w * 2] = (o[w * 2] & 0xffff0000u) | kNaN;
+      if (nan & 0x00008000u) o[w * 2] = (o[w * 2] & 0x0000ffffu) | (kNaN << 16);
+      if (nan & 0x00800000u) o[w * 2 + 1] = (o[w * 2 + 1] & 0xffff0000u) | kNaN;
+      if (nan & 0x80000000u) o[w * 2 + 1] = (o[w * 2 + 1] & 0x0000ffffu) | (kNaN << 16);
     }
-    o[w * 2] = h[0] | (h[1] << 16);
-    o[w * 2 + 1] = h[2] | (h[3] << 16);
   }
-  o0 = u32x4{o[0], o[1], o[2], o[3]};
-  o1 = u32x4{o[4], o[5], o[6], o[7]};
+  return u32x4{o[0], o[1], o[2], o[3]};
 }
 
 // ----------------------------------------------------------------------------
@@ -531,46 +536,37 @@ struct DequantParams {
   const float *v_scales;
   int64_t dst_num_blocks;
   int64_t chunk_elems; // fp8 bytes per chunk == elements
-  int64_t n;
-  uint32_t tiles_per_chunk;
+  int64_t n;  // blocks per plane of the transfer buffer
+  int64_t j0; // first block of this launch
 };
 
-// Tile = U * 256 lanes * 16 fp8 bytes in, twice that out.
-// grid: x = n * tiles_per_chunk, y = 2 (K, V), z = num_layers.
-template <int U, int OUT_DTYPE>
-__global__ __launch_bounds__(kThreads) void emm_unpack_dequant_fp8_kernel(
-    const DequantParams p) {
-  constexpr int64_t TILE = (int64_t)U * kThreads * 16;
-  uint32_t j = blockIdx.x, tile = 0;
-  if (p.tiles_per_chunk != 1) {
-    j = blockIdx.x / p.tiles_per_chunk;
-    tile = blockIdx.x - j * p.tiles_per_chunk;
-  }
-  const uint32_t kv = blockIdx.y, l = blockIdx.z;
-  const int64_t b = p.dst_idx[j];
-  if ((uint64_t)b >= (uint64_t)p.dst_num_blocks) return;
-  const float scale = kv == 0 ? p.k_scales[l] : p.v_scales[l];
+// One workgroup converts one tile of 4 KiB of fp8 bytes into 8 KiB. A wave owns 1 KiB of
+// input: lane i loads bytes [8i, 8i+8) and [512+8i, 512+8i+8) and stores the two 16-byte
+// results at twice those offsets, so that every load instruction covers 512 contiguous bytes
+// and every store instruction 1 KiB of whole cache lines.
+// grid: x = tiles per chunk, y = blocks (at most kMaxGridY per launch), z = 2 * layers.
+template <int OUT_DTYPE>
+__global__ __launch_bounds__(kThreads) void emm_unpack_dequant_fp8_kernel(const DequantParams p) {
+  constexpr int64_t TILE = (int64_t)kThreads * 16;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t j = p.j0 + blockIdx.y;
+  const uint32_t pl = blockIdx.z, l = pl >> 1, kv = pl & 1;
   const int64_t chunk = p.chunk_elems;
-  const int64_t tile_off = (int64_t)tile * TILE;
-  const char *src = p.packed + (((int64_t)l * 2 + kv) * p.n + j) * chunk + tile_off;
-  char *dst = p.dst_layers[l] + (((int64_t)kv * p.dst_num_blocks + b) * chunk + tile_off) * 2;
-  const int64_t limit = chunk - tile_off;
-  u32x4 v[U];
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    const int64_t off = ((int64_t)u * kThreads + threadIdx.x) * 16;
-    if (off < limit) v[u] = ld<u32x4, true>(src + off);
-  }
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    const int64_t off = ((int64_t)u * kThreads + threadIdx.x) * 16;
-    if (off < limit) {
-      u32x4 o0, o1;
-      dequant16<OUT_DTYPE>(v[u], scale, o0, o1);
-      st<u32x4, true>(dst + off * 2, o0);
-      st<u32x4, true>(dst + off * 2 + 16, o1);
-    }
-  }
+  const int64_t off0 = (int64_t)blockIdx.x * TILE + wave * 1024 + lane * 8;
+  const int64_t off1 = off0 + 512;
+  const bool live0 = off0 < chunk, live1 = off1 < chunk; // chunk is a multiple of 16
+  char *dst_layer = p.dst_layers[l];
+  const float scale = kv == 0 ? p.k_scales[l] : p.v_scales[l];
+  // the source does not depend on the block id: load first, then wait for the id
+  const char *src = p.packed + ((int64_t)pl * p.n + j) * chunk;
+  const u32x2 a = ld<u32x2, true>(src + (live0 ? off0 : 0));
+  const u32x2 c = ld<u32x2, true>(src + (live1 ? off1 : 0));
+  int64_t b = p.dst_idx[j];
+  asm volatile("" : "+s"(b) : : "memory");
+  if ((uint64_t)b >= (uint64_t)p.dst_num_blocks) return;
+  char *dst = dst_layer + ((int64_t)kv * p.dst_num_blocks + b) * chunk * 2;
+  if (live0) st_stream<u32x4, 1>(dst + off0 * 2, dequant8<OUT_DTYPE>(a, scale));
+  if (live1) st_stream<u32x4, 1>(dst + off1 * 2, dequant8<OUT_DTYPE>(c, scale));
 }
 
 // ----------------------------------------------------------------------------
@@ -658,10 +654,11 @@ __global__ __launch_bounds__(kThreads) void emm_append_kernel(const AppendParams
   }
 }
 
-// fp8 append. VEC_ELEMS = 16: each lane converts 16 contiguous 16-bit elements
-// (two 16-byte loads) into one 16-byte store, a wave covers 1024 elements per
-// step; VEC_ELEMS = 8: 16 bytes in, 8 bytes out; VEC_ELEMS = 1: element-wise
-// path for odd row sizes or misaligned bases.
+// fp8 append. VEC_ELEMS = 8: a wave converts a row in pieces of 1024 elements; lane i
+// loads elements [8i, 8i+8) and [512+8i, 512+8i+8) of the piece (two 16-byte loads, each
+// instruction 1 KiB contiguous) and stores the two 8-byte results at those element offsets
+// (each instruction 512 contiguous bytes of whole cache lines). VEC_ELEMS = 1:
+// element-wise path for rows that are not a multiple of 8 elements or misaligned bases.
 template <int SRC_DTYPE, int VEC_ELEMS, int R>
 __global__ __launch_bounds__(kThreads) void emm_append_fp8_kernel(const AppendParams p) {
   const int lane = threadIdx.x & 63;
@@ -677,45 +674,37 @@ __global__ __launch_bounds__(kThreads) void emm_append_fp8_kernel(const AppendPa
 
   int64_t slot[R];
   fetch_slots<R>(slot, p.slot_mapping, t0, p.num_tokens);
-  if constexpr (VEC_ELEMS == 16) {
-    int64_t e = (int64_t)lane * 16;
+  if constexpr (VEC_ELEMS == 8) {
+    int64_t e0 = (int64_t)lane * 8, e1 = e0 + 512;
     u32x4 a[R], b[R];
+    // first piece: issued before the slots are waited for (rows of padded tokens are read and dropped)
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      if (t0 + r < p.num_tokens && e < row) {
-        const char *sp = src_base + ((t0 + r) * stride + e) * 2;
-        a[r] = ld<u32x4, true>(sp);
-        b[r] = ld<u32x4, true>(sp + 16);
+      if (t0 + r < p.num_tokens) {
+        const char *sp = src_base + (t0 + r) * stride * 2;
+        a[r] = ld<u32x4, true>(sp + (e0 < row ? e0 : 0) * 2);
+        b[r] = ld<u32x4, true>(sp + (e1 < row ? e1 : 0) * 2);
       }
     resolve_slots<R>(slot, p.num_slots);
-    while (e < row) {
+    while (e0 < row) {
 #pragma unroll
       for (int r = 0; r < R; ++r)
         if (slot[r] >= 0) {
-          const u32x2 lo = quant8<SRC_DTYPE>(a[r], scale), hi = quant8<SRC_DTYPE>(b[r], scale);
-          st_stream<u32x4, 1>(dst_base + slot[r] * row + e, u32x4{lo[0], lo[1], hi[0], hi[1]});
+          char *dp = dst_base + slot[r] * row;
+          st_stream<u32x2, 1>(dp + e0, quant8<SRC_DTYPE>(a[r], scale));
+          if (e1 < row) st_stream<u32x2, 1>(dp + e1, quant8<SRC_DTYPE>(b[r], scale));
         }
-      e += 64 * 16;
-      if (e < row) {
+      e0 += 1024;
+      e1 += 1024;
+      if (e0 < row) {
 #pragma unroll
         for (int r = 0; r < R; ++r)
           if (slot[r] >= 0) {
-            const char *sp = src_base + ((t0 + r) * stride + e) * 2;
-            a[r] = ld<u32x4, true>(sp);
-            b[r] = ld<u32x4, true>(sp + 16);
+            const char *sp = src_base + (t0 + r) * stride * 2;
+            a[r] = ld<u32x4, true>(sp + e0 * 2);
+            b[r] = ld<u32x4, true>(sp + (e1 < row ? e1 : e0) * 2);
           }
       }
-    }
-  } else if constexpr (VEC_ELEMS == 8) {
-    resolve_slots<R>(slot, p.num_slots);
-    for (int64_t e = (int64_t)lane * 8; e < row; e += 64 * 8) {
-      u32x4 v[R];
-#pragma unroll
-      for (int r = 0; r < R; ++r)
-        if (slot[r] >= 0) v[r] = ld<u32x4, true>(src_base + ((t0 + r) * stride + e) * 2);
-#pragma unroll
-      for (int r = 0; r < R; ++r)
-        if (slot[r] >= 0) st<u32x2, true>(dst_base + slot[r] * row + e, quant8<SRC_DTYPE>(v[r], scale));
     }
   } else {
     resolve_slots<R>(slot, p.num_slots);
@@ -819,8 +808,7 @@ int append_fp8(const void *const *k, const void *const *v, void *const *kc, void
   if (!k_scales || !v_scales) return fail(EMM_EINVAL, "%s: scale pointer is null", what);
   AppendParams p;
   memset(&p, 0, sizeof(p));
-  int width = 16;
-  if (row_elems % 16 || ks % 8 || vs % 8) width = (row_elems % 8 || ks % 8 || vs % 8) ? 1 : 8;
+  int width = (row_elems % 8 || ks % 8 || vs % 8) ? 1 : 8;
   for (int l = 0; l < num_layers; ++l) {
     p.key[l] = (const char *)k[l];
     p.value[l] = (const char *)v[l];
@@ -828,9 +816,7 @@ int append_fp8(const void *const *k, const void *const *v, void *const *kc, void
     p.value_cache[l] = (char *)vc[l];
     if (!aligned(k[l], 2) || !aligned(v[l], 2))
       return fail(EMM_EINVAL, "%s: 16-bit source not 2-byte aligned at layer %d", what, l);
-    if (!aligned(k[l], 16) || !aligned(v[l], 16)) width = 1;
-    if (width == 16 && (!aligned(kc[l], 16) || !aligned(vc[l], 16))) width = 8;
-    if (width == 8 && (!aligned(kc[l], 8) || !aligned(vc[l], 8))) width = 1;
+    if (!aligned(k[l], 16) || !aligned(v[l], 16) || !aligned(kc[l], 8) || !aligned(vc[l], 8)) width = 1;
   }
   p.slot_mapping = slot_mapping;
   p.k_scales = k_scales;
@@ -844,14 +830,13 @@ int append_fp8(const void *const *k, const void *const *v, void *const *kc, void
   // flight per lane in a large launch; a small launch needs the extra workgroups of one row
   int rows = (num_tokens * num_layers >= 100000) ? 2 : 1;
   if (g_append_rows == 1 || g_append_rows == 2 || g_append_rows == 4) rows = g_append_rows;
-  dim3 grid = append_grid(num_tokens, num_layers, width == 16 ? rows : 4);
+  dim3 grid = append_grid(num_tokens, num_layers, width == 8 ? rows : 4);
 #define EMM_FP8_LAUNCH(DT)                                                                  \
-  if (width == 16) {                                                                        \
-    if (rows == 4) emm_append_fp8_kernel<DT, 16, 4><<<grid, kThreads, 0, s>>>(p);           \
-    else if (rows == 2) emm_append_fp8_kernel<DT, 16, 2><<<grid, kThreads, 0, s>>>(p);      \
-    else emm_append_fp8_kernel<DT, 16, 1><<<grid, kThreads, 0, s>>>(p);                     \
-  } else if (width == 8) emm_append_fp8_kernel<DT, 8, 4><<<grid, kThreads, 0, s>>>(p);      \
-  else emm_append_fp8_kernel<DT, 1, 4><<<grid, kThreads, 0, s>>>(p);
+  if (width == 8) {                                                                         \
+    if (rows == 4) emm_append_fp8_kernel<DT, 8, 4><<<grid, kThreads, 0, s>>>(p);            \
+    else if (rows == 2) emm_append_fp8_kernel<DT, 8, 2><<<grid, kThreads, 0, s>>>(p);       \
+    else emm_append_fp8_kernel<DT, 8, 1><<<grid, kThreads, 0, s>>>(p);                      \
+  } else emm_append_fp8_kernel<DT, 1, 4><<<grid, kThreads, 0, s>>>(p);
   if (src_dtype == EMM_DTYPE_BF16) { EMM_FP8_LAUNCH(EMM_DTYPE_BF16) } else { EMM_FP8_LAUNCH(EMM_DTYPE_F16) }
 #undef EMM_FP8_LAUNCH
   return check_launch(what);
@@ -880,7 +865,7 @@ __global__ __launch_bounds__(kThreads) void emm_concat_rows_kernel(const ConcatP
     if (p.tile_start[mid] <= w) lo = mid; else hi = mid - 1;
   }
   const int64_t off = (int64_t)(w - p.tile_start[lo]) * TILE;
-  copy_tile<V, kThreads, U, 0>(p.src[lo] + off, p.dst + p.dst_off[lo] + off, p.nbytes[lo] - off);
+  copy_tile<V, kThreads, U, sizeof(V) == 16 ? 1 : 0>(p.src[lo] + off, p.dst + p.dst_off[lo] + off, p.nbytes[lo] - off);
 }
 
 hipStream_t as_stream(emm_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
@@ -995,18 +980,21 @@ int emm_kv_unpack_dequant_fp8(void *const *layer_ptrs, int num_layers, int64_t n
   p.dst_num_blocks = num_blocks;
   p.chunk_elems = chunk_elems;
   p.n = n;
-  constexpr int U = 2;
-  const int64_t tile = (int64_t)U * kThreads * 16;
+  const int64_t tile = (int64_t)kThreads * 16;
   const int64_t tpc = (chunk_elems + tile - 1) / tile;
-  if (tpc > 0x7fffffffLL || n * tpc > 0x7fffffffLL)
-    return fail(EMM_EINVAL, "%s: grid too large", what);
-  p.tiles_per_chunk = (uint32_t)tpc;
-  dim3 grid((uint32_t)(n * tpc), 2, (uint32_t)num_layers);
-  if (out_dtype == EMM_DTYPE_BF16)
-    emm_unpack_dequant_fp8_kernel<U, EMM_DTYPE_BF16><<<grid, kThreads, 0, as_stream(stream)>>>(p);
-  else
-    emm_unpack_dequant_fp8_kernel<U, EMM_DTYPE_F16><<<grid, kThreads, 0, as_stream(stream)>>>(p);
-  return check_launch(what);
+  if (tpc > 0x7fffffffLL) return fail(EMM_EINVAL, "%s: grid too large", what);
+  for (int64_t j0 = 0; j0 < n; j0 += kMaxGridY) {
+    const int64_t ny = (n - j0 < kMaxGridY) ? (n - j0) : kMaxGridY;
+    p.j0 = j0;
+    dim3 grid((uint32_t)tpc, (uint32_t)ny, (uint32_t)(2 * num_layers));
+    if (out_dtype == EMM_DTYPE_BF16)
+      emm_unpack_dequant_fp8_kernel<EMM_DTYPE_BF16><<<grid, kThreads, 0, as_stream(stream)>>>(p);
+    else
+      emm_unpack_dequant_fp8_kernel<EMM_DTYPE_F16><<<grid, kThreads, 0, as_stream(stream)>>>(p);
+    const int rc2 = check_launch(what);
+    if (rc2 != EMM_OK) return rc2;
+  }
+  return EMM_OK;
 }
 
 int emm_reshape_and_cache(const void *key, const void *value, void *key_cache,
@@ -1063,7 +1051,6 @@ int emm_concat_rows(const void *const *srcs, const int64_t *nbytes, int n, void 
     return fail(EMM_EINVAL, "%s: null pointer / negative offset", what);
   ConcatParams p;
   memset(&p, 0, sizeof(p));
-  constexpr int U = 4;
   int al = common_align(16, (const char *)dst + dst_offset_bytes);
   int64_t off = dst_offset_bytes;
   int m = 0;
@@ -1081,7 +1068,9 @@ int emm_concat_rows(const void *const *srcs, const int64_t *nbytes, int n, void 
   }
   if (m == 0) return EMM_OK;
   if (al == 8) al = 4;
-  const int64_t tile = (int64_t)U * kThreads * al;
+  // 16-byte lanes: one vector per lane (4 KiB tiles); narrower lanes: four
+  const int unroll = al == 16 ? 1 : 4;
+  const int64_t tile = (int64_t)unroll * kThreads * al;
   uint64_t tiles = 0;
   for (int i = 0; i < m; ++i) {
     p.tile_start[i] = (uint32_t)tiles;
@@ -1094,10 +1083,10 @@ int emm_concat_rows(const void *const *srcs, const int64_t *nbytes, int n, void 
   dim3 grid((uint32_t)tiles);
   hipStream_t s = as_stream(stream);
   switch (al) {
-  case 16: emm_concat_rows_kernel<u32x4, U><<<grid, kThreads, 0, s>>>(p); break;
-  case 4: emm_concat_rows_kernel<uint32_t, U><<<grid, kThreads, 0, s>>>(p); break;
-  case 2: emm_concat_rows_kernel<uint16_t, U><<<grid, kThreads, 0, s>>>(p); break;
-  default: emm_concat_rows_kernel<uint8_t, U><<<grid, kThreads, 0, s>>>(p); break;
+  case 16: emm_concat_rows_kernel<u32x4, 1><<<grid, kThreads, 0, s>>>(p); break;
+  case 4: emm_concat_rows_kernel<uint32_t, 4><<<grid, kThreads, 0, s>>>(p); break;
+  case 2: emm_concat_rows_kernel<uint16_t, 4><<<grid, kThreads, 0, s>>>(p); break;
+  default: emm_concat_rows_kernel<uint8_t, 4><<<grid, kThreads, 0, s>>>(p); break;
   }
   return check_launch(what);
 }
