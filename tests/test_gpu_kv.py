@@ -605,3 +605,86 @@ def test_cfg2_full_size_migration_properties():
     assert ok, "copy_blocks changed a source block"
     del src, dst
     torch.cuda.empty_cache()
+
+
+# ------------------------------------------------------------------ prepared plan / HIP graph
+def test_layered_append_plan_reuse_and_graph_replay():
+    """A prepared whole-step append is reused with new data and new slots, and the per-layer
+    appends replayed from a captured HIP graph give the eager result on every replay (the
+    program's own eager work and synchronisations run between the replays)."""
+    NB, bs, H, D, T, L = 64, 16, 4, 128, 300, 3
+    g = torch.Generator().manual_seed(15)
+    keys = [torch.zeros((T, H, D), dtype=torch.bfloat16, device=DEV) for _ in range(L)]
+    values = [torch.zeros((T, H, D), dtype=torch.bfloat16, device=DEV) for _ in range(L)]
+    slots_g = torch.zeros(T, dtype=torch.long, device=DEV)
+    pool_plan = [torch.zeros((2, NB, bs, H, D), dtype=torch.bfloat16, device=DEV) for _ in range(L)]
+    pool_graph = [torch.zeros((2, NB, bs, H, D), dtype=torch.bfloat16, device=DEV) for _ in range(L)]
+    pool_c = [torch.zeros((2, NB, bs, H, D), dtype=torch.bfloat16) for _ in range(L)]
+    plan = cache_ops.layered_append(keys, values, pool_plan, "auto")
+
+    def per_layer():
+        for l in range(L):
+            cache_ops.reshape_and_cache_flash(keys[l], values[l], pool_graph[l][0], pool_graph[l][1], slots_g, "auto")
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        per_layer()                      # warm-up outside capture
+    torch.cuda.current_stream().wait_stream(side)
+    for p in pool_graph:
+        p.zero_()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        per_layer()
+    for it in range(4):
+        slots = make_slots(NB * bs, T, 100 + it, pad_frac=0.1)
+        slots_g.copy_(slots)
+        for l in range(L):
+            k = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+            v = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+            keys[l].copy_(k)
+            values[l].copy_(v)
+            orc.c_reshape_and_cache(k, v, pool_c[l][0], pool_c[l][1], slots)
+        plan(slots_g)
+        graph.replay()
+        torch.cuda.synchronize()
+        # unrelated eager work between replays
+        junk = kv_ops.kv_pack(PoolView(pool_plan), [1, 2, 3])
+        assert junk.shape[2] == 3
+        for l in range(L):
+            assert same_bits(pool_plan[l], pool_c[l]), f"plan, iteration {it}, layer {l}"
+            assert same_bits(pool_graph[l], pool_c[l]), f"graph replay {it}, layer {l}"
+
+
+def test_large_block_count_splits_launches():
+    """More than 65 535 blocks in one call (the grid's y limit): tiny chunks keep it small."""
+    NB, n = 70000, 66000
+    g = torch.Generator().manual_seed(16)
+    src_c = [torch.randint(0, 255, (2, NB, 1, 1, 16), generator=g, dtype=torch.uint8)]
+    si = torch.randperm(NB, generator=g)[:n]
+    di = torch.randperm(NB, generator=g)[:n]
+    src_g = to_dev(src_c)
+    buf = kv_ops.kv_pack(PoolView(src_g), si.to(DEV))
+    assert same_bits(buf, orc.c_kv_pack(src_c, si.numpy()))
+    dst_g = [torch.zeros_like(src_g[0])]
+    kv_ops.kv_unpack(PoolView(dst_g), di.to(DEV), buf)
+    dst_c = [torch.zeros_like(src_c[0])]
+    orc.c_kv_unpack(dst_c, di.numpy(), raw(buf))
+    assert same_bits(dst_g[0], dst_c[0])
+    dst2 = [torch.zeros_like(src_g[0])]
+    kv_ops.kv_migrate(PoolView(src_g), si.to(DEV), PoolView(dst2), di.to(DEV))
+    assert same_bits(dst2[0], dst_c[0])
+    mapping = torch.stack([si[:33000], di[:33000]], 1)
+    free_dst = torch.tensor(sorted(set(range(NB)) - set(si.tolist()))[:4000])
+    mapping = torch.stack([si[:4000], free_dst], 1).contiguous()
+    cp_g = to_dev(src_c)
+    kv_ops.copy_blocks(PoolView(cp_g), mapping.to(DEV))
+    cp_c = [src_c[0].clone()]
+    orc.c_copy_blocks(cp_c, mapping.numpy())
+    assert same_bits(cp_g[0], cp_c[0])
+    # dequantising unpack with more than 65 535 blocks
+    dq_g = [torch.zeros((2, NB, 1, 1, 16), dtype=torch.bfloat16, device=DEV)]
+    dq_c = [torch.zeros((2, NB, 1, 1, 16), dtype=torch.bfloat16)]
+    kv_ops.kv_unpack_dequant_fp8(PoolView(dq_g), di.to(DEV), buf, [0.05], [0.07])
+    orc.c_unpack_dequant_fp8(dq_c, di.numpy(), raw(buf), [0.05], [0.07])
+    assert same_bits(dq_g[0], dq_c[0])
