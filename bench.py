@@ -257,6 +257,12 @@ def main():
     print(json.dumps(result), flush=True)
 
 
+def _wall(fn):
+    t0 = time.perf_counter()
+    fn()
+    return time.perf_counter() - t0
+
+
 def timed(fn, iters, warmup=2):
     """Median and min milliseconds of fn() over iters runs, HIP events on the current stream."""
     for _ in range(warmup):
@@ -420,6 +426,44 @@ def extended(dev):
         del buf
     out["fp8_70b_shape"]["dequant_unpack_GBps"] = round(3 * pay / (t_dq * 1e-3) / 1e9, 1)
     del src, sp, dq, dqp
+    torch.cuda.empty_cache()
+
+    # ---- GPU <-> CPU swap (pinned host pool, kernels read / write it over PCIe): Qwen2-7B layout
+    from elasticmm_amd.worker import KVWorker
+    w = KVWorker(0, "cuda:0", 16)
+    w.init_kvcache(4096, 2048, num_layers=28, num_kv_heads=4, head_size=128, dtype=torch.bfloat16)
+    for t in w.kv_cache:
+        t.normal_(0.0, 0.5)
+    gsw = torch.Generator().manual_seed(6)
+    nsw = 1024
+    gpu_ids = torch.randperm(4096, generator=gsw)[:nsw].to(dev)
+    cpu_ids = torch.randperm(2048, generator=gsw)[:nsw].to(dev)
+    sw_bytes = nsw * 28 * 2 * 16 * 4 * 128 * 2
+
+    def swap(is_in):
+        w.swap_blocks(["r"], cpu_ids if is_in else gpu_ids, gpu_ids if is_in else cpu_ids, is_in)
+        (w.swap_in_stream if is_in else w.swap_out_stream).synchronize()
+
+    t_out = min(_wall(lambda: swap(False)) for _ in range(4))
+    t_in = min(_wall(lambda: swap(True)) for _ in range(4))
+    stage_g = torch.empty(sw_bytes, dtype=torch.uint8, device=dev)
+    stage_c = torch.empty(sw_bytes, dtype=torch.uint8, pin_memory=True)
+
+    def d2h():
+        stage_c.copy_(stage_g, non_blocking=True)
+        torch.cuda.synchronize()
+
+    def h2d():
+        stage_g.copy_(stage_c, non_blocking=True)
+        torch.cuda.synchronize()
+
+    t_d2h = min(_wall(d2h) for _ in range(4))
+    t_h2d = min(_wall(h2d) for _ in range(4))
+    out["swap_pcie"] = {"blocks": nsw, "GB": round(sw_bytes / 1e9, 3),
+                        "swap_out_GBps": round(sw_bytes / t_out / 1e9, 1), "swap_in_GBps": round(sw_bytes / t_in / 1e9, 1),
+                        "contiguous_memcpy_d2h_GBps": round(sw_bytes / t_d2h / 1e9, 1),
+                        "contiguous_memcpy_h2d_GBps": round(sw_bytes / t_h2d / 1e9, 1)}
+    del w, stage_g, stage_c
     torch.cuda.empty_cache()
 
     # ---- rebalancing: ~200 GB bf16 pool in the Qwen2-7B layout, move 50 % of the live half

@@ -845,27 +845,37 @@ int append_fp8(const void *const *k, const void *const *v, void *const *kc, void
 // ----------------------------------------------------------------------------
 // concat_rows: ragged segments -> one contiguous buffer
 // ----------------------------------------------------------------------------
+constexpr int kSegGroup = 12; // segments per group of the two-level tile -> segment search
+constexpr int kSegGroups = EMM_MAX_SEGMENTS / kSegGroup;
+static_assert(kSegGroups * kSegGroup == EMM_MAX_SEGMENTS, "segment table must split into whole groups");
+
 struct ConcatParams {
   const char *src[EMM_MAX_SEGMENTS];
   int64_t dst_off[EMM_MAX_SEGMENTS];
   int64_t nbytes[EMM_MAX_SEGMENTS];
-  uint32_t tile_start[EMM_MAX_SEGMENTS + 1]; // prefix sum of tiles per segment
+  uint32_t tile_start[EMM_MAX_SEGMENTS]; // first tile of each segment; unused entries 0xFFFFFFFF
+  uint32_t group_start[kSegGroups];      // tile_start[kSegGroup * g]
   char *dst;
-  int32_t n;
 };
 
 template <typename V, int U>
 __global__ __launch_bounds__(kThreads) void emm_concat_rows_kernel(const ConcatParams p) {
   constexpr int64_t TILE = (int64_t)U * kThreads * sizeof(V);
   const uint32_t w = blockIdx.x;
-  // wave-uniform binary search: last segment whose first tile is <= w
-  int lo = 0, hi = p.n - 1;
-  while (lo < hi) {
-    const int mid = (lo + hi + 1) >> 1;
-    if (p.tile_start[mid] <= w) lo = mid; else hi = mid - 1;
-  }
-  const int64_t off = (int64_t)(w - p.tile_start[lo]) * TILE;
-  copy_tile<V, kThreads, U, sizeof(V) == 16 ? 1 : 0>(p.src[lo] + off, p.dst + p.dst_off[lo] + off, p.nbytes[lo] - off);
+  // Wave-uniform search for the last segment whose first tile is <= w, as two rounds
+  // of counting over small fixed tables (two dependent fetches of the argument block
+  // instead of the seven of a binary search over 96 entries).
+  int g = -1;
+#pragma unroll
+  for (int k = 0; k < kSegGroups; ++k) g += p.group_start[k] <= w ? 1 : 0;
+  const uint32_t *ts = p.tile_start + g * kSegGroup;
+  int i = -1;
+#pragma unroll
+  for (int k = 0; k < kSegGroup; ++k) i += ts[k] <= w ? 1 : 0;
+  const int seg = g * kSegGroup + i;
+  const int64_t off = (int64_t)(w - p.tile_start[seg]) * TILE;
+  copy_tile<V, kThreads, U, sizeof(V) == 16 ? 1 : 0>(p.src[seg] + off, p.dst + p.dst_off[seg] + off,
+                                                     p.nbytes[seg] - off);
 }
 
 hipStream_t as_stream(emm_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
@@ -1072,14 +1082,14 @@ int emm_concat_rows(const void *const *srcs, const int64_t *nbytes, int n, void 
   const int unroll = al == 16 ? 1 : 4;
   const int64_t tile = (int64_t)unroll * kThreads * al;
   uint64_t tiles = 0;
+  for (int i = 0; i < EMM_MAX_SEGMENTS; ++i) p.tile_start[i] = 0xffffffffu;
   for (int i = 0; i < m; ++i) {
     p.tile_start[i] = (uint32_t)tiles;
     tiles += (uint64_t)((p.nbytes[i] + tile - 1) / tile);
     if (tiles > 0x7fffffffULL) return fail(EMM_EINVAL, "%s: grid too large", what);
   }
-  p.tile_start[m] = (uint32_t)tiles;
+  for (int g = 0; g < kSegGroups; ++g) p.group_start[g] = p.tile_start[g * kSegGroup];
   p.dst = (char *)dst;
-  p.n = m;
   dim3 grid((uint32_t)tiles);
   hipStream_t s = as_stream(stream);
   switch (al) {

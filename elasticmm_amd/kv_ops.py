@@ -75,7 +75,10 @@ class PoolView:
     ``[num_blocks, tokens, dim]`` is viewed with num_kv = 1).
     """
 
-    def __init__(self, kv_cache: Union[Sequence[torch.Tensor], torch.Tensor], num_kv_dim: bool = True):
+    def __init__(self, kv_cache: Union[Sequence[torch.Tensor], torch.Tensor], num_kv_dim: bool = True,
+                 pinned_host_for: Optional[torch.device] = None):
+        """``pinned_host_for``: accept page-locked host tensors (a CPU swap pool) that the
+        kernels of the given GPU read and write directly over PCIe."""
         if isinstance(kv_cache, torch.Tensor):
             layers = list(kv_cache.unbind(0))
         else:
@@ -84,13 +87,18 @@ class PoolView:
             raise ValueError("empty KV pool")
         first = layers[0]
         for i, t in enumerate(layers):
-            _require_gpu(t, "PoolView")
+            if pinned_host_for is not None:
+                if t.is_cuda or not t.is_pinned():
+                    raise RuntimeError("PoolView: a host pool must consist of pinned (page-locked) CPU tensors")
+            else:
+                _require_gpu(t, "PoolView")
             if t.shape != first.shape or t.dtype != first.dtype or t.device != first.device:
                 raise ValueError(f"layer {i} differs from layer 0 in shape / dtype / device")
             if not t.is_contiguous():
                 raise ValueError(f"layer {i} is not contiguous")
         self.layers: List[torch.Tensor] = layers
-        self.device = first.device
+        self.device = first.device if pinned_host_for is None else torch.device(pinned_host_for)
+        self.on_host = pinned_host_for is not None
         self.dtype = first.dtype
         self.elem_bytes = first.element_size()
         if num_kv_dim:
@@ -164,6 +172,8 @@ def kv_migrate(src: PoolView, src_indices: IndexLike, dst: PoolView, dst_indices
     lib = _lib.load()
     if (src.num_layers, src.num_kv, src.chunk_bytes, src.device) != (dst.num_layers, dst.num_kv, dst.chunk_bytes, dst.device):
         raise ValueError("kv_migrate: pools differ in layers / kv / chunk size / device")
+    if src.on_host and dst.on_host:
+        raise ValueError("kv_migrate: at least one pool must live in GPU memory")
     si = block_index_tensor(src_indices, src.num_blocks, src.device)
     di = block_index_tensor(dst_indices, dst.num_blocks, dst.device)
     if si.numel() != di.numel():

@@ -11,6 +11,7 @@ methods that touch KV / vision-embedding tensors:
   collective_transfer_kv                                      worker.py:939-1005
   extract_vision_blocks / write_vision_blocks                 worker.py:1007-1036
   init_kvcache (pool allocation only)                         worker.py:358-418
+  swap_blocks / wait_for_all_swap_in / wait_for_all_swap_out  worker.py:467-526
 
 Model loading, Ray actor plumbing and step_* execution are not part of this
 class. The cross-GPU hop (``torch.distributed.send/recv``) is replaced by a
@@ -77,6 +78,14 @@ class KVWorker:
         self.global_rank = global_rank
         self.nccl_pg_initialized = link is not None and global_rank is not None
         self.peers: Dict[int, "KVWorker"] = {}
+        # CPU swap tier (worker.py:98-108): created lazily, they need a GPU
+        self.kv_swap: Optional[List[torch.Tensor]] = None
+        self._swap_pool: Optional[PoolView] = None
+        self.swap_in_stream: Optional[torch.cuda.Stream] = None
+        self.swap_out_stream: Optional[torch.cuda.Stream] = None
+        self.swap_event_table: Dict[str, torch.cuda.Event] = {}
+        self.latest_swap_in_event: Optional[torch.cuda.Event] = None
+        self.latest_swap_out_event: Optional[torch.cuda.Event] = None
 
     # ----- pool -----------------------------------------------------------
     def init_kvcache(self, num_gpu_blocks: int, num_cpu_blocks: int = 0, *, num_layers: int, num_kv_heads: int,
@@ -92,12 +101,21 @@ class KVWorker:
         else:
             layers = [torch.empty(shape, dtype=dtype, device=self.device) for _ in range(num_layers)]
         self.bind_kv_cache(layers)
+        if num_cpu_blocks > 0:
+            cpu_shape = (2, num_cpu_blocks, self.block_size, num_kv_heads, head_size)
+            self.bind_kv_swap([torch.empty(cpu_shape, dtype=dtype, pin_memory=True) for _ in range(num_layers)])
         return []  # placeholder for an IPC handle, as in the reference (worker.py:418)
 
     def bind_kv_cache(self, kv_cache: Sequence[torch.Tensor]) -> None:
         """Adopt an existing pool (e.g. the list vLLM's CacheEngine allocated)."""
         self.kv_cache = list(kv_cache)
         self._pool = PoolView(self.kv_cache)
+
+    def bind_kv_swap(self, kv_swap: Sequence[torch.Tensor]) -> None:
+        """Adopt a CPU swap pool: L pinned host tensors ``[2, num_cpu_blocks, bs, H, D]`` (the
+        layout of vLLM's ``cpu_cache``, worker.py:389)."""
+        self.kv_swap = list(kv_swap)
+        self._swap_pool = PoolView(self.kv_swap, pinned_host_for=self.device)
 
     def init_vecache(self, num_gpu_blocks: int = 0, num_cpu_blocks: int = 0) -> List[int]:
         """Vision embeddings are kept per request id (worker.py:431-437)."""
@@ -311,6 +329,56 @@ class KVWorker:
             raise ValueError(f"[KVWorker] Unknown collective transfer mode: {mode}")
         torch.cuda.synchronize(self.device)
         return {"bytes": bytes_transferred, "mode": mode}
+
+    # ----- GPU <-> CPU swap (worker.py:467-526) ------------------------------
+    def wait_for_all_swap_out(self) -> None:
+        if self.latest_swap_out_event:
+            self.latest_swap_out_event.wait()
+
+    def wait_for_all_swap_in(self) -> None:
+        if self.latest_swap_in_event:
+            self.latest_swap_in_event.wait()
+
+    def swap_blocks(self, request_ids: List[str], source_block_ids: List[int], target_block_ids: List[int],
+                    is_swap_in: bool) -> None:
+        """Copy blocks between the CPU swap pool and the GPU pool: swap-in moves CPU block
+        ``source_block_ids[i]`` to GPU block ``target_block_ids[i]``, swap-out the other way.
+        One kernel per call reads / writes the pinned host pool directly over PCIe (all layers,
+        K and V), on the swap-in / swap-out side stream. A request's swaps are ordered by its
+        event; the event is recorded after the copy so that waiting on it means the data has
+        arrived (the reference records it before issuing the copy, worker.py:499-500, and then
+        indexes the per-layer list as one tensor, :521/:526, which cannot run)."""
+        if self.kv_cache is None or self.kv_swap is None:
+            raise RuntimeError("KV cache / swap pool not initialized")
+        if len(source_block_ids) != len(target_block_ids):
+            raise ValueError(f"Block count mismatch: src={len(source_block_ids)}, dst={len(target_block_ids)}")
+        if self.swap_in_stream is None:
+            self.swap_in_stream = torch.cuda.Stream(self.device)
+            self.swap_out_stream = torch.cuda.Stream(self.device)
+        stream = self.swap_in_stream if is_swap_in else self.swap_out_stream
+        # the side stream starts after what the caller has queued so far (blocks being swapped
+        # out must have been written; blocks being swapped in must no longer be read)
+        stream.wait_stream(torch.cuda.current_stream(self.device))
+        for request_id in request_ids:
+            if request_id in self.swap_event_table:
+                self.swap_event_table[request_id].wait(stream)
+        with torch.cuda.stream(stream):
+            if is_swap_in:
+                kv_ops.kv_migrate(self._swap_pool, source_block_ids, self.pool, target_block_ids)
+            else:
+                kv_ops.kv_migrate(self.pool, source_block_ids, self._swap_pool, target_block_ids)
+            event = torch.cuda.Event()
+            event.record(stream)
+        for request_id in request_ids:
+            self.swap_event_table[request_id] = event
+        if is_swap_in:
+            self.latest_swap_in_event = event
+        else:
+            self.latest_swap_out_event = event
+
+    def clear_request_resource(self, request_id: str) -> None:
+        """worker.py:528-532: forget the request's swap event."""
+        self.swap_event_table.pop(request_id, None)
 
     # ----- vision embeddings (worker.py:1007-1036, worker_steps.py:252-267) --
     def extract_vision_blocks(self, request_id: str) -> torch.Tensor:

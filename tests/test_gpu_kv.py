@@ -688,3 +688,46 @@ def test_large_block_count_splits_launches():
     kv_ops.kv_unpack_dequant_fp8(PoolView(dq_g), di.to(DEV), buf, [0.05], [0.07])
     orc.c_unpack_dequant_fp8(dq_c, di.numpy(), raw(buf), [0.05], [0.07])
     assert same_bits(dq_g[0], dq_c[0])
+
+
+# ------------------------------------------------------------------ GPU <-> CPU swap
+def test_swap_blocks_out_and_in():
+    L, NB, NBC, bs, H, D = 3, 24, 10, 16, 2, 64
+    w = KVWorker(0, DEV, bs)
+    w.init_kvcache(NB, NBC, num_layers=L, num_kv_heads=H, head_size=D, dtype=torch.bfloat16)
+    assert len(w.kv_swap) == L and w.kv_swap[0].is_pinned() and tuple(w.kv_swap[0].shape) == (2, NBC, bs, H, D)
+    g = torch.Generator().manual_seed(17)
+    gpu_c = [torch.randn((2, NB, bs, H, D), generator=g).to(torch.bfloat16) for _ in range(L)]
+    for t, c in zip(w.kv_cache, gpu_c):
+        t.copy_(c)
+    for t in w.kv_swap:
+        t.fill_(-4.0)
+    torch.cuda.synchronize()
+    src_gpu, dst_cpu = [5, 17, 2, 23], [9, 0, 4, 1]
+    w.swap_blocks(["r1", "r2"], src_gpu, dst_cpu, is_swap_in=False)
+    w.wait_for_all_swap_out()
+    torch.cuda.synchronize()
+    cpu_want = [torch.full((2, NBC, bs, H, D), -4.0, dtype=torch.bfloat16) for _ in range(L)]
+    for l in range(L):
+        cpu_want[l][:, dst_cpu] = gpu_c[l][:, src_gpu]
+        assert same_bits(w.kv_swap[l], cpu_want[l]), f"swap-out layer {l}"
+        assert same_bits(w.kv_cache[l], gpu_c[l])
+    # swap the same blocks back in under other GPU block ids; ordered after the swap-out by r1's event
+    back = [20, 21, 22, 0]
+    w.swap_blocks(["r1"], dst_cpu, back, is_swap_in=True)
+    w.wait_for_all_swap_in()
+    torch.cuda.synchronize()
+    for l in range(L):
+        want = gpu_c[l].clone()
+        want[:, back] = gpu_c[l][:, src_gpu]
+        assert same_bits(w.kv_cache[l], want), f"swap-in layer {l}"
+    assert set(w.swap_event_table) == {"r1", "r2"}
+    w.clear_request_resource("r1")
+    assert set(w.swap_event_table) == {"r2"}
+    with pytest.raises(ValueError, match="Block count mismatch"):
+        w.swap_blocks(["r1"], [1, 2], [3], True)
+    with pytest.raises(IndexError):
+        w.swap_blocks(["r1"], [NBC], [3], True)
+    fresh = KVWorker(0, DEV, bs)
+    with pytest.raises(RuntimeError, match="not initialized"):
+        fresh.swap_blocks(["r"], [0], [0], True)
