@@ -460,7 +460,11 @@ __device__ __forceinline__ float half_bits_to_f32(uint32_t h) {
     return f16_bits_to_f32(h);
 }
 
-// 8 sixteen-bit values (one u32x4) -> 8 e4m3fn bytes (one u32x2), q = rne(x / scale)
+// 8 sixteen-bit values (one u32x4) -> 8 e4m3fn bytes (one u32x2), q = rne(x / scale).
+// The division is the compiler's correctly rounded IEEE sequence. A reciprocal plus one
+// fma correction step (exact for 2^-30 <= |scale| <= 2^30, verified on the device against
+// this division for every 16-bit input x 2^20 scales) was measured and gave no speed-up:
+// the kernel is bound by the 1 KiB row scatter, not by the arithmetic.
 template <int SRC_DTYPE>
 __device__ __forceinline__ u32x2 quant8(u32x4 in, float scale) {
   u32x2 out;
@@ -691,8 +695,10 @@ __global__ __launch_bounds__(kThreads) void emm_append_fp8_kernel(const AppendPa
       for (int r = 0; r < R; ++r)
         if (slot[r] >= 0) {
           char *dp = dst_base + slot[r] * row;
-          st_stream<u32x2, 1>(dp + e0, quant8<SRC_DTYPE>(a[r], scale));
-          if (e1 < row) st_stream<u32x2, 1>(dp + e1, quant8<SRC_DTYPE>(b[r], scale));
+          const u32x2 qa = quant8<SRC_DTYPE>(a[r], scale);
+          const u32x2 qb = quant8<SRC_DTYPE>(b[r], scale);
+          st_stream<u32x2, 1>(dp + e0, qa);
+          if (e1 < row) st_stream<u32x2, 1>(dp + e1, qb);
         }
       e0 += 1024;
       e1 += 1024;
@@ -826,10 +832,7 @@ int append_fp8(const void *const *k, const void *const *v, void *const *kc, void
   p.key_stride = ks;
   p.value_stride = vs;
   p.num_slots = num_slots;
-  // rows per wave: the conversion is arithmetic-heavy, two rows per wave keep more loads in
-  // flight per lane in a large launch; a small launch needs the extra workgroups of one row
-  int rows = (num_tokens * num_layers >= 100000) ? 2 : 1;
-  if (g_append_rows == 1 || g_append_rows == 2 || g_append_rows == 4) rows = g_append_rows;
+  const int rows = (g_append_rows == 1 || g_append_rows == 2 || g_append_rows == 4) ? g_append_rows : 1;
   dim3 grid = append_grid(num_tokens, num_layers, width == 8 ? rows : 4);
 #define EMM_FP8_LAUNCH(DT)                                                                  \
   if (width == 8) {                                                                         \

@@ -731,3 +731,32 @@ def test_swap_blocks_out_and_in():
     fresh = KVWorker(0, DEV, bs)
     with pytest.raises(RuntimeError, match="not initialized"):
         fresh.swap_blocks(["r"], [0], [0], True)
+
+
+def test_fp8_append_scale_range_paths():
+    """Extreme and awkward scales (powers of two far from 1, all-ones mantissas, a negative
+    scale, the smallest normal and the largest finite float): the quotient must be the one
+    correctly rounded fp32 division of the oracle for every bf16 and f16 input."""
+    import struct
+
+    def f32(bits):
+        return struct.unpack("<f", struct.pack("<I", bits))[0]
+
+    scales = [2.0 ** -30, 2.0 ** 30, 2.0 ** -31, 2.0 ** 31, 3.0e10, 1.0e-12, f32(0x3DFFFFFF), f32(0x3C7FFFFF),
+              f32(0x3F7FFFFF), -0.05, 0.013671875, 1.0 / 3.0, 448.0, f32(0x00800000), f32(0x7F7FFFFF)]
+    slots = torch.arange(64, device=DEV)
+    for dtype in (torch.bfloat16, torch.float16):
+        allx = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype)
+        key = allx.view(64, 8, 128).to(DEV)
+        for s in scales:
+            s32 = float(np.float32(s))
+            kc = torch.zeros((4, 16, 8, 128), dtype=torch.uint8, device=DEV)
+            vc = torch.zeros_like(kc)
+            sc = torch.tensor([s32], dtype=torch.float32, device=DEV)
+            cache_ops.reshape_and_cache_flash(key, key, kc, vc, slots, "fp8", sc, sc)
+            got = raw(kc)
+            want = orc.c_quant_fp8(allx, s32).reshape(-1)
+            bad = np.nonzero(got != want)[0]
+            assert bad.size == 0, f"{dtype} scale {s32!r}: {bad.size} mismatches, first input bits {bad[:6].tolist()} " \
+                                  f"got {got[bad[:6]].tolist()} want {want[bad[:6]].tolist()}"
+            assert (raw(vc) == want).all()
