@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--blocks", type=int, default=60000, help="pool size in blocks (BASELINE: 60000)")
+    ap.add_argument("--blocks", type=int, default=60000, help="pool size in blocks (the Qwen2-7B migration workload uses 60000)")
     ap.add_argument("--requests", type=int, default=32)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements (append, batched, copy)")
@@ -373,7 +373,7 @@ def append_bench(kv, NB, bs, H, D, cache_dtype_name, k_scales, v_scales, dev, T=
 
 
 def extended(dev):
-    """The two other BASELINE shapes at full size (run with --extended; needs the whole GPU):
+    """The two other target shapes at full size (run with --extended; needs the whole GPU):
     the fp8-e4m3 70B-class per-GPU shape and the elastic rebalancing of a ~200 GB pool."""
     from elasticmm_amd import kv_ops
     from elasticmm_amd.kv_ops import PoolView

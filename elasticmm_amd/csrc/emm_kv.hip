@@ -1,14 +1,16 @@
 // libemm_kv — KV-cache data-movement kernels for gfx950 (MI355X) behind the C ABI
 // declared in include/emm_kv.h.
 //
-// Everything here is HBM-bandwidth work: the kernels move 16 bytes per lane per
-// access, every wave touches 1 KiB of contiguous memory per instruction, all
-// loads of a tile are issued before the first store, and loads/stores are
-// non-temporal (streaming data is never re-read, so it should not displace
-// other lines in L2 / Infinity Cache). Block-table entries and slot-mapping
-// entries are wave-uniform: they are fetched once per wave on the scalar path
-// (or broadcast with readfirstlane) and all address arithmetic that depends on
-// them stays in scalar registers.
+// Everything here is HBM-bandwidth work. The shape every kernel follows was found
+// by measurement on MI355X: a 256-thread workgroup moves one 4 KiB tile, each lane
+// issues ONE 16-byte non-temporal load and ONE 16-byte store, every wave
+// instruction covers 1 KiB of contiguous memory, and stores are system-scope
+// write-through (sc0 sc1). Unrolled or persistent variants are slower on this part
+// (the memory counter of gfx9 retires loads and stores in order, so a lane that
+// loads after it has stored waits for a write acknowledgement). Block-table and
+// slot-mapping entries are wave-uniform: they are fetched once per wave and all
+// address arithmetic that depends on them stays in scalar registers; loads that do
+// not depend on them are issued before they are waited for.
 //
 // Pool layout (per layer): [num_kv, num_blocks, chunk] contiguous, where
 // chunk = block_size * num_kv_heads * head_dim elements.
@@ -50,18 +52,12 @@ int check_launch(const char *what) {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-template <int BYTES> struct VecOf;
-template <> struct VecOf<16> { typedef u32x4 type; };
-template <> struct VecOf<8> { typedef u32x2 type; };
-template <> struct VecOf<4> { typedef uint32_t type; };
-template <> struct VecOf<2> { typedef uint16_t type; };
-template <> struct VecOf<1> { typedef uint8_t type; };
-
 // Cache policies of the streaming accessors. Loads are always non-temporal.
 //   0  store nt                (compiler builtin)
 //   1  store sc0 sc1           (system-scope write-through)
 //   2  store sc0 sc1 nt
 //   3  plain load / plain store
+// (the block-move kernels instantiate 0 and 1; 2 and 3 exist for experiments)
 // The sc0/sc1 forms exist only as instruction modifiers, so 16-byte stores under
 // policies 1 and 2 are emitted with a one-line asm statement (a vector store).
 // Every pointer these kernels dereference is device (global) memory. Saying so in
@@ -265,21 +261,21 @@ __global__ __launch_bounds__(T) void emm_block_move_kernel(const MoveParams p) {
   store_tile<V, T, U, POLICY>(v, dst, limit);
 }
 
-// Launch variant of the 16-byte path: bits 0-3 vectors per lane (1, 2, 4),
-// bits 4-7 workgroup size code (0: 256, 1: 64), bits 8-11 cache policy + 1.
-// 0 selects the default.
+// Launch variant of the 16-byte path (benchmarks only): bits 0-3 vectors per lane
+// (1 or 4), bits 8-11 cache policy + 1 (policy 0: nt stores, 1: sc0 sc1 stores).
+// 0 selects the default: one vector per lane, sc0 sc1 stores. The sweep that chose
+// it also covered 64-thread workgroups, two vectors per lane and the sc0 sc1 nt /
+// plain policies; none was faster and they are no longer instantiated.
 int g_move_variant = 0;
 
 bool aligned(const void *p, int a) { return ((uintptr_t)p & (uintptr_t)(a - 1)) == 0; }
 
-template <typename V, int T, int U, bool SP, bool DP>
+template <typename V, int U, bool SP, bool DP>
 void launch_move_policy(const MoveParams &p, dim3 grid, int policy, hipStream_t s) {
-  switch (policy) {
-  case 1: emm_block_move_kernel<V, T, U, SP, DP, 1><<<grid, T, 0, s>>>(p); break;
-  case 2: emm_block_move_kernel<V, T, U, SP, DP, 2><<<grid, T, 0, s>>>(p); break;
-  case 3: emm_block_move_kernel<V, T, U, SP, DP, 3><<<grid, T, 0, s>>>(p); break;
-  default: emm_block_move_kernel<V, T, U, SP, DP, 0><<<grid, T, 0, s>>>(p); break;
-  }
+  if (policy == 1 && sizeof(V) == 16)
+    emm_block_move_kernel<V, kThreads, U, SP, DP, 1><<<grid, kThreads, 0, s>>>(p);
+  else
+    emm_block_move_kernel<V, kThreads, U, SP, DP, 0><<<grid, kThreads, 0, s>>>(p);
 }
 
 template <bool SP, bool DP>
@@ -289,16 +285,14 @@ int launch_move(MoveParams &p, int planes, int min_align, hipStream_t s, const c
   int vec = 16;
   while (vec > 1 && (p.chunk_bytes % vec != 0 || min_align % vec != 0)) vec >>= 1;
   if (vec == 8) vec = 4; // 8-byte lanes are not instantiated
-  int threads = 256, unroll = 1, policy = 1;
+  int unroll = 1, policy = 1;
   if (vec == 16 && g_move_variant > 0) {
-    const int u = g_move_variant & 0xf;
-    if (u == 1 || u == 2 || u == 4) unroll = u;
-    if (((g_move_variant >> 4) & 0xf) == 1) threads = 64;
+    if ((g_move_variant & 0xf) == 4) unroll = 4;
     const int pc = (g_move_variant >> 8) & 0xf;
-    if (pc >= 1 && pc <= 4) policy = pc - 1;
+    if (pc == 1 || pc == 2) policy = pc - 1;
   }
-  if (vec != 16) { threads = 256; unroll = 4; policy = 0; }
-  const int64_t tile_bytes = (int64_t)unroll * threads * vec;
+  if (vec != 16) { unroll = 4; policy = 0; } // rare unaligned shapes: narrower lanes, four per lane
+  const int64_t tile_bytes = (int64_t)unroll * kThreads * vec;
   const int64_t tpc = (p.chunk_bytes + tile_bytes - 1) / tile_bytes;
   if (tpc > 0x7fffffffLL)
     return fail(EMM_EINVAL, "%s: chunk of %lld bytes needs too many tiles", what, (long long)p.chunk_bytes);
@@ -311,24 +305,11 @@ int launch_move(MoveParams &p, int planes, int min_align, hipStream_t s, const c
     q.j_end = j0 + ny;
     dim3 grid((uint32_t)tpc, (uint32_t)ny, (uint32_t)planes);
     if (SP && DP) grid = dim3((uint32_t)tpc, (uint32_t)(planes * kRun), (uint32_t)((ny + kRun - 1) / kRun));
-    bool done = false;
-#define EMM_MOVE_CASE(VB, TT, UU)                                                           \
-  if (!done && vec == VB && threads == TT && unroll == UU) {                                \
-    launch_move_policy<typename VecOf<VB>::type, TT, UU, SP, DP>(q, grid, policy, s);       \
-    done = true;                                                                            \
-  }
-    EMM_MOVE_CASE(16, 256, 1)
-    EMM_MOVE_CASE(16, 256, 2)
-    EMM_MOVE_CASE(16, 256, 4)
-    EMM_MOVE_CASE(16, 64, 1)
-    EMM_MOVE_CASE(16, 64, 2)
-    EMM_MOVE_CASE(16, 64, 4)
-    // rare unaligned shapes: narrower lanes, one fixed tile shape
-    EMM_MOVE_CASE(4, 256, 4)
-    EMM_MOVE_CASE(2, 256, 4)
-    EMM_MOVE_CASE(1, 256, 4)
-#undef EMM_MOVE_CASE
-    if (!done) return fail(EMM_EINVAL, "%s: no kernel for vec=%d threads=%d unroll=%d", what, vec, threads, unroll);
+    if (vec == 16 && unroll == 1) launch_move_policy<u32x4, 1, SP, DP>(q, grid, policy, s);
+    else if (vec == 16) launch_move_policy<u32x4, 4, SP, DP>(q, grid, policy, s);
+    else if (vec == 4) launch_move_policy<uint32_t, 4, SP, DP>(q, grid, 0, s);
+    else if (vec == 2) launch_move_policy<uint16_t, 4, SP, DP>(q, grid, 0, s);
+    else launch_move_policy<uint8_t, 4, SP, DP>(q, grid, 0, s);
     const int rc = check_launch(what);
     if (rc != EMM_OK) return rc;
   }

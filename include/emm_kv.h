@@ -209,9 +209,10 @@ int emm_concat_rows(const void *const *srcs, const int64_t *nbytes, int n,
 int emm_stream_copy(const void *src, void *dst, int64_t nbytes,
                     emm_stream_t stream);
 
-/* Tuning hook: 0 = library default; otherwise selects a launch variant of the
- * block-move kernels (see emm_kv.hip). Process-wide, not thread-safe; meant
- * for benchmarks. Returns the previous value. */
+/* Tuning hook for benchmarks: 0 = library default. Bits 0-3: vectors per lane of
+ * the block-move kernels (1 or 4); bits 8-11: store policy + 1 (1: non-temporal,
+ * 2: sc0 sc1); bits 12-15: token rows per wave of the append kernels (1, 2, 4).
+ * Process-wide, not thread-safe. Returns the previous value. */
 int emm_set_move_variant(int variant);
 
 #ifdef __cplusplus

@@ -26,7 +26,7 @@ tests/test_oracle.py:
       reduces to a plain reshape, -1 rows leave the cache unchanged).
       The reference holds no golden vectors or tests for this path.
   fp8 quantise (append): c_quant_fp8 == torch's ``.to(torch.float8_e4m3fn)``
-      (the library routine BASELINE names) on all 65 536 bf16 inputs x 6 scales
+      (the library routine that defines the contract) on all 65 536 bf16 inputs x 6 scales
       and on the explicit known answers 448, 464, 465, 480, -1000, 2^-9, 2^-10,
       2^-10*1.0001, 17, 18, 19, inf (bytes 126,126,127,127,255,1,0,1,88,89,90,127);
       SHA-256 of each sweep committed under tests/golden/.

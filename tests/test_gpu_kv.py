@@ -2,7 +2,7 @@
 
 Bit-exact everywhere (byte moves and the fp8 cast alike): pools, transfer buffers
 and caches are compared as raw bit patterns. Small and medium shapes are compared
-with the oracle in full; the BASELINE-size shapes are checked through
+with the oracle in full; the full-size shapes (two 51 GiB pools) are checked through
 size-independent properties (every moved block equals its source, everything
 else keeps its canary) evaluated on the device with torch indexing as a second,
 independent implementation.
@@ -544,7 +544,7 @@ def test_worker_coordinated_pull_and_collective():
         dst.write_kv_blocks([1, 2], torch.zeros(shape, dtype=torch.bfloat16, device=DEV))
 
 
-# ------------------------------------------------------------------ BASELINE-size properties
+# ------------------------------------------------------------------ full-size properties
 def test_cfg2_full_size_migration_properties():
     """Qwen2-7B KV shape at full size: 28 x [2,60000,16,4,128] bf16 twice (2 x 51.3 GiB).
     Checked with torch's own device indexing as the second implementation."""
