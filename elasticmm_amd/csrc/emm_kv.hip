@@ -185,6 +185,7 @@ struct MoveParams {
   int64_t n;      // blocks per plane of the linear buffer
   int64_t j0;     // first block of this launch
   int64_t j_end;  // one past the last block of this launch
+  int32_t group_log2; // grouped order for moves with a linear side (0 = off)
   int64_t plane0; // first plane of this launch (linear side)
 };
 
@@ -213,6 +214,12 @@ __global__ __launch_bounds__(T) void emm_block_move_kernel(const MoveParams p) {
     uint32_t run = blockIdx.z + pl * (gridDim.z / (gridDim.y / kRun));
     if (run >= gridDim.z) run -= gridDim.z;
     j = p.j0 + (int64_t)run * kRun + (blockIdx.y % kRun);
+    if (j >= p.j_end) return;
+  } else if (p.group_log2 > 0) {
+    // groups of 2^group_log2 blocks per plane visit (y = plane * G + position, z = group)
+    const uint32_t G = 1u << p.group_log2;
+    pl = blockIdx.y >> p.group_log2;
+    j = p.j0 + ((int64_t)blockIdx.z << p.group_log2) + (blockIdx.y & (G - 1));
     if (j >= p.j_end) return;
   } else {
     pl = blockIdx.z;
@@ -305,6 +312,18 @@ int launch_move(MoveParams &p, int planes, int min_align, hipStream_t s, const c
     q.j_end = j0 + ny;
     dim3 grid((uint32_t)tpc, (uint32_t)ny, (uint32_t)planes);
     if (SP && DP) grid = dim3((uint32_t)tpc, (uint32_t)(planes * kRun), (uint32_t)((ny + kRun - 1) / kRun));
+    // Scatter from a linear buffer (unpack): visiting a plane for thousands of blocks in a row
+    // keeps all writes inside that plane's address window, which this memory system serves
+    // about 12 % slower than writes spread over the whole pool. Long tables are therefore
+    // walked in groups of 128 blocks per plane visit (y = plane * 128 + position, z = group);
+    // short tables already leave a plane after a few hundred blocks. Gathers (pack) measured
+    // faster in the plain order and keep it.
+    int glog = (!SP && DP && ny >= 1024) ? 7 : 0;
+    if ((g_move_variant >> 16) & 0xf) glog = ((g_move_variant >> 16) & 0xf) == 0xf ? 0 : (g_move_variant >> 16) & 0xf;
+    if (!(SP && DP) && glog > 0 && (planes << glog) <= kMaxGridY) {
+      q.group_log2 = glog;
+      grid = dim3((uint32_t)tpc, (uint32_t)(planes << glog), (uint32_t)((ny + (1 << glog) - 1) >> glog));
+    }
     if (vec == 16 && unroll == 1) launch_move_policy<u32x4, 1, SP, DP>(q, grid, policy, s);
     else if (vec == 16) launch_move_policy<u32x4, 4, SP, DP>(q, grid, policy, s);
     else if (vec == 4) launch_move_policy<uint32_t, 4, SP, DP>(q, grid, 0, s);
@@ -521,8 +540,10 @@ struct DequantParams {
   const float *v_scales;
   int64_t dst_num_blocks;
   int64_t chunk_elems; // fp8 bytes per chunk == elements
-  int64_t n;  // blocks per plane of the transfer buffer
-  int64_t j0; // first block of this launch
+  int64_t n;     // blocks per plane of the transfer buffer
+  int64_t j0;    // first block of this launch
+  int64_t j_end; // one past its last block
+  int32_t group_log2;
 };
 
 // One workgroup converts one tile of 4 KiB of fp8 bytes into 8 KiB. A wave owns 1 KiB of
@@ -534,8 +555,17 @@ template <int OUT_DTYPE>
 __global__ __launch_bounds__(kThreads) void emm_unpack_dequant_fp8_kernel(const DequantParams p) {
   constexpr int64_t TILE = (int64_t)kThreads * 16;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t j = p.j0 + blockIdx.y;
-  const uint32_t pl = blockIdx.z, l = pl >> 1, kv = pl & 1;
+  uint32_t pl;
+  int64_t j;
+  if (p.group_log2 > 0) { // long tables: groups of blocks per plane visit, as in the plain unpack
+    pl = blockIdx.y >> p.group_log2;
+    j = p.j0 + ((int64_t)blockIdx.z << p.group_log2) + (blockIdx.y & ((1u << p.group_log2) - 1));
+    if (j >= p.j_end) return;
+  } else {
+    pl = blockIdx.z;
+    j = p.j0 + blockIdx.y;
+  }
+  const uint32_t l = pl >> 1, kv = pl & 1;
   const int64_t chunk = p.chunk_elems;
   const int64_t off0 = (int64_t)blockIdx.x * TILE + wave * 1024 + lane * 8;
   const int64_t off1 = off0 + 512;
@@ -708,6 +738,9 @@ __global__ __launch_bounds__(kThreads) void emm_append_fp8_kernel(const AppendPa
   }
 }
 
+// A walk that cycles through the planes in short runs of tokens (as the long unpack does with
+// blocks) was measured for the whole-step launch and made no difference: a plane is left after
+// 8 MiB of rows anyway.
 dim3 append_grid(int64_t num_tokens, int num_layers, int rows_per_wave) {
   const int64_t rows_per_group = (int64_t)kWavesPerGroup * rows_per_wave;
   return dim3((uint32_t)((num_tokens + rows_per_group - 1) / rows_per_group), 2, (uint32_t)num_layers);
@@ -876,7 +909,7 @@ int emm_abi_version(void) { return EMM_KV_ABI_VERSION; }
 
 int emm_set_move_variant(int variant) {
   const int old = g_move_variant | (g_append_rows << 12);
-  g_move_variant = variant & 0xfff;
+  g_move_variant = variant & 0xf0fff;
   g_append_rows = (variant >> 12) & 0xf; // rows per wave of the append kernels
   return old;
 }
@@ -980,7 +1013,13 @@ int emm_kv_unpack_dequant_fp8(void *const *layer_ptrs, int num_layers, int64_t n
   for (int64_t j0 = 0; j0 < n; j0 += kMaxGridY) {
     const int64_t ny = (n - j0 < kMaxGridY) ? (n - j0) : kMaxGridY;
     p.j0 = j0;
+    p.j_end = j0 + ny;
+    p.group_log2 = 0;
     dim3 grid((uint32_t)tpc, (uint32_t)ny, (uint32_t)(2 * num_layers));
+    if (ny >= 1024 && ((2 * num_layers) << 7) <= kMaxGridY) {
+      p.group_log2 = 7;
+      grid = dim3((uint32_t)tpc, (uint32_t)((2 * num_layers) << 7), (uint32_t)((ny + 127) >> 7));
+    }
     if (out_dtype == EMM_DTYPE_BF16)
       emm_unpack_dequant_fp8_kernel<EMM_DTYPE_BF16><<<grid, kThreads, 0, as_stream(stream)>>>(p);
     else
