@@ -1,0 +1,232 @@
+"""KVTransferManager — the caller of the KV data path, same call shape as the reference's
+``V0KVTransferManager`` (elasticmm/engine/v0/kv_transfer.py).
+
+What is kept: the method enum (:14-19), the rank-keyed worker registry (:100-168), the
+coroutine ``transfer_kv_cache(request_id, src_rank, dst_rank, src_blocks, dst_blocks) -> bool``
+that dispatches on the method (:224-262), the statistics that leave out the first (cold-start)
+transfer (:82-86, :506-515, :843-859), the metrics callback, and the optional batching that
+concatenates several requests' block lists into one transfer (:341-418).
+
+What is different: workers are ``KVWorker`` objects in this process, not Ray actors, so the calls
+are plain method calls. The reference's batching path is disabled in the product and its enqueue
+code refers to undefined names (:439); here the queue is keyed by (src_rank, dst_rank) and a flush
+moves the merged tables with one pack launch and one unpack launch.
+"""
+from __future__ import annotations
+
+import time
+from enum import Enum
+from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
+
+
+class TransferMethod(Enum):
+    """kv_transfer.py:14-19. CUDA_IPC is the reference's placeholder for a fused device-side
+    migration op; here it is the fused same-device ``kv_migrate`` (no transfer buffer)."""
+    CUDA_IPC = "cuda_ipc"
+    NCCL = "nccl"
+    P2P_COPY = "p2p_copy"
+    STAGED_COPY = "staged_copy"
+
+
+class KVTransferManager:
+    def __init__(self, transfer_method: TransferMethod = TransferMethod.P2P_COPY, enable_batching: bool = False,
+                 batch_size: int = 3, batch_timeout: float = 0.005,
+                 metrics_callback: Optional[Callable[..., None]] = None):
+        self.transfer_method = transfer_method
+        self.enable_batching = enable_batching
+        self.metrics_callback = metrics_callback
+        self.worker_registry: Dict[int, Any] = {}
+        self.rank_to_stage: Dict[int, str] = {}
+        self._transfer_queue: Dict[Tuple[int, int], List[Tuple[str, List[int], List[int]]]] = {}
+        self._batch_flush_threshold = batch_size
+        self._batch_flush_timeout = batch_timeout
+        self._last_flush_time: Dict[Tuple[int, int], float] = {}
+        # statistics exclude the first transfer (cold start), as in the reference
+        self.transfer_count = 0
+        self.total_transfer_time = 0.0
+        self.total_bytes_transferred = 0
+        self.first_transfer_done = False
+
+    # ----- registry (kv_transfer.py:113-168) ---------------------------------
+    def register_workers(self, stage: str, workers: Sequence[Any], global_ranks: Sequence[int]) -> None:
+        for worker, rank in zip(workers, global_ranks):
+            if worker is not None and rank >= 0:
+                self.register_worker(rank, worker, stage)
+
+    def register_worker(self, global_rank: int, worker: Any, stage: str) -> None:
+        self.worker_registry[global_rank] = worker
+        self.rank_to_stage[global_rank] = stage.lower()
+
+    def unregister_worker(self, global_rank: int) -> None:
+        self.worker_registry.pop(global_rank, None)
+        self.rank_to_stage.pop(global_rank, None)
+
+    def update_worker_stage(self, global_rank: int, new_stage: str) -> None:
+        if global_rank not in self.worker_registry:
+            print(f"[KVTransferManager] Warning: Rank {global_rank} not registered")
+            return
+        self.rank_to_stage[global_rank] = new_stage.lower()
+
+    # ----- transfer (kv_transfer.py:224-262) ----------------------------------
+    async def transfer_kv_cache(self, request_id: str, src_rank: int, dst_rank: int, src_blocks: List[int],
+                                dst_blocks: List[int]) -> bool:
+        return self.transfer_kv_cache_sync(request_id, src_rank, dst_rank, src_blocks, dst_blocks)
+
+    def transfer_kv_cache_sync(self, request_id: str, src_rank: int, dst_rank: int, src_blocks: List[int],
+                               dst_blocks: List[int]) -> bool:
+        if self.transfer_method == TransferMethod.NCCL:
+            if self.enable_batching:
+                return self._enqueue(request_id, src_rank, dst_rank, src_blocks, dst_blocks)
+            return self._transfer_via_p2p(request_id, src_rank, src_blocks, dst_rank, dst_blocks)
+        if self.transfer_method == TransferMethod.P2P_COPY:
+            return self._transfer_via_p2p_copy(request_id, src_rank, src_blocks, dst_rank, dst_blocks)
+        if self.transfer_method == TransferMethod.CUDA_IPC:
+            return self._transfer_via_device_migrate(request_id, src_rank, src_blocks, dst_rank, dst_blocks)
+        return False
+
+    def _workers(self, src_rank: int, dst_rank: int):
+        src_worker = self.worker_registry.get(src_rank)
+        dst_worker = self.worker_registry.get(dst_rank)
+        if src_worker is None or dst_worker is None:
+            print(f"[KVTransferManager] Workers not found: src_rank={src_rank}, dst_rank={dst_rank}")
+            return None, None
+        return src_worker, dst_worker
+
+    def _account(self, elapsed: float, nbytes: int, num_blocks: int, transfers: int = 1) -> None:
+        if not self.first_transfer_done:
+            self.first_transfer_done = True
+        else:
+            self.transfer_count += transfers
+            self.total_transfer_time += elapsed
+            self.total_bytes_transferred += nbytes
+        if self.metrics_callback:
+            self.metrics_callback(transfer_time_sec=elapsed, num_blocks=num_blocks)
+
+    def _transfer_via_p2p(self, request_id, src_rank, src_blocks, dst_rank, dst_blocks) -> bool:
+        """kv_transfer.py:420-524: one coordinated call on the destination worker."""
+        src_worker, dst_worker = self._workers(src_rank, dst_rank)
+        if src_worker is None:
+            return False
+        try:
+            start_time = time.perf_counter()
+            recv_result = dst_worker.p2p_coordinated_transfer_kv(src_worker, src_rank, src_blocks, dst_blocks,
+                                                                 timeout=10.0)
+            elapsed = time.perf_counter() - start_time
+            if "error" in recv_result:
+                print(f"[KVTransferManager] transfer failed for {request_id}: {recv_result.get('error')}")
+                return False
+            nbytes = recv_result.get("bytes", 0)
+            if nbytes == 0:
+                return False
+            self._account(elapsed, nbytes, len(src_blocks))
+            return True
+        except Exception as e:  # pre-flight errors of the worker are reported as a failed transfer
+            print(f"[KVTransferManager] P2P transfer failed: {e}")
+            return False
+
+    def _transfer_via_p2p_copy(self, request_id, src_rank, src_blocks, dst_rank, dst_blocks) -> bool:
+        """kv_transfer.py:693-750: extract on the source, write on the destination."""
+        src_worker, dst_worker = self._workers(src_rank, dst_rank)
+        if src_worker is None:
+            return False
+        try:
+            start_time = time.perf_counter()
+            kv_data = src_worker.extract_kv_blocks(src_blocks)
+            dst_worker.write_kv_blocks(dst_blocks, kv_data)
+            elapsed = time.perf_counter() - start_time
+            self.transfer_count += 1
+            if self.metrics_callback:
+                self.metrics_callback(transfer_time_sec=elapsed, num_blocks=len(src_blocks))
+            return True
+        except Exception as e:
+            print(f"[KVTransferManager] P2P copy failed: {e}")
+            return False
+
+    def _transfer_via_device_migrate(self, request_id, src_rank, src_blocks, dst_rank, dst_blocks) -> bool:
+        """The slot the reference reserves for a fused device-side op (kv_transfer.py:303-331,
+        ``block_migration_ops.migrate_blocks``): pool-to-pool in one launch, both pools on one device."""
+        from . import kv_ops
+
+        src_worker, dst_worker = self._workers(src_rank, dst_rank)
+        if src_worker is None:
+            return False
+        try:
+            start_time = time.perf_counter()
+            kv_ops.kv_migrate(src_worker.pool, src_blocks, dst_worker.pool, dst_blocks)
+            elapsed = time.perf_counter() - start_time
+            self.transfer_count += 1
+            if self.metrics_callback:
+                self.metrics_callback(transfer_time_sec=elapsed, num_blocks=len(src_blocks))
+            return True
+        except Exception as e:
+            print(f"[KVTransferManager] device migrate failed: {e}")
+            return False
+
+    # ----- batching (kv_transfer.py:341-418, :434-462) -------------------------
+    def _enqueue(self, request_id, src_rank, dst_rank, src_blocks, dst_blocks) -> bool:
+        key = (src_rank, dst_rank)
+        if key not in self._transfer_queue:
+            self._transfer_queue[key] = []
+            self._last_flush_time[key] = time.perf_counter()
+        self._transfer_queue[key].append((request_id, list(src_blocks), list(dst_blocks)))
+        now = time.perf_counter()
+        if (len(self._transfer_queue[key]) >= self._batch_flush_threshold
+                or now - self._last_flush_time[key] >= self._batch_flush_timeout):
+            self._last_flush_time[key] = now
+            return self.flush_transfer_batch(src_rank, dst_rank)
+        return True  # queued, flushed later
+
+    def flush_transfer_batch(self, src_rank: int, dst_rank: int) -> bool:
+        """Merge the queued requests' tables and move them with one send / one receive."""
+        key = (src_rank, dst_rank)
+        transfers = self._transfer_queue.get(key) or []
+        if not transfers:
+            return True
+        self._transfer_queue[key] = []
+        all_src_blocks: List[int] = []
+        all_dst_blocks: List[int] = []
+        for _, src_blocks, dst_blocks in transfers:
+            all_src_blocks.extend(src_blocks)
+            all_dst_blocks.extend(dst_blocks)
+        src_worker, dst_worker = self._workers(src_rank, dst_rank)
+        if src_worker is None:
+            return False
+        try:
+            start_time = time.perf_counter()
+            send_result = src_worker.p2p_send_kv(dst_rank, all_src_blocks)
+            if "error" in send_result:
+                return False
+            recv_result = dst_worker.p2p_recv_kv(src_rank, all_dst_blocks)
+            if "error" in recv_result:
+                return False
+            elapsed = time.perf_counter() - start_time
+            nbytes = recv_result.get("bytes", 0)
+            if nbytes == 0:
+                return False
+            self.transfer_count += len(transfers)
+            self.total_transfer_time += elapsed
+            self.total_bytes_transferred += nbytes
+            return True
+        except Exception as e:
+            print(f"[KVTransferManager] Batched transfer failed: {e}")
+            return False
+
+    def flush_all(self) -> bool:
+        ok = True
+        for src_rank, dst_rank in list(self._transfer_queue):
+            ok = self.flush_transfer_batch(src_rank, dst_rank) and ok
+        return ok
+
+    # ----- statistics (kv_transfer.py:843-859) ---------------------------------
+    def get_stats(self) -> Dict[str, Any]:
+        return {
+            "transfer_count": self.transfer_count,
+            "total_transfer_time": self.total_transfer_time,
+            "total_bytes_transferred": self.total_bytes_transferred,
+            "avg_transfer_time": (self.total_transfer_time / self.transfer_count if self.transfer_count > 0 else 0.0),
+        }
+
+    def reset_stats(self) -> None:
+        self.transfer_count = 0
+        self.total_transfer_time = 0.0
+        self.total_bytes_transferred = 0

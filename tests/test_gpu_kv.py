@@ -760,3 +760,25 @@ def test_fp8_append_scale_range_paths():
             assert bad.size == 0, f"{dtype} scale {s32!r}: {bad.size} mismatches, first input bits {bad[:6].tolist()} " \
                                   f"got {got[bad[:6]].tolist()} want {want[bad[:6]].tolist()}"
             assert (raw(vc) == want).all()
+
+
+# ------------------------------------------------------------------ transfer manager on real workers
+def test_transfer_manager_methods_move_the_same_bytes():
+    from elasticmm_amd.kv_transfer import KVTransferManager, TransferMethod
+
+    si, di = [3, 30, 7, 12], [0, 1, 29, 15]
+    for method, batching in ((TransferMethod.P2P_COPY, False), (TransferMethod.NCCL, False),
+                             (TransferMethod.CUDA_IPC, False), (TransferMethod.NCCL, True)):
+        src, dst = make_pair()
+        m = KVTransferManager(method, enable_batching=batching, batch_size=2, batch_timeout=1e9)
+        m.register_workers("prefill", [src], [0])
+        m.register_workers("decoding", [dst], [1])
+        if batching:
+            assert m.transfer_kv_cache_sync("a", 0, 1, si[:2], di[:2]) is True
+            assert m.transfer_kv_cache_sync("b", 0, 1, si[2:], di[2:]) is True     # reaches the batch size: flush
+            assert m.get_stats()["transfer_count"] == 2
+        else:
+            assert m.transfer_kv_cache_sync("a", 0, 1, si, di) is True
+        torch.cuda.synchronize()
+        check_moved(src, dst, si, di)
+        assert m.transfer_kv_cache_sync("bad", 0, 1, [999], [0]) is (True if batching else False)

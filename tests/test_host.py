@@ -97,3 +97,80 @@ def test_block_manager_free_list_order():
         bm.allocate_blocks("d", 5)
     ids = bm.get_block_table("b") + bm.get_block_table("c")
     assert len(set(ids)) == len(ids)
+
+
+# ------------------------------------------------------------------ transfer manager (fake workers)
+class _FakeWorker:
+    def __init__(self, rank, fail=False):
+        self.rank, self.fail, self.calls = rank, fail, []
+
+    def extract_kv_blocks(self, blocks):
+        self.calls.append(("extract", list(blocks)))
+        return ("data", list(blocks))
+
+    def write_kv_blocks(self, blocks, data):
+        self.calls.append(("write", list(blocks), data))
+
+    def p2p_coordinated_transfer_kv(self, src, src_rank, src_blocks, dst_blocks, timeout=10.0):
+        self.calls.append(("coord", src_rank, list(src_blocks), list(dst_blocks), timeout))
+        if self.fail:
+            return {"error": "boom", "bytes": 0, "blocks": 0}
+        return {"bytes": 100 * len(dst_blocks), "blocks": len(dst_blocks)}
+
+    def p2p_send_kv(self, dst_rank, blocks):
+        self.calls.append(("send", dst_rank, list(blocks)))
+        return {"bytes": 100 * len(blocks), "blocks": len(blocks)}
+
+    def p2p_recv_kv(self, src_rank, blocks):
+        self.calls.append(("recv", src_rank, list(blocks)))
+        return {"bytes": 100 * len(blocks), "blocks": len(blocks)}
+
+
+def test_transfer_manager_dispatch_stats_and_batching():
+    import asyncio
+
+    from elasticmm_amd.kv_transfer import KVTransferManager, TransferMethod
+
+    seen = []
+    m = KVTransferManager(TransferMethod.NCCL, metrics_callback=lambda **kw: seen.append(kw))
+    a, b = _FakeWorker(0), _FakeWorker(1)
+    m.register_workers("Prefill", [a, None], [0, -1])
+    m.register_worker(1, b, "DECODING")
+    assert m.rank_to_stage == {0: "prefill", 1: "decoding"}
+    assert asyncio.run(m.transfer_kv_cache("r0", 0, 1, [1, 2], [7, 8])) is True
+    assert b.calls[-1] == ("coord", 0, [1, 2], [7, 8], 10.0)
+    # the first transfer is the cold start: counted by the callback, not by the statistics
+    assert m.get_stats()["transfer_count"] == 0 and len(seen) == 1 and seen[0]["num_blocks"] == 2
+    assert m.transfer_kv_cache_sync("r1", 0, 1, [3], [9]) is True
+    st = m.get_stats()
+    assert st["transfer_count"] == 1 and st["total_bytes_transferred"] == 100 and st["avg_transfer_time"] >= 0.0
+    assert m.transfer_kv_cache_sync("r2", 0, 5, [3], [9]) is False            # unknown rank
+    b.fail = True
+    assert m.transfer_kv_cache_sync("r3", 0, 1, [3], [9]) is False            # error dict -> False
+    m.reset_stats()
+    assert m.get_stats()["transfer_count"] == 0
+    m.update_worker_stage(1, "Prefill")
+    assert m.rank_to_stage[1] == "prefill"
+    m.unregister_worker(1)
+    assert 1 not in m.worker_registry
+
+    # p2p_copy: extract on the source, write on the destination
+    m2 = KVTransferManager(TransferMethod.P2P_COPY)
+    a, b = _FakeWorker(0), _FakeWorker(1)
+    m2.register_workers("prefill", [a, b], [0, 1])
+    assert m2.transfer_kv_cache_sync("r", 0, 1, [4, 5], [6, 7]) is True
+    assert a.calls == [("extract", [4, 5])] and b.calls == [("write", [6, 7], ("data", [4, 5]))]
+    assert m2.get_stats()["transfer_count"] == 1
+    assert KVTransferManager(TransferMethod.STAGED_COPY).transfer_kv_cache_sync("r", 0, 1, [1], [2]) is False
+
+    # batching: three requests are merged into one send / one recv with concatenated tables
+    m3 = KVTransferManager(TransferMethod.NCCL, enable_batching=True, batch_size=3, batch_timeout=1e9)
+    a, b = _FakeWorker(0), _FakeWorker(1)
+    m3.register_workers("prefill", [a, b], [0, 1])
+    assert m3.transfer_kv_cache_sync("q0", 0, 1, [1, 2], [11, 12]) is True and not a.calls
+    assert m3.transfer_kv_cache_sync("q1", 0, 1, [3], [13]) is True and not a.calls
+    assert m3.transfer_kv_cache_sync("q2", 0, 1, [4, 5], [14, 15]) is True
+    assert a.calls == [("send", 1, [1, 2, 3, 4, 5])] and b.calls == [("recv", 0, [11, 12, 13, 14, 15])]
+    assert m3.get_stats()["transfer_count"] == 3 and m3.get_stats()["total_bytes_transferred"] == 500
+    assert m3.transfer_kv_cache_sync("q3", 0, 1, [6], [16]) is True and len(a.calls) == 1
+    assert m3.flush_all() is True and a.calls[-1] == ("send", 1, [6])
