@@ -321,7 +321,65 @@ def secondary(src_w, dst_w, dev_tables, payload, L, bs, H, D, NB, dev):
         med, mn = timed(lambda: kv_ops.copy_blocks(sp, mapping), 10)
         out["copy_blocks_GBps"] = round(2 * P * L * 2 * chunk / (med * 1e-3) / 1e9, 1)
     out["append"] = append_bench(src_w.kv_cache, NB, bs, H, D, torch.bfloat16, None, None, dev)
+    out["append_paged_layout"] = paged_append_bench(src_w.kv_cache, NB, bs, H, D, dev)
     return out
+
+
+def paged_append_bench(kv, NB, bs, H, D, dev, T=8448, decode=256):
+    """The same step appended into the paged-attention layout (key [NB,H,D/8,bs,8], value [NB,H,D,bs],
+    viewed over the same pool memory): `decode` single tokens in random blocks, then one prompt of
+    T - decode tokens that fills blocks in order (its blocks start off the 16-token grid of the token
+    list). Bytes: 2 x 2 x row per token, as for the flash layout."""
+    from elasticmm_amd import cache_ops
+
+    L = len(kv)
+    x = 16 // kv[0].element_size()
+    g = torch.Generator(device=dev).manual_seed(4)
+    blocks = torch.randperm(NB, device=dev, generator=g)
+    dec = blocks[:decode] * bs + torch.randint(bs, (decode,), device=dev, generator=g)
+    nb_prompt = (T - decode + bs - 1) // bs + 1
+    prompt = (blocks[decode:decode + nb_prompt, None] * bs + torch.arange(bs, device=dev)[None, :]).reshape(-1)
+    first = bs - 5  # the prompt resumes 5 slots before a block boundary
+    slots = torch.cat([dec, prompt[first:first + T - decode]]).contiguous()
+    keys = [torch.randn((T, H, D), device=dev, generator=g).to(torch.bfloat16) for _ in range(L)]
+    values = [torch.randn((T, H, D), device=dev, generator=g).to(torch.bfloat16) for _ in range(L)]
+    kcs = [kv[l][0].view(NB, H, D // x, bs, x) for l in range(L)]
+    vcs = [kv[l][1].view(NB, H, D, bs) for l in range(L)]
+    step_bytes = L * (T * 2 * H * D * 2 * 2 + 8 * T)
+
+    def per_layer():
+        for l in range(L):
+            cache_ops.reshape_and_cache(keys[l], values[l], kcs[l], vcs[l], slots, "auto")
+
+    def entry(ms):
+        return {"tokens_per_s": round(T / (ms * 1e-3)), "ms_per_step": round(ms, 4),
+                "GBps": round(step_bytes / (ms * 1e-3) / 1e9, 1)}
+
+    res = {"T": T, "decode_tokens": decode, "layers": L, "algorithmic_bytes_per_step": step_bytes}
+    med, _ = timed(per_layer, 20)
+    res["per_layer_calls_eager"] = entry(med)
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        per_layer()
+    torch.cuda.current_stream().wait_stream(side)
+    with torch.cuda.graph(graph):
+        per_layer()
+    med, _ = timed(graph.replay, 20)
+    res["per_layer_calls_hip_graph"] = entry(med)
+    plan = cache_ops.paged_layered_append(keys, values, kcs, vcs)
+    med, _ = timed(lambda: plan(slots), 20)
+    res["one_launch_all_layers"] = entry(med)
+    # a decode-only step: every token alone in its block (each 2-byte V element and each 16-byte K piece
+    # lands in a cache line of its own, so the memory system rewrites the token's whole block region)
+    Td = 256
+    dplan = cache_ops.paged_layered_append([k[:Td] for k in keys], [v[:Td] for v in values], kcs, vcs)
+    dslots = dec[:Td].contiguous() if decode >= Td else slots[:Td].contiguous()
+    med, _ = timed(lambda: dplan(dslots), 20)
+    res["decode_only_256_tokens_one_launch"] = {"tokens_per_s": round(Td / (med * 1e-3)), "ms_per_step": round(med, 4),
+                                                "GBps": round(L * Td * 2 * H * D * 4 / (med * 1e-3) / 1e9, 1)}
+    return res
 
 
 def append_bench(kv, NB, bs, H, D, cache_dtype_name, k_scales, v_scales, dev, T=8448):

@@ -1,4 +1,4 @@
-"""vLLM-shaped cache operators: ``reshape_and_cache_flash`` and ``copy_blocks``.
+"""vLLM-shaped cache operators: ``reshape_and_cache_flash``, ``reshape_and_cache`` and ``copy_blocks``.
 
 The reference reaches both inside vLLM (``vllm>=0.10.1``, V0 engine): the append
 from ``model_runner.execute_model`` (elasticmm/engine/v0/worker_steps.py:281, :438)
@@ -36,6 +36,24 @@ def reshape_and_cache_flash(key: torch.Tensor, value: torch.Tensor, key_cache: t
         raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
 
 
+def reshape_and_cache(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
+                      slot_mapping: torch.Tensor, kv_cache_dtype: str = "auto",
+                      k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None) -> None:
+    """The append of vLLM's PagedAttention backends (its default attention path on ROCm): key, value
+    ``[num_tokens, num_heads, head_size]``; key_cache ``[num_blocks, num_heads, head_size // x, block_size, x]``,
+    value_cache ``[num_blocks, num_heads, head_size, block_size]``, x = 16 // cache element size."""
+    if kv_cache_dtype == "auto":
+        if key_cache.element_size() != key.element_size():
+            raise ValueError("kv_cache_dtype='auto' needs a cache of the key's element size")
+        kv_ops.reshape_and_cache_paged(key, value, key_cache, value_cache, slot_mapping)
+    elif kv_cache_dtype in ("fp8", "fp8_e4m3"):
+        if key_cache.element_size() != 1:
+            raise ValueError("fp8 KV cache must be a 1-byte tensor (float8_e4m3fn or uint8)")
+        kv_ops.reshape_and_cache_paged(key, value, key_cache, value_cache, slot_mapping, k_scale, v_scale)
+    else:
+        raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
+
+
 def reshape_and_cache_flash_layers(keys: Sequence[torch.Tensor], values: Sequence[torch.Tensor],
                                    kv_caches: Sequence[torch.Tensor], slot_mapping: torch.Tensor,
                                    kv_cache_dtype: str = "auto", k_scales=None, v_scales=None) -> None:
@@ -60,6 +78,18 @@ def layered_append(keys: Sequence[torch.Tensor], values: Sequence[torch.Tensor],
         return kv_ops.LayeredAppend(keys, values, key_caches, value_caches)
     if kv_cache_dtype in ("fp8", "fp8_e4m3"):
         return kv_ops.LayeredAppend(keys, values, key_caches, value_caches, k_scales, v_scales)
+    raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
+
+
+def paged_layered_append(keys: Sequence[torch.Tensor], values: Sequence[torch.Tensor],
+                         key_caches: Sequence[torch.Tensor], value_caches: Sequence[torch.Tensor],
+                         kv_cache_dtype: str = "auto", k_scales=None, v_scales=None) -> kv_ops.PagedLayeredAppend:
+    """The prepared whole-step append for the paged-attention layout: ``key_caches[l]`` is
+    ``[NB, H, D // x, bs, x]``, ``value_caches[l]`` ``[NB, H, D, bs]``; ``plan(slot_mapping)`` is one launch."""
+    if kv_cache_dtype == "auto":
+        return kv_ops.PagedLayeredAppend(keys, values, key_caches, value_caches)
+    if kv_cache_dtype in ("fp8", "fp8_e4m3"):
+        return kv_ops.PagedLayeredAppend(keys, values, key_caches, value_caches, k_scales, v_scales)
     raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
 
 

@@ -860,6 +860,274 @@ int append_fp8(const void *const *k, const void *const *v, void *const *kc, void
 }
 
 // ----------------------------------------------------------------------------
+// reshape_and_cache, paged-attention layout: the one place where source and
+// destination layouts transpose, staged through LDS
+// ----------------------------------------------------------------------------
+// key_cache   [num_blocks, num_heads, head_size / x, block_size, x]   x = 16 / cache element bytes
+// value_cache [num_blocks, num_heads, head_size, block_size]
+// key / value [num_tokens, num_heads * head_size] (row stride given)
+// For one block the K region is (row_elems / x) groups of [block_size][x] = block_size * 16 bytes,
+// the V region is row_elems runs of block_size elements. A token contributes one 16-byte piece to
+// every K group and one element to every V run, so tokens that fill a block in order produce
+// contiguous output; a single token produces 16-byte (K) and element-sized (V) stores at a stride
+// of block_size * 16 bytes resp. block_size elements.
+struct PagedParams {
+  const char *key[EMM_MAX_LAYERS];
+  const char *value[EMM_MAX_LAYERS];
+  char *key_cache[EMM_MAX_LAYERS];
+  char *value_cache[EMM_MAX_LAYERS];
+  const int64_t *slot_mapping;
+  const float *k_scales; // fp8 cache only: one float per layer
+  const float *v_scales;
+  int64_t num_tokens;
+  int64_t row_elems; // num_heads * head_size
+  int64_t key_stride; // elements
+  int64_t value_stride;
+  int64_t num_blocks;
+  int32_t block_size;
+  int32_t vec_src; // 1: sources allow 16-byte loads
+};
+
+constexpr int kPagedTokens = 16; // tokens per tile: the tile owns the runs that start in it
+constexpr int kPagedRows = 32;   // LDS rows: an owned run may reach 15 tokens past the tile
+constexpr int kPagedSeg = 256;   // row elements per tile
+
+// One workgroup transposes the rows of up to 31 tokens x up to 256 row elements of K or V.
+//
+// Runs. Consecutive tokens with consecutive slots inside one 16-slot-aligned window of a block
+// form a run (at most 16 tokens). A run belongs to the tile its first token lies in, so a tile
+// of 16 tokens owns runs that may extend up to 15 tokens into the next tile, and leaves the
+// head of a run that started in the previous tile to that tile: prompts written in order give
+// whole 16-token runs no matter where they start in the token list. Wave 0 finds the runs from
+// the 32 slots after the tile start with two ballots and writes a compact list of the owned
+// tokens (block, offset, token) to LDS.
+// Phase 1: coalesced 16-byte loads of the owned source rows (quantised to e4m3fn here when the
+// cache is fp8) into LDS, rows padded by 16 bytes so that a column walk touches every bank once.
+// Phase 2, K: lane q handles (group q / 16, owned token q % 16): one 16-byte LDS read, one
+// 16-byte store; 16 neighbouring lanes cover one group, so a run of n tokens gives n * 16
+// contiguous bytes per group and a whole block 16 KiB.
+// Phase 2, V: for a whole run of 16 tokens (at most one per tile) lane q gathers one 16-byte
+// piece of the run's [element][16 tokens] region from a column of the tile (8 or 16
+// element-sized LDS reads); the other owned tokens are stored one element per lane, token
+// fastest, which the memory pipeline merges where tokens have neighbouring slots.
+// grid: x = token tiles, y = 2 * row segments (bit 0: K | V), z = layers.
+template <int CE, int SRC_DTYPE>
+__global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(const PagedParams p) {
+  constexpr int X = 16 / CE;               // elements per 16-byte piece of the cache
+  constexpr int ROW = kPagedSeg * CE + 16; // LDS row stride in bytes
+  __shared__ __attribute__((aligned(16))) char tile[kPagedRows * ROW];
+  __shared__ int64_t s_blk[kPagedRows];
+  __shared__ int32_t s_off[kPagedRows];
+  __shared__ int32_t s_tok[kPagedRows];
+  __shared__ int32_t s_count; // owned tokens
+  __shared__ int32_t s_whole; // position of the whole run in the owned list, or -1
+  const int tid = threadIdx.x;
+  const uint32_t kv = blockIdx.y & 1u, seg = blockIdx.y >> 1;
+  const int64_t t0 = (int64_t)blockIdx.x * kPagedTokens;
+  const int64_t e0 = (int64_t)seg * kPagedSeg;
+  const int64_t left = p.row_elems - e0;
+  const int seg_elems = left < kPagedSeg ? (int)left : kPagedSeg; // multiple of X
+  const uint32_t l = blockIdx.z;
+  const char *src = kv == 0 ? p.key[l] : p.value[l];
+  char *cache = kv == 0 ? p.key_cache[l] : p.value_cache[l];
+  const int64_t stride = kv == 0 ? p.key_stride : p.value_stride;
+  const int bs = p.block_size;
+
+  float scale = 1.0f;
+  if constexpr (CE == 1) scale = kv == 0 ? p.k_scales[l] : p.v_scales[l];
+
+  // ---- phase 0 (wave 0): runs and the list of owned tokens ----
+  if (tid < 64) {
+    const int i = tid;
+    const int64_t t = t0 + i;
+    int64_t s = -1, prev = -1;
+    if (i < kPagedRows && t < p.num_tokens) {
+      s = p.slot_mapping[t];
+      if (t > 0) prev = p.slot_mapping[t - 1];
+    }
+    const bool valid = s >= 0 && s < p.num_blocks * bs;
+    int64_t blk = 0;
+    int32_t off = 0;
+    if (valid) {
+      blk = s / bs;
+      off = (int32_t)(s - blk * bs);
+    }
+    const bool cont = valid && s == prev + 1 && (off & 15) != 0; // continues the previous token's run
+    const uint64_t starts = __ballot(!cont); // bit j: token j starts a run or is skipped (lanes >= 32: set)
+    const uint64_t below = starts & ((2ull << i) - 1ull);
+    const int head = below ? 63 - __builtin_clzll(below) : -1; // first token of this token's run
+    const bool owned = valid && head >= 0 && head < kPagedTokens;
+    const uint64_t owned_mask = __ballot(owned);
+    const int k = __builtin_popcountll(owned_mask & ((1ull << i) - 1ull));
+    if (owned) {
+      s_blk[k] = blk;
+      s_off[k] = off;
+      s_tok[k] = i;
+    }
+    // a run of 16 tokens starts at a multiple of 16 slots; its V region is 16-byte aligned if
+    // the block's is
+    const bool whole = owned && !cont && i < kPagedTokens && ((bs * CE) & 15) == 0 &&
+                       __builtin_ctzll(starts >> (i + 1)) + 1 == 16;
+    const uint64_t whole_mask = __ballot(whole);
+    if (i == 0) {
+      s_count = __builtin_popcountll(owned_mask);
+      s_whole = whole_mask ? __builtin_popcountll(owned_mask & ((1ull << __builtin_ctzll(whole_mask)) - 1ull)) : -1;
+    }
+  }
+  __syncthreads();
+  const int count = s_count;
+  if (count == 0) return;
+
+  // ---- phase 1: owned source rows into LDS ----
+  if (p.vec_src) {
+    const int pieces = seg_elems >> 3; // 16-byte source pieces per row
+    for (int q = tid; q < count * pieces; q += kThreads) {
+      const int r = q / pieces, c = q - r * pieces;
+      const u32x4 v = ld<u32x4, true>(src + ((t0 + s_tok[r]) * stride + e0 + c * 8) * 2);
+      if constexpr (CE == 2)
+        *reinterpret_cast<u32x4 *>(tile + r * ROW + c * 16) = v;
+      else
+        *reinterpret_cast<u32x2 *>(tile + r * ROW + c * 8) = quant8<SRC_DTYPE>(v, scale);
+    }
+  } else {
+    for (int q = tid; q < count * seg_elems; q += kThreads) {
+      const int r = q / seg_elems, c = q - r * seg_elems;
+      const uint16_t h = ld<uint16_t, false>(src + ((t0 + s_tok[r]) * stride + e0 + c) * 2);
+      if constexpr (CE == 2)
+        *reinterpret_cast<uint16_t *>(tile + r * ROW + c * 2) = h;
+      else
+        *reinterpret_cast<uint8_t *>(tile + r * ROW + c) =
+            (uint8_t)f32_to_e4m3fn(half_bits_to_f32<SRC_DTYPE>(h) / scale);
+    }
+  }
+  __syncthreads();
+
+  if (kv == 0) {
+    // ---- K: 16-byte pieces, token fastest ----
+    const int groups = seg_elems / X;
+    const int64_t g0 = e0 / X, groups_per_block = p.row_elems / X;
+    for (int base = 0; base < count; base += 16) {
+      for (int q = tid; q < groups * 16; q += kThreads) {
+        const int g = q >> 4, r = base + (q & 15);
+        if (r >= count) continue;
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(tile + r * ROW + g * 16);
+        char *dst = cache + ((s_blk[r] * groups_per_block + g0 + g) * bs + s_off[r]) * 16;
+        st_stream<u32x4, 1>(dst, v);
+      }
+    }
+    return;
+  }
+  const int whole = s_whole;
+  if (whole >= 0) {
+    // ---- V, whole run: 16-byte pieces of the run's [element][16 tokens] region ----
+    const int64_t blk = s_blk[whole];
+    const int off0 = s_off[whole];
+    const char *rows = tile + whole * ROW;
+    for (int q = tid; q < seg_elems * CE; q += kThreads) {
+      uint32_t w[4];
+      int e;
+      if constexpr (CE == 2) {
+        e = q >> 1;
+        const char *col = rows + (q & 1) * 8 * ROW + e * 2;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t lo = *reinterpret_cast<const uint16_t *>(col + (2 * i) * ROW);
+          const uint32_t hi = *reinterpret_cast<const uint16_t *>(col + (2 * i + 1) * ROW);
+          w[i] = lo | (hi << 16);
+        }
+      } else {
+        e = q;
+        const char *col = rows + e;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          uint32_t x = 0;
+#pragma unroll
+          for (int k = 0; k < 4; ++k)
+            x |= (uint32_t) * reinterpret_cast<const uint8_t *>(col + (4 * i + k) * ROW) << (8 * k);
+          w[i] = x;
+        }
+      }
+      char *dst = cache + ((blk * p.row_elems + e0 + e) * bs + off0) * CE + (CE == 2 ? (q & 1) * 16 : 0);
+      st_stream<u32x4, 1>(dst, u32x4{w[0], w[1], w[2], w[3]});
+    }
+  }
+  // ---- V, the other owned tokens: one element per lane, element fastest ----
+  // (a wave instruction covers 64 consecutive elements of one token: 64 sectors in 16 consecutive
+  // cache lines of the block's V region)
+  const int rest = whole >= 0 ? count - 16 : count;
+  for (int i = 0; i < rest; ++i) {
+    const int r = (whole >= 0 && i >= whole) ? i + 16 : i; // step over the whole run
+    char *base = cache + ((s_blk[r] * p.row_elems + e0) * bs + s_off[r]) * CE;
+    for (int e = tid; e < seg_elems; e += kThreads) {
+      char *dst = base + (int64_t)e * bs * CE;
+      if constexpr (CE == 2)
+        st<uint16_t, false>(dst, *reinterpret_cast<const uint16_t *>(tile + r * ROW + e * 2));
+      else
+        st<uint8_t, false>(dst, *reinterpret_cast<const uint8_t *>(tile + r * ROW + e));
+    }
+  }
+}
+
+int append_paged(const void *const *k, const void *const *v, void *const *kc, void *const *vc, int num_layers,
+                 const int64_t *slot_mapping, int64_t num_tokens, int num_heads, int head_size,
+                 int block_size, int64_t num_blocks, int64_t ks, int64_t vs, int src_dtype,
+                 int cache_elem_bytes, const float *k_scales, const float *v_scales, hipStream_t s,
+                 const char *what) {
+  if (num_layers < 0 || num_layers > EMM_MAX_LAYERS)
+    return fail(EMM_EINVAL, "%s: num_layers=%d outside [0, %d]", what, num_layers, EMM_MAX_LAYERS);
+  if (num_tokens < 0 || num_heads < 0 || head_size < 0 || block_size <= 0 || num_blocks < 0 || ks < 0 || vs < 0)
+    return fail(EMM_EINVAL, "%s: negative size", what);
+  if (cache_elem_bytes != 1 && cache_elem_bytes != 2)
+    return fail(EMM_EINVAL, "%s: cache_elem_bytes=%d, expected 2 (16-bit cache) or 1 (fp8 cache)", what,
+                cache_elem_bytes);
+  if (src_dtype != EMM_DTYPE_BF16 && src_dtype != EMM_DTYPE_F16)
+    return fail(EMM_EINVAL, "%s: unknown src_dtype %d", what, src_dtype);
+  const int x = 16 / cache_elem_bytes;
+  if (head_size % x)
+    return fail(EMM_EINVAL, "%s: head_size=%d is not a multiple of x=%d", what, head_size, x);
+  const int64_t row_elems = (int64_t)num_heads * head_size;
+  if (num_tokens == 0 || row_elems == 0 || num_layers == 0) return EMM_OK;
+  if (!k || !v || !kc || !vc || !slot_mapping) return fail(EMM_EINVAL, "%s: null pointer", what);
+  if (cache_elem_bytes == 1 && (!k_scales || !v_scales)) return fail(EMM_EINVAL, "%s: scale pointer is null", what);
+  if (ks < row_elems || vs < row_elems) return fail(EMM_EINVAL, "%s: token stride smaller than the row", what);
+  const int64_t tiles = (num_tokens + kPagedTokens - 1) / kPagedTokens;
+  const int64_t segs = (row_elems + kPagedSeg - 1) / kPagedSeg;
+  if (tiles > 0x7fffffffLL || segs * 2 > kMaxGridY) return fail(EMM_EINVAL, "%s: too many tokens / too long rows", what);
+  PagedParams p;
+  memset(&p, 0, sizeof(p));
+  p.vec_src = ks % 8 == 0 && vs % 8 == 0;
+  for (int l = 0; l < num_layers; ++l) {
+    if (!k[l] || !v[l] || !kc[l] || !vc[l]) return fail(EMM_EINVAL, "%s: null tensor pointer at layer %d", what, l);
+    if (!aligned(k[l], 2) || !aligned(v[l], 2))
+      return fail(EMM_EINVAL, "%s: 16-bit source not 2-byte aligned at layer %d", what, l);
+    if (!aligned(kc[l], 16) || !aligned(vc[l], 16))
+      return fail(EMM_EINVAL, "%s: cache not 16-byte aligned at layer %d", what, l);
+    if (!aligned(k[l], 16) || !aligned(v[l], 16)) p.vec_src = 0;
+    p.key[l] = (const char *)k[l];
+    p.value[l] = (const char *)v[l];
+    p.key_cache[l] = (char *)kc[l];
+    p.value_cache[l] = (char *)vc[l];
+  }
+  p.slot_mapping = slot_mapping;
+  p.k_scales = k_scales;
+  p.v_scales = v_scales;
+  p.num_tokens = num_tokens;
+  p.row_elems = row_elems;
+  p.key_stride = ks;
+  p.value_stride = vs;
+  p.num_blocks = num_blocks;
+  p.block_size = block_size;
+  const dim3 grid((uint32_t)tiles, (uint32_t)(segs * 2), (uint32_t)num_layers);
+  if (cache_elem_bytes == 2)
+    emm_append_paged_kernel<2, EMM_DTYPE_BF16><<<grid, kThreads, 0, s>>>(p);
+  else if (src_dtype == EMM_DTYPE_BF16)
+    emm_append_paged_kernel<1, EMM_DTYPE_BF16><<<grid, kThreads, 0, s>>>(p);
+  else
+    emm_append_paged_kernel<1, EMM_DTYPE_F16><<<grid, kThreads, 0, s>>>(p);
+  return check_launch(what);
+}
+
+// ----------------------------------------------------------------------------
 // concat_rows: ragged segments -> one contiguous buffer
 // ----------------------------------------------------------------------------
 constexpr int kSegGroup = 12; // segments per group of the two-level tile -> segment search
@@ -1072,6 +1340,30 @@ int emm_reshape_and_cache_fp8_layers(const void *const *key_ptrs, const void *co
                     slot_mapping, num_tokens, row_elems, key_stride_elems, value_stride_elems,
                     num_slots, k_scales, v_scales, src_dtype, as_stream(stream),
                     "emm_reshape_and_cache_fp8_layers");
+}
+
+int emm_reshape_and_cache_paged(const void *key, const void *value, void *key_cache, void *value_cache,
+                                const int64_t *slot_mapping, int64_t num_tokens, int num_heads,
+                                int head_size, int block_size, int64_t num_blocks,
+                                int64_t key_stride_elems, int64_t value_stride_elems, int src_dtype,
+                                int cache_elem_bytes, const float *k_scale, const float *v_scale,
+                                emm_stream_t stream) {
+  return append_paged(&key, &value, &key_cache, &value_cache, 1, slot_mapping, num_tokens, num_heads,
+                      head_size, block_size, num_blocks, key_stride_elems, value_stride_elems, src_dtype,
+                      cache_elem_bytes, k_scale, v_scale, as_stream(stream), "emm_reshape_and_cache_paged");
+}
+
+int emm_reshape_and_cache_paged_layers(const void *const *key_ptrs, const void *const *value_ptrs,
+                                       void *const *key_cache_ptrs, void *const *value_cache_ptrs,
+                                       int num_layers, const int64_t *slot_mapping, int64_t num_tokens,
+                                       int num_heads, int head_size, int block_size, int64_t num_blocks,
+                                       int64_t key_stride_elems, int64_t value_stride_elems,
+                                       int src_dtype, int cache_elem_bytes, const float *k_scales,
+                                       const float *v_scales, emm_stream_t stream) {
+  return append_paged(key_ptrs, value_ptrs, key_cache_ptrs, value_cache_ptrs, num_layers, slot_mapping,
+                      num_tokens, num_heads, head_size, block_size, num_blocks, key_stride_elems,
+                      value_stride_elems, src_dtype, cache_elem_bytes, k_scales, v_scales, as_stream(stream),
+                      "emm_reshape_and_cache_paged_layers");
 }
 
 int emm_concat_rows(const void *const *srcs, const int64_t *nbytes, int n, void *dst,

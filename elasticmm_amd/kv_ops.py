@@ -321,6 +321,120 @@ def reshape_and_cache(key: torch.Tensor, value: torch.Tensor, key_cache: torch.T
         raise TypeError(f"unsupported source/cache element sizes {eb}/{ceb}")
 
 
+def _paged_geometry(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor):
+    """Checks one layer of a paged-layout append; returns (T, H, D, bs, NB, ks, vs, cache_elem_bytes)."""
+    for t in (key, value, key_cache, value_cache):
+        _require_gpu(t, "reshape_and_cache_paged")
+    if key.dim() != 3 or value.shape != key.shape:
+        raise ValueError("key and value must be [num_tokens, num_heads, head_size] of one shape")
+    T, H, D = (int(v) for v in key.shape)
+    if key_cache.dim() != 5 or value_cache.dim() != 4:
+        raise ValueError("key_cache must be [NB, H, D/x, bs, x] and value_cache [NB, H, D, bs]")
+    NB, Hc, Dx, bs, x = (int(v) for v in key_cache.shape)
+    ceb = key_cache.element_size()
+    eb = key.element_size()
+    if eb != 2 or value.element_size() != 2 or ceb not in (1, 2) or value_cache.element_size() != ceb:
+        raise TypeError(f"unsupported source/cache element sizes {eb}/{ceb}")
+    if x != 16 // ceb or Hc != H or Dx * x != D:
+        raise ValueError(f"key_cache shape {tuple(key_cache.shape)} does not match H={H}, D={D}, x={16 // ceb}")
+    if tuple(value_cache.shape) != (NB, H, D, bs):
+        raise ValueError(f"value_cache shape {tuple(value_cache.shape)} does not match key_cache")
+    if not key_cache.is_contiguous() or not value_cache.is_contiguous():
+        raise ValueError("caches must be contiguous")
+    _, _, ks = _row_geometry(key, "key")
+    _, _, vs = _row_geometry(value, "value")
+    return T, H, D, bs, NB, ks, vs, ceb
+
+
+def _check_slot_mapping(slot_mapping: torch.Tensor, T: int) -> torch.Tensor:
+    if slot_mapping.dtype != torch.long or not slot_mapping.is_cuda:
+        raise TypeError("slot_mapping must be an int64 GPU tensor")
+    if not slot_mapping.is_contiguous():
+        slot_mapping = slot_mapping.contiguous()
+    if slot_mapping.numel() < T:
+        raise ValueError("slot_mapping is shorter than the token count")
+    return slot_mapping
+
+
+def reshape_and_cache_paged(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor,
+                            value_cache: torch.Tensor, slot_mapping: torch.Tensor,
+                            k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None) -> None:
+    """Append one layer into the paged-attention layout:
+    ``key_cache[b, h, d // x, o, d % x] = key[t, h, d]``, ``value_cache[b, h, d, o] = value[t, h, d]``
+    with ``b, o = divmod(slot_mapping[t], block_size)``; slots < 0 are skipped.
+
+    key / value are ``[T, H, D]``; key_cache ``[NB, H, D // x, bs, x]`` and value_cache
+    ``[NB, H, D, bs]``, contiguous, x = 16 // cache element size. A 1-byte cache with a
+    16-bit source is quantised to fp8-e4m3fn with ``k_scale`` / ``v_scale``."""
+    lib = _lib.load()
+    T, H, D, bs, NB, ks, vs, ceb = _paged_geometry(key, value, key_cache, value_cache)
+    slot_mapping = _check_slot_mapping(slot_mapping, T)
+    k_ptr = v_ptr = None
+    keep = None
+    if ceb == 1:
+        if k_scale is None or v_scale is None:
+            raise ValueError("fp8 cache needs k_scale and v_scale")
+        keep = (_scales_tensor(k_scale, 1, key.device), _scales_tensor(v_scale, 1, key.device))
+        k_ptr, v_ptr = keep[0].data_ptr(), keep[1].data_ptr()
+    code = _half_code(key.dtype, "reshape_and_cache_paged") if ceb == 1 else 0
+    check(lib.emm_reshape_and_cache_paged(key.data_ptr(), value.data_ptr(), key_cache.data_ptr(),
+                                          value_cache.data_ptr(), slot_mapping.data_ptr(), T, H, D, bs, NB, ks, vs,
+                                          code, ceb, k_ptr, v_ptr, _stream_ptr(key.device)),
+          "emm_reshape_and_cache_paged")
+
+
+class PagedLayeredAppend:
+    """The paged-layout append for all layers of one step in a single launch (per group of
+    EMM_MAX_LAYERS): tensors validated and pointer tables built once, then one C call per
+    ``slot_mapping``. The object keeps the tensors alive."""
+
+    def __init__(self, keys: Sequence[torch.Tensor], values: Sequence[torch.Tensor],
+                 key_caches: Sequence[torch.Tensor], value_caches: Sequence[torch.Tensor],
+                 k_scales=None, v_scales=None):
+        self.lib = _lib.load()
+        L = len(keys)
+        if not (len(values) == len(key_caches) == len(value_caches) == L):
+            raise ValueError("per-layer lists differ in length")
+        self.num_layers = L
+        self._keep = (list(keys), list(values), list(key_caches), list(value_caches))
+        if L == 0:
+            return
+        self.geom = _paged_geometry(keys[0], values[0], key_caches[0], value_caches[0])
+        for l in range(1, L):
+            if _paged_geometry(keys[l], values[l], key_caches[l], value_caches[l]) != self.geom:
+                raise ValueError(f"layer {l}: geometry differs from layer 0")
+        self.device = keys[0].device
+        self.fp8 = self.geom[7] == 1
+        self.code = 0
+        self.k_s = self.v_s = None
+        if self.fp8:
+            if k_scales is None or v_scales is None:
+                raise ValueError("fp8 cache needs k_scales and v_scales")
+            self.code = _half_code(keys[0].dtype, "PagedLayeredAppend")
+            self.k_s = _scales_tensor(k_scales, L, self.device)
+            self.v_s = _scales_tensor(v_scales, L, self.device)
+        self.groups = []
+        for l0 in range(0, L, EMM_MAX_LAYERS):
+            sl = slice(l0, l0 + EMM_MAX_LAYERS)
+            self.groups.append((l0, ptr_table([t.data_ptr() for t in keys[sl]]),
+                                ptr_table([t.data_ptr() for t in values[sl]]),
+                                ptr_table([t.data_ptr() for t in key_caches[sl]]),
+                                ptr_table([t.data_ptr() for t in value_caches[sl]])))
+
+    def __call__(self, slot_mapping: torch.Tensor) -> None:
+        if self.num_layers == 0:
+            return
+        T, H, D, bs, NB, ks, vs, ceb = self.geom
+        slot_mapping = _check_slot_mapping(slot_mapping, T)
+        stream = _stream_ptr(self.device)
+        for l0, kt, vt, kct, vct in self.groups:
+            k_ptr = self.k_s.data_ptr() + 4 * l0 if self.fp8 else None
+            v_ptr = self.v_s.data_ptr() + 4 * l0 if self.fp8 else None
+            check(self.lib.emm_reshape_and_cache_paged_layers(kt, vt, kct, vct, len(kt), slot_mapping.data_ptr(), T, H,
+                                                              D, bs, NB, ks, vs, self.code, ceb, k_ptr, v_ptr, stream),
+                  "emm_reshape_and_cache_paged_layers")
+
+
 class LayeredAppend:
     """All layers of one step appended with a single launch (per group of EMM_MAX_LAYERS).
 

@@ -193,6 +193,54 @@ int emm_reshape_and_cache_fp8_layers(const void *const *key_ptrs,
                                      emm_stream_t stream);
 
 /*
+ * reshape_and_cache (paged-attention layout) — append into the transposed pool
+ * of vLLM's PagedAttention backends:
+ *   key_cache   [num_blocks, num_heads, head_size / x, block_size, x]
+ *   value_cache [num_blocks, num_heads, head_size, block_size]
+ * with x = 16 / cache_elem_bytes (8 for a 16-bit cache, 16 for fp8). For token t
+ * with s = slot_mapping[t], b = s / block_size, o = s % block_size:
+ *   key_cache[b, h, d / x, o, d % x] = key[t, h, d]
+ *   value_cache[b, h, d, o]          = value[t, h, d]
+ * s < 0 and s >= num_blocks * block_size are skipped. cache_elem_bytes = 2 copies
+ * bits (any 16-bit type); cache_elem_bytes = 1 quantises to e4m3fn with the rule of
+ * emm_reshape_and_cache_fp8 (k_scale / v_scale: DEVICE pointers to one float each,
+ * ignored for a 16-bit cache). Strides in elements. This is vLLM's
+ * reshape_and_cache(key, value, key_cache, value_cache, slot_mapping,
+ * kv_cache_dtype, k_scale, v_scale), the append that
+ * elasticmm/engine/v0/worker_steps.py:281, :438 reaches when vLLM selects a
+ * PagedAttention backend (its default on ROCm) instead of flash-attn; the pool
+ * bound at worker.py:408-412 is then [2, num_blocks, block_size * H * D] per layer,
+ * which pack / unpack / copy_blocks move unchanged (one block is still one chunk).
+ */
+int emm_reshape_and_cache_paged(const void *key, const void *value,
+                                void *key_cache, void *value_cache,
+                                const int64_t *slot_mapping, int64_t num_tokens,
+                                int num_heads, int head_size, int block_size,
+                                int64_t num_blocks, int64_t key_stride_elems,
+                                int64_t value_stride_elems, int src_dtype,
+                                int cache_elem_bytes, const float *k_scale,
+                                const float *v_scale, emm_stream_t stream);
+
+/* Paged-layout append for all layers of one step in a single launch (pointer
+ * tables as in emm_reshape_and_cache_layers; k_scales / v_scales: DEVICE float
+ * arrays of num_layers, fp8 caches only). */
+int emm_reshape_and_cache_paged_layers(const void *const *key_ptrs,
+                                       const void *const *value_ptrs,
+                                       void *const *key_cache_ptrs,
+                                       void *const *value_cache_ptrs,
+                                       int num_layers,
+                                       const int64_t *slot_mapping,
+                                       int64_t num_tokens, int num_heads,
+                                       int head_size, int block_size,
+                                       int64_t num_blocks,
+                                       int64_t key_stride_elems,
+                                       int64_t value_stride_elems,
+                                       int src_dtype, int cache_elem_bytes,
+                                       const float *k_scales,
+                                       const float *v_scales,
+                                       emm_stream_t stream);
+
+/*
  * concat_rows — copy n ragged segments back to back into `dst`: segment i is
  * nbytes[i] bytes at srcs[i]. HOST arrays (n <= EMM_MAX_SEGMENTS per call;
  * `dst_offset_bytes` lets the caller continue a longer list). Replaces

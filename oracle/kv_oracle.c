@@ -209,6 +209,40 @@ void orc_reshape_and_cache_fp8(const uint16_t *key, const uint16_t *value,
   }
 }
 
+/* ---- reshape_and_cache, paged-attention layout (vLLM; same call sites when a
+ * PagedAttention backend is selected): key_cache [NB, H, D/x, bs, x],
+ * value_cache [NB, H, D, bs], x = 16 / cache element bytes. Written from the
+ * layout definition with explicit index arithmetic; cache_elem_bytes 2 copies
+ * bits, 1 quantises to e4m3fn. */
+void orc_reshape_and_cache_paged(const uint16_t *key, const uint16_t *value,
+                                 void *key_cache, void *value_cache,
+                                 const int64_t *slot_mapping, int64_t num_tokens,
+                                 int num_heads, int head_size, int block_size,
+                                 int64_t num_blocks, int64_t key_stride,
+                                 int64_t value_stride, int src_dtype,
+                                 int cache_elem_bytes, float k_scale, float v_scale) {
+  const int x = 16 / cache_elem_bytes;
+  for (int64_t t = 0; t < num_tokens; ++t) {
+    const int64_t s = slot_mapping[t];
+    if (s < 0 || s >= num_blocks * block_size) continue;
+    const int64_t b = s / block_size, o = s % block_size;
+    for (int h = 0; h < num_heads; ++h)
+      for (int d = 0; d < head_size; ++d) {
+        const uint16_t kx = key[t * key_stride + (int64_t)h * head_size + d];
+        const uint16_t vx = value[t * value_stride + (int64_t)h * head_size + d];
+        const int64_t ki = ((((b * num_heads + h) * (head_size / x) + d / x) * block_size + o) * x) + d % x;
+        const int64_t vi = ((b * num_heads + h) * head_size + d) * block_size + o;
+        if (cache_elem_bytes == 2) {
+          ((uint16_t *)key_cache)[ki] = kx;
+          ((uint16_t *)value_cache)[vi] = vx;
+        } else {
+          ((uint8_t *)key_cache)[ki] = orc_f32_to_e4m3fn(half_to_f32(kx, src_dtype) / k_scale);
+          ((uint8_t *)value_cache)[vi] = orc_f32_to_e4m3fn(half_to_f32(vx, src_dtype) / v_scale);
+        }
+      }
+  }
+}
+
 /* ---- dequant-unpack: packed fp8 [L,2,n,chunk] -> 16-bit pool under idx */
 void orc_kv_unpack_dequant_fp8(void *const *layers, int num_layers,
                                int64_t num_blocks, int64_t chunk_elems,

@@ -155,6 +155,29 @@ def ref_reshape_and_cache_flash(key: torch.Tensor, value: torch.Tensor, key_cach
             cache.view(NB * bs, H, D).index_copy_(0, slots, rows)
 
 
+def ref_reshape_and_cache_paged(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor,
+                                value_cache: torch.Tensor, slot_mapping: torch.Tensor,
+                                kv_cache_dtype: str = "auto",
+                                k_scale: Optional[torch.Tensor] = None,
+                                v_scale: Optional[torch.Tensor] = None) -> None:
+    """vLLM reshape_and_cache (PagedAttention layout) as torch indexed assignment:
+    key_cache [NB, H, D/x, bs, x], value_cache [NB, H, D, bs]; for slot >= 0 with
+    b, o = divmod(slot, bs): ``key_cache[b, :, :, o, :] = key[t].view(H, D/x, x)`` and
+    ``value_cache[b, :, :, o] = value[t]``. fp8 caches are given as uint8."""
+    NB, H, Dx, bs, x = key_cache.shape
+    valid = slot_mapping >= 0
+    slots = slot_mapping[valid]
+    b = torch.div(slots, bs, rounding_mode="floor")
+    o = slots - b * bs
+    k, v = key[valid], value[valid]
+    if kv_cache_dtype.startswith("fp8"):
+        k = (k.float() / k_scale.float().reshape(())).to(torch.float8_e4m3fn).view(torch.uint8)
+        v = (v.float() / v_scale.float().reshape(())).to(torch.float8_e4m3fn).view(torch.uint8)
+    # two index tensors separated by slices: the indexed dimension comes first in the result
+    key_cache[b, :, :, o, :] = k.reshape(-1, H, Dx, x)
+    value_cache[b, :, :, o] = v
+
+
 def ref_unpack_dequant_fp8(kv_cache: Sequence[torch.Tensor], block_indices: Sequence[int],
                            packed_fp8: torch.Tensor, k_scales: torch.Tensor, v_scales: torch.Tensor) -> None:
     """Dequantising unpack: ``pool[l][kv, idx] = (q.float() * scale).to(pool dtype)``.
@@ -278,6 +301,19 @@ def c_reshape_and_cache_fp8(key: torch.Tensor, value: torch.Tensor, key_cache_u8
                                     _dtype_code(key.dtype))
 
 
+def c_reshape_and_cache_paged(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor,
+                              value_cache: torch.Tensor, slot_mapping, k_scale: float = 1.0,
+                              v_scale: float = 1.0) -> None:
+    T, H, D = key.shape
+    NB, _, _, bs, x = key_cache.shape
+    slots = _i64(slot_mapping)
+    lib().orc_reshape_and_cache_paged(_ptr(_np_bytes(key)), _ptr(_np_bytes(value)), _ptr(_np_bytes(key_cache)),
+                                      _ptr(_np_bytes(value_cache)), _ptr(slots), ctypes.c_int64(T), H, D, bs,
+                                      ctypes.c_int64(NB), ctypes.c_int64(H * D), ctypes.c_int64(H * D),
+                                      _dtype_code(key.dtype), key_cache.element_size(),
+                                      ctypes.c_float(k_scale), ctypes.c_float(v_scale))
+
+
 def c_unpack_dequant_fp8(layers: Sequence[torch.Tensor], idx, packed_u8, k_scales, v_scales) -> None:
     views = [_np_bytes(p) for p in layers]
     NB = layers[0].shape[1]
@@ -338,6 +374,18 @@ def brute_reshape_and_cache(key, value, key_cache, value_cache, slot_mapping) ->
             for d in range(D):
                 key_cache[blk, off, h, d] = key[t, h, d]
                 value_cache[blk, off, h, d] = value[t, h, d]
+
+
+def brute_reshape_and_cache_paged(key, value, key_cache, value_cache, slot_mapping) -> None:
+    NB, H, Dx, bs, x = key_cache.shape
+    for t, s in enumerate([int(v) for v in slot_mapping]):
+        if s < 0:
+            continue
+        blk, off = s // bs, s % bs
+        for h in range(H):
+            for d in range(Dx * x):
+                key_cache[blk, h, d // x, off, d % x] = key[t, h, d]
+                value_cache[blk, h, d, off] = value[t, h, d]
 
 
 def brute_copy_blocks(kv_caches, mapping) -> None:

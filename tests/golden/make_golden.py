@@ -11,6 +11,9 @@ writes
     kv_small.npz     seeded tiny pools, block tables, slot mapping and the
                      expected results of pack / unpack / append / copy_blocks /
                      concat (raw little-endian bit patterns as uint16 / uint8)
+    paged_small.npz  an append into the paged-attention layout, stated as a flat-slot
+                     index_copy followed by a permute of the whole cache (not as an
+                     indexed assignment into the transposed layout)
     fp8_kat.json     known answers of the fp8-e4m3fn cast: the explicit vector of
                      special values and the SHA-256 of the exhaustive sweep of
                      all 65 536 bf16 (and f16) bit patterns at several scales,
@@ -75,6 +78,29 @@ def kv_small():
     )
 
 
+def paged_small():
+    g = torch.Generator().manual_seed(4321)
+    NB, bs, H, D, x, T = 5, 4, 2, 16, 8, 13
+    key = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+    value = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+    slots = torch.randperm(NB * bs, generator=g)[:T].clone()
+    slots[4] = -1
+    slots[11] = -1
+    # fill values differ per position so that a transposed write into the wrong place shows
+    kflat = (torch.arange(NB * bs * H * D, dtype=torch.float32) % 251).to(torch.bfloat16).view(NB * bs, H, D)
+    vflat = (torch.arange(NB * bs * H * D, dtype=torch.float32) % 241).to(torch.bfloat16).view(NB * bs, H, D)
+    k_before = kflat.view(NB, bs, H, D // x, x).permute(0, 2, 3, 1, 4).contiguous()
+    v_before = vflat.view(NB, bs, H, D).permute(0, 2, 3, 1).contiguous()
+    valid = slots >= 0
+    kflat = kflat.clone().index_copy_(0, slots[valid], key[valid])
+    vflat = vflat.clone().index_copy_(0, slots[valid], value[valid])
+    k_after = kflat.view(NB, bs, H, D // x, x).permute(0, 2, 3, 1, 4).contiguous()
+    v_after = vflat.view(NB, bs, H, D).permute(0, 2, 3, 1).contiguous()
+    np.savez_compressed(os.path.join(HERE, "paged_small.npz"), key=bits16(key), value=bits16(value),
+                        slots=slots.numpy(), key_cache_before=bits16(k_before), value_cache_before=bits16(v_before),
+                        key_cache_after=bits16(k_after), value_cache_after=bits16(v_after))
+
+
 def fp8_kat():
     special = [448, 464, 465, 480, -1000, 2 ** -9, 2 ** -10, 2 ** -10 * 1.0001, 17, 18, 19, float("inf"),
                float("-inf"), float("nan"), -0.0, 0.0, -2 ** -11, 479.9, 1e-40, 0.5, -1.75, 2 ** -6, 2 ** -7 * 1.9]
@@ -100,5 +126,6 @@ def fp8_kat():
 
 if __name__ == "__main__":
     kv_small()
+    paged_small()
     fp8_kat()
     print("wrote", sorted(os.listdir(HERE)))

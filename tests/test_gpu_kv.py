@@ -349,6 +349,138 @@ def test_append_out_of_range_slot_is_skipped():
 
 
 # ------------------------------------------------------------------ fp8
+# ---------------------------------------------------------------- append, paged-attention layout
+def paged_slots(NB, bs, T, seed, whole_frac=0.6, pad_frac=0.05, phase=0):
+    """A slot table shaped like a serving step: prompts that fill whole blocks in order (the first
+    one starts at token `phase`, so block starts are not aligned to token tiles unless phase = 0),
+    partial runs, and single scattered tokens; a few padded entries."""
+    g = torch.Generator().manual_seed(seed)
+    blocks = torch.randperm(NB, generator=g).tolist()
+    slots = []
+    for _ in range(phase):
+        b = blocks.pop()
+        slots.append(b * bs + int(torch.randint(bs, (1,), generator=g)))
+    while len(slots) < T * whole_frac and blocks:
+        b = blocks.pop()
+        slots.extend(range(b * bs, (b + 1) * bs))
+    while len(slots) < T and blocks:
+        b = blocks.pop()
+        run = int(torch.randint(1, bs + 1, (1,), generator=g))
+        start = int(torch.randint(0, bs - run + 1, (1,), generator=g))
+        slots.extend(range(b * bs + start, b * bs + start + run))
+    slots = torch.tensor(slots[:T], dtype=torch.long)
+    pad = torch.rand(len(slots), generator=g) < pad_frac
+    slots[pad] = -1
+    return slots
+
+
+def paged_caches_cpu(NB, H, D, bs, dtype, fill_mod=61):
+    eb = 1 if dtype == torch.uint8 else 2
+    x = 16 // eb
+    n = NB * H * D * bs
+    base = (torch.arange(n, dtype=torch.float32) % fill_mod)
+    base = base.to(torch.uint8) if dtype == torch.uint8 else base.to(dtype)
+    return base.view(NB, H, D // x, bs, x).clone(), base.view(NB, H, D, bs).clone()
+
+
+@pytest.mark.parametrize("dtype,NB,bs,H,D,T,phase,desc", [
+    (torch.bfloat16, 1024, 16, 4, 128, 8448, 0, "Qwen2-7B rows, prompts aligned to token tiles"),
+    (torch.bfloat16, 1024, 16, 4, 128, 8448, 5, "Qwen2-7B rows, prompts off the tile grid"),
+    (torch.float16, 300, 16, 8, 128, 2500, 3, "70B-shape rows: two row segments per token"),
+    (torch.float16, 96, 8, 3, 40, 333, 0, "120-element rows, block size 8"),
+    (torch.bfloat16, 48, 32, 2, 64, 700, 0, "block size 32"),
+    (torch.bfloat16, 33, 16, 5, 104, 1, 0, "a single token; 520-element rows (second segment of 8)"),
+])
+def test_paged_append_against_oracle(dtype, NB, bs, H, D, T, phase, desc):
+    say(f"paged append: {desc}")
+    g = torch.Generator().manual_seed(NB + T)
+    key = torch.randn((T, H, D), generator=g).to(dtype)
+    value = torch.randn((T, H, D), generator=g).to(dtype)
+    slots = paged_slots(NB, bs, T, seed=T, phase=phase)
+    assert len(slots) == T
+    kc, vc = paged_caches_cpu(NB, H, D, bs, dtype)
+    kc_g, vc_g = kc.to(DEV), vc.to(DEV)
+    cache_ops.reshape_and_cache(key.to(DEV), value.to(DEV), kc_g, vc_g, slots.to(DEV), "auto")
+    orc.c_reshape_and_cache_paged(key, value, kc, vc, slots)
+    assert same_bits(kc_g, kc) and same_bits(vc_g, vc)
+    if T <= 2500:  # the torch statement as a second witness
+        kr, vr = paged_caches_cpu(NB, H, D, bs, dtype)
+        orc.ref_reshape_and_cache_paged(key, value, kr, vr, slots)
+        assert same_bits(kc_g, kr) and same_bits(vc_g, vr)
+
+
+def test_paged_append_strided_sources_random_slots_and_golden(golden_dir):
+    NB, bs, H, D, T = 24, 16, 2, 64, 101
+    g = torch.Generator().manual_seed(77)
+    qkv = torch.randn((T, 3 * H * D + 4), generator=g).to(torch.float16)  # row stride not a multiple of 8 elements
+    slots = make_slots(NB * bs, T, 77, pad_frac=0.1)
+    qkv_g = qkv.to(DEV)
+    for lo in (H * D, H * D + 1):  # second view: base not 16-byte aligned
+        k_g = qkv_g[:, lo:lo + H * D].view(T, H, D)
+        v_g = qkv_g[:, lo + H * D:lo + 2 * H * D].view(T, H, D)
+        kc, vc = paged_caches_cpu(NB, H, D, bs, torch.float16)
+        kc_g, vc_g = kc.to(DEV), vc.to(DEV)
+        cache_ops.reshape_and_cache(k_g, v_g, kc_g, vc_g, slots.to(DEV))
+        orc.c_reshape_and_cache_paged(qkv[:, lo:lo + H * D].reshape(T, H, D).contiguous(),
+                                      qkv[:, lo + H * D:lo + 2 * H * D].reshape(T, H, D).contiguous(), kc, vc, slots)
+        assert same_bits(kc_g, kc) and same_bits(vc_g, vc)
+    z = np.load(os.path.join(golden_dir, "paged_small.npz"))
+    bf = torch.bfloat16
+    as_t = lambda a: torch.from_numpy(a.view(np.int16).copy()).view(bf)  # noqa: E731
+    kc_g, vc_g = as_t(z["key_cache_before"]).to(DEV), as_t(z["value_cache_before"]).to(DEV)
+    cache_ops.reshape_and_cache(as_t(z["key"]).to(DEV), as_t(z["value"]).to(DEV), kc_g, vc_g,
+                                torch.from_numpy(z["slots"]).to(DEV))
+    assert same_bits(kc_g, z["key_cache_after"]) and same_bits(vc_g, z["value_cache_after"])
+    # a slot past the pool and an empty call
+    kc_g2 = kc_g.clone()
+    x = torch.ones((2, kc_g.shape[1], kc_g.shape[2] * kc_g.shape[4]), dtype=bf, device=DEV)
+    cache_ops.reshape_and_cache(x, x, kc_g2, vc_g, torch.tensor([kc_g.shape[0] * kc_g.shape[3], -1], device=DEV))
+    cache_ops.reshape_and_cache(x[:0], x[:0], kc_g2, vc_g, torch.empty(0, dtype=torch.long, device=DEV))
+    assert torch.equal(kc_g2, kc_g)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_paged_append_all_layers_in_one_launch(fp8):
+    L, NB, bs, H, D, T = 5, 96, 16, 2, 128, 900
+    g = torch.Generator().manual_seed(31)
+    slots = paged_slots(NB, bs, T, seed=31, phase=7)
+    keys = [(torch.randn((T, H, D), generator=g) * 2).to(torch.bfloat16) for _ in range(L)]
+    values = [(torch.randn((T, H, D), generator=g) * 2).to(torch.bfloat16) for _ in range(L)]
+    ks = torch.linspace(0.02, 0.08, L)
+    vs = torch.linspace(0.5, 0.1, L)
+    cdt = torch.uint8 if fp8 else torch.bfloat16
+    caches = [paged_caches_cpu(NB, H, D, bs, cdt, fill_mod=31 + l) for l in range(L)]
+    kcs = [c[0].to(DEV) for c in caches]
+    vcs = [c[1].to(DEV) for c in caches]
+    plan = cache_ops.paged_layered_append([k.to(DEV) for k in keys], [v.to(DEV) for v in values], kcs, vcs,
+                                          "fp8" if fp8 else "auto", ks, vs)
+    plan(slots.to(DEV))
+    for l in range(L):
+        kc, vc = caches[l]
+        orc.c_reshape_and_cache_paged(keys[l], values[l], kc, vc, slots, float(ks[l]), float(vs[l]))
+        assert same_bits(kcs[l], kc) and same_bits(vcs[l], vc), f"layer {l}"
+
+
+@pytest.mark.parametrize("dtype,phase", [(torch.bfloat16, 0), (torch.float16, 2)])
+def test_paged_append_fp8(dtype, phase):
+    NB, bs, H, D, T = 200, 16, 4, 128, 2000
+    g = torch.Generator().manual_seed(5)
+    key = (torch.randn((T, H, D), generator=g) * 4).to(dtype)
+    value = (torch.randn((T, H, D), generator=g) * 300).to(dtype)  # part of it overflows to NaN
+    slots = paged_slots(NB, bs, T, seed=9, phase=phase, pad_frac=0.01)
+    ks, vs = torch.tensor([0.05]), torch.tensor([0.61])
+    kc, vc = paged_caches_cpu(NB, H, D, bs, torch.uint8)
+    kc_g, vc_g = kc.to(DEV), vc.to(DEV)
+    cache_ops.reshape_and_cache(key.to(DEV), value.to(DEV), kc_g.view(torch.float8_e4m3fn),
+                                vc_g.view(torch.float8_e4m3fn), slots.to(DEV), "fp8", ks.to(DEV), vs.to(DEV))
+    orc.c_reshape_and_cache_paged(key, value, kc, vc, slots, float(ks), float(vs))
+    assert same_bits(kc_g, kc) and same_bits(vc_g, vc)
+    kr, vr = paged_caches_cpu(NB, H, D, bs, torch.uint8)
+    orc.ref_reshape_and_cache_paged(key, value, kr, vr, slots, "fp8", ks, vs)
+    assert same_bits(kc_g, kr) and same_bits(vc_g, vr)
+    assert int((vc_g.cpu() & 0x7F).eq(0x7F).sum()) > 100
+
+
 def test_fp8_append_exhaustive_bf16_and_f16(golden_dir):
     """Every 16-bit input x several scales through the append kernel: 64 tokens x 1024
     elements is exactly the 65 536 bit patterns."""

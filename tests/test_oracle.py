@@ -171,6 +171,105 @@ def test_reshape_and_cache_all_padding_leaves_cache():
     assert (kc == 2.0).all() and (vc == 4.0).all()
 
 
+# ---------------------------------------------------------------- append, paged-attention layout
+def _paged_caches(NB, H, D, bs, dtype, x=None):
+    x = x or 16 // torch.empty((), dtype=dtype).element_size()
+    kc = (torch.arange(NB * H * D * bs, dtype=torch.float32) % 61).to(dtype).view(NB, H, D // x, bs, x).clone()
+    vc = (torch.arange(NB * H * D * bs, dtype=torch.float32) % 59).to(dtype).view(NB, H, D, bs).clone()
+    return kc, vc
+
+
+def test_paged_append_three_statements_agree():
+    NB, bs, H, D, T = 4, 4, 2, 16, 9
+    g = torch.Generator().manual_seed(17)
+    key = torch.randn((T, H, D), generator=g).to(torch.float16)
+    value = torch.randn((T, H, D), generator=g).to(torch.float16)
+    slots = torch.tensor([13, 2, -1, 0, 15, -1, 8, 9, 5])
+    outs = []
+    for fn in (orc.ref_reshape_and_cache_paged, orc.c_reshape_and_cache_paged, orc.brute_reshape_and_cache_paged):
+        kc, vc = _paged_caches(NB, H, D, bs, torch.float16)
+        fn(key, value, kc, vc, slots)
+        outs.append((kc, vc))
+    for kc, vc in outs[1:]:
+        assert torch.equal(kc, outs[0][0]) and torch.equal(vc, outs[0][1])
+    kc, vc = outs[0]
+    # slot 13, bs 4 -> block 3, offset 1; element d = 11 of head 1 sits in group 1 at position 3
+    assert kc[3, 1, 1, 1, 3] == key[0, 1, 11] and vc[3, 1, 11, 1] == value[0, 1, 11]
+    k0, v0 = _paged_caches(NB, H, D, bs, torch.float16)
+    untouched = sorted(set(range(NB * bs)) - {13, 2, 0, 15, 8, 9, 5})
+    for s in untouched:
+        assert torch.equal(kc[s // bs, :, :, s % bs], k0[s // bs, :, :, s % bs])
+        assert torch.equal(vc[s // bs, :, :, s % bs], v0[s // bs, :, :, s % bs])
+
+
+def test_paged_append_identity_slots_is_a_permute():
+    """slot = arange: the caches are the [NB, bs, H, D] reshape of the inputs with the token axis
+    moved inwards (a statement that uses no index arithmetic at all)."""
+    NB, bs, H, D, x = 3, 8, 2, 16, 8
+    T = NB * bs
+    g = torch.Generator().manual_seed(18)
+    key = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+    value = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+    for fn in (orc.c_reshape_and_cache_paged, orc.ref_reshape_and_cache_paged):
+        kc = torch.zeros((NB, H, D // x, bs, x), dtype=torch.bfloat16)
+        vc = torch.zeros((NB, H, D, bs), dtype=torch.bfloat16)
+        fn(key, value, kc, vc, torch.arange(T))
+        assert torch.equal(kc, key.view(NB, bs, H, D // x, x).permute(0, 2, 3, 1, 4))
+        assert torch.equal(vc, value.view(NB, bs, H, D).permute(0, 2, 3, 1))
+
+
+def test_paged_append_equals_flash_append_then_permute():
+    """Any slot table: appending in the flash layout (pinned above) and permuting the whole cache
+    gives the paged caches."""
+    NB, bs, H, D, x, T = 6, 4, 3, 8, 8, 11
+    g = torch.Generator().manual_seed(19)
+    key = torch.randn((T, H, D), generator=g).to(torch.float16)
+    value = torch.randn((T, H, D), generator=g).to(torch.float16)
+    slots = torch.randperm(NB * bs, generator=g)[:T].clone()
+    slots[3] = -1
+    kf = torch.randn((NB, bs, H, D), generator=g).to(torch.float16)
+    vf = torch.randn((NB, bs, H, D), generator=g).to(torch.float16)
+    kc = kf.view(NB, bs, H, D // x, x).permute(0, 2, 3, 1, 4).contiguous()
+    vc = vf.permute(0, 2, 3, 1).contiguous()
+    orc.c_reshape_and_cache(key, value, kf, vf, slots)
+    orc.c_reshape_and_cache_paged(key, value, kc, vc, slots)
+    assert torch.equal(kc, kf.view(NB, bs, H, D // x, x).permute(0, 2, 3, 1, 4))
+    assert torch.equal(vc, vf.permute(0, 2, 3, 1))
+
+
+def test_paged_append_fp8_is_cast_then_same_placement():
+    NB, bs, H, D, x, T = 3, 4, 2, 32, 16, 10
+    g = torch.Generator().manual_seed(20)
+    key = (torch.randn((T, H, D), generator=g) * 3).to(torch.bfloat16)
+    value = (torch.randn((T, H, D), generator=g) * 200).to(torch.bfloat16)  # some values overflow to NaN
+    slots = torch.tensor([11, 10, -1, 0, 1, 2, 3, 7, 5, -1])
+    ks, vs = 0.037, 0.5
+    res = []
+    for which in ("ref", "c"):
+        kc = torch.full((NB, H, D // x, bs, x), 0x11, dtype=torch.uint8)
+        vc = torch.full((NB, H, D, bs), 0x22, dtype=torch.uint8)
+        if which == "ref":
+            orc.ref_reshape_and_cache_paged(key, value, kc, vc, slots, "fp8", torch.tensor(ks), torch.tensor(vs))
+        else:
+            orc.c_reshape_and_cache_paged(key, value, kc, vc, slots, ks, vs)
+        res.append((kc, vc))
+    assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])
+    q = torch.from_numpy(orc.c_quant_fp8(value, vs))
+    assert torch.equal(res[1][1][2, :, :, 3], q[0])  # slot 11 -> block 2, offset 3
+    assert (res[1][1] == 0x7F).any() or (res[1][1] == 0xFF).any()
+
+
+def test_golden_paged_small(golden_dir):
+    z = np.load(os.path.join(golden_dir, "paged_small.npz"))
+    bf = torch.bfloat16
+    key, value = from_bits16(z["key"], bf), from_bits16(z["value"], bf)
+    for fn in (orc.c_reshape_and_cache_paged, orc.ref_reshape_and_cache_paged):
+        kc, vc = from_bits16(z["key_cache_before"], bf), from_bits16(z["value_cache_before"], bf)
+        fn(key, value, kc, vc, torch.from_numpy(z["slots"]))
+        assert bits16(kc).tobytes() == z["key_cache_after"].tobytes()
+        assert bits16(vc).tobytes() == z["value_cache_after"].tobytes()
+
+
 # ---------------------------------------------------------------- copy_blocks
 def test_copy_blocks_three_statements_and_sources_unchanged():
     L, NB = 2, 10
