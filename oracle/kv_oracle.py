@@ -25,6 +25,11 @@ tests/test_oracle.py:
       blocks, canary-filled untouched blocks stay untouched, slot = arange(T)
       reduces to a plain reshape, -1 rows leave the cache unchanged).
       The reference holds no golden vectors or tests for this path.
+  reshape_and_cache, paged-attention layout: ref_* == c_* == brute_*; identity slots reduce to a
+      permute of the reshaped input; for any slot table the result equals the flash-layout append
+      (pinned above) followed by a permute of the whole cache; golden vector
+      tests/golden/paged_small.npz generated from that second statement. vLLM's own kernel is
+      absent: parity unpinned against it.
   fp8 quantise (append): c_quant_fp8 == torch's ``.to(torch.float8_e4m3fn)``
       (the library routine that defines the contract) on all 65 536 bf16 inputs x 6 scales
       and on the explicit known answers 448, 464, 465, 480, -1000, 2^-9, 2^-10,
