@@ -38,6 +38,8 @@ SIGNATURES = {
                                           _P, _P, c_int, _P]),
     "emm_reshape_and_cache_fp8_layers": (c_int, [_PP, _PP, _PP, _PP, c_int, _P, c_int64, c_int64, c_int64,
                                                  c_int64, c_int64, _P, _P, c_int, _P]),
+    "emm_reshape_and_cache_strided": (c_int, [_PP, _PP, _PP, _PP, c_int, _P, c_int64, c_int, c_int64, c_int, c_int64,
+                                              c_int64, c_int64, c_int64, c_int64, c_int64, _P]),
     "emm_reshape_and_cache_paged": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int64, c_int64,
                                             c_int64, c_int, c_int, _P, _P, _P]),
     "emm_reshape_and_cache_paged_layers": (c_int, [_PP, _PP, _PP, _PP, c_int, _P, c_int64, c_int, c_int, c_int,

@@ -20,14 +20,18 @@ def reshape_and_cache_flash(key: torch.Tensor, value: torch.Tensor, key_cache: t
                             value_cache: torch.Tensor, slot_mapping: torch.Tensor, kv_cache_dtype: str = "auto",
                             k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None) -> None:
     """key, value ``[num_tokens, num_heads, head_size]``; caches
-    ``[num_blocks, block_size, num_heads, head_size]``; ``slot_mapping`` int64
+    ``[num_blocks, block_size, num_heads, head_size]`` (contiguous, or for "auto" a strided view with
+    contiguous head rows such as a permuted head-major pool); ``slot_mapping`` int64
     ``[num_tokens]`` with -1 for padded tokens. ``kv_cache_dtype`` is "auto" (cache
     dtype == key dtype, bit copy) or "fp8" / "fp8_e4m3" (cache is 1 byte wide and
     is written as ``e4m3fn(float(x) / scale)``)."""
     if kv_cache_dtype == "auto":
         if key_cache.element_size() != key.element_size():
             raise ValueError("kv_cache_dtype='auto' needs a cache of the key's element size")
-        kv_ops.reshape_and_cache(key, value, key_cache, value_cache, slot_mapping)
+        if key_cache.is_contiguous() and value_cache.is_contiguous():
+            kv_ops.reshape_and_cache(key, value, key_cache, value_cache, slot_mapping)
+        else:  # e.g. the head-major pool [NB, H, bs, D] passed as a permuted view
+            kv_ops.reshape_and_cache_strided([key], [value], [key_cache], [value_cache], slot_mapping)
     elif kv_cache_dtype in ("fp8", "fp8_e4m3"):
         if key_cache.element_size() != 1:
             raise ValueError("fp8 KV cache must be a 1-byte tensor (float8_e4m3fn or uint8)")

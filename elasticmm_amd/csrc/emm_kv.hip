@@ -860,6 +860,119 @@ int append_fp8(const void *const *k, const void *const *v, void *const *kc, void
 }
 
 // ----------------------------------------------------------------------------
+// reshape_and_cache, flash layout with free cache strides (e.g. the head-major
+// pool [num_blocks, num_heads, block_size, head_size])
+// ----------------------------------------------------------------------------
+struct StridedParams {
+  const char *key[EMM_MAX_LAYERS];
+  const char *value[EMM_MAX_LAYERS];
+  char *key_cache[EMM_MAX_LAYERS];
+  char *value_cache[EMM_MAX_LAYERS];
+  const int64_t *slot_mapping;
+  int64_t num_tokens;
+  int64_t row_bytes; // num_heads * head_bytes
+  int64_t key_stride; // bytes
+  int64_t value_stride;
+  int64_t num_blocks;
+  int64_t block_stride; // bytes between blocks, between the slots of a block, between heads
+  int64_t page_stride;
+  int64_t head_stride;
+  int32_t block_size;
+  int32_t head_bytes;
+};
+
+// One wave moves one token row of K or V; the row is cut into heads, head h of slot (b, o) goes to
+// cache + b * block_stride + o * page_stride + h * head_stride. No transpose happens below the
+// size of a head row (256 bytes for head_size 128 in 16 bits), so no staging is needed: every
+// store instruction still covers whole head rows.
+// grid: x = groups of 4 tokens, y = 2 (K, V), z = layers.
+template <typename V>
+__global__ __launch_bounds__(kThreads) void emm_append_strided_kernel(const StridedParams p) {
+  constexpr int64_t VB = sizeof(V);
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const uint32_t kv = blockIdx.y, l = blockIdx.z;
+  const int64_t t = (int64_t)blockIdx.x * kWavesPerGroup + wave;
+  if (t >= p.num_tokens) return;
+  const char *src = (kv == 0 ? p.key[l] : p.value[l]) + t * (kv == 0 ? p.key_stride : p.value_stride);
+  char *dst_base = kv == 0 ? p.key_cache[l] : p.value_cache[l];
+  int64_t s = ld<int64_t, false>((const char *)(p.slot_mapping + t));
+  int64_t off = (int64_t)lane * VB;
+  V v;
+  if (off < p.row_bytes) v = ld_stream<V, 0>(src + off); // issued before the slot is waited for
+  s = uniform64(s);
+  if ((uint64_t)s >= (uint64_t)(p.num_blocks * p.block_size)) return;
+  const int64_t blk = s / p.block_size;
+  const int64_t pos = s - blk * p.block_size;
+  char *dst = dst_base + blk * p.block_stride + pos * p.page_stride;
+  while (off < p.row_bytes) {
+    const uint32_t h = (uint32_t)off / (uint32_t)p.head_bytes;
+    const uint32_t in = (uint32_t)off - h * (uint32_t)p.head_bytes;
+    st_stream<V, 0>(dst + (int64_t)h * p.head_stride + in, v);
+    off += 64 * VB;
+    if (off < p.row_bytes) v = ld_stream<V, 0>(src + off);
+  }
+}
+
+int append_strided(const void *const *k, const void *const *v, void *const *kc, void *const *vc, int num_layers,
+                   const int64_t *slot_mapping, int64_t num_tokens, int num_heads, int64_t head_bytes,
+                   int block_size, int64_t num_blocks, int64_t ks, int64_t vs, int64_t block_stride,
+                   int64_t page_stride, int64_t head_stride, hipStream_t s, const char *what) {
+  if (num_layers < 0 || num_layers > EMM_MAX_LAYERS)
+    return fail(EMM_EINVAL, "%s: num_layers=%d outside [0, %d]", what, num_layers, EMM_MAX_LAYERS);
+  if (num_tokens < 0 || num_heads < 0 || head_bytes < 0 || block_size <= 0 || num_blocks < 0 || ks < 0 || vs < 0 ||
+      block_stride < 0 || page_stride < 0 || head_stride < 0)
+    return fail(EMM_EINVAL, "%s: negative size", what);
+  const int64_t row_bytes = (int64_t)num_heads * head_bytes;
+  if (num_tokens == 0 || row_bytes == 0 || num_layers == 0) return EMM_OK;
+  if (head_bytes > 0x7fffffffLL || row_bytes > 0xffffffffLL) return fail(EMM_EINVAL, "%s: row too long", what);
+  if (!k || !v || !kc || !vc || !slot_mapping) return fail(EMM_EINVAL, "%s: null pointer", what);
+  if (ks < row_bytes || vs < row_bytes) return fail(EMM_EINVAL, "%s: token stride smaller than the row", what);
+  if (head_stride < head_bytes || page_stride < head_bytes)
+    return fail(EMM_EINVAL, "%s: head / page stride smaller than a head row", what);
+  if ((num_tokens + kWavesPerGroup - 1) / kWavesPerGroup > 0x7fffffffLL)
+    return fail(EMM_EINVAL, "%s: too many tokens", what);
+  StridedParams p;
+  memset(&p, 0, sizeof(p));
+  int al = 16;
+  for (int l = 0; l < num_layers; ++l) {
+    if (!k[l] || !v[l] || !kc[l] || !vc[l]) return fail(EMM_EINVAL, "%s: null tensor pointer at layer %d", what, l);
+    p.key[l] = (const char *)k[l];
+    p.value[l] = (const char *)v[l];
+    p.key_cache[l] = (char *)kc[l];
+    p.value_cache[l] = (char *)vc[l];
+    al = common_align(al, k[l]);
+    al = common_align(al, v[l]);
+    al = common_align(al, kc[l]);
+    al = common_align(al, vc[l]);
+  }
+  p.slot_mapping = slot_mapping;
+  p.num_tokens = num_tokens;
+  p.row_bytes = row_bytes;
+  p.key_stride = ks;
+  p.value_stride = vs;
+  p.num_blocks = num_blocks;
+  p.block_stride = block_stride;
+  p.page_stride = page_stride;
+  p.head_stride = head_stride;
+  p.block_size = block_size;
+  p.head_bytes = (int32_t)head_bytes;
+  int vec = al;
+  while (vec > 1 && (head_bytes % vec || ks % vec || vs % vec || block_stride % vec || page_stride % vec ||
+                     head_stride % vec))
+    vec >>= 1;
+  const dim3 grid((uint32_t)((num_tokens + kWavesPerGroup - 1) / kWavesPerGroup), 2, (uint32_t)num_layers);
+  switch (vec) {
+  case 16: emm_append_strided_kernel<u32x4><<<grid, kThreads, 0, s>>>(p); break;
+  case 8: emm_append_strided_kernel<u32x2><<<grid, kThreads, 0, s>>>(p); break;
+  case 4: emm_append_strided_kernel<uint32_t><<<grid, kThreads, 0, s>>>(p); break;
+  case 2: emm_append_strided_kernel<uint16_t><<<grid, kThreads, 0, s>>>(p); break;
+  default: emm_append_strided_kernel<uint8_t><<<grid, kThreads, 0, s>>>(p); break;
+  }
+  return check_launch(what);
+}
+
+// ----------------------------------------------------------------------------
 // reshape_and_cache, paged-attention layout: the one place where source and
 // destination layouts transpose, staged through LDS
 // ----------------------------------------------------------------------------
@@ -1340,6 +1453,19 @@ int emm_reshape_and_cache_fp8_layers(const void *const *key_ptrs, const void *co
                     slot_mapping, num_tokens, row_elems, key_stride_elems, value_stride_elems,
                     num_slots, k_scales, v_scales, src_dtype, as_stream(stream),
                     "emm_reshape_and_cache_fp8_layers");
+}
+
+int emm_reshape_and_cache_strided(const void *const *key_ptrs, const void *const *value_ptrs,
+                                  void *const *key_cache_ptrs, void *const *value_cache_ptrs,
+                                  int num_layers, const int64_t *slot_mapping, int64_t num_tokens,
+                                  int num_heads, int64_t head_bytes, int block_size, int64_t num_blocks,
+                                  int64_t key_stride_bytes, int64_t value_stride_bytes,
+                                  int64_t block_stride_bytes, int64_t page_stride_bytes,
+                                  int64_t head_stride_bytes, emm_stream_t stream) {
+  return append_strided(key_ptrs, value_ptrs, key_cache_ptrs, value_cache_ptrs, num_layers, slot_mapping,
+                        num_tokens, num_heads, head_bytes, block_size, num_blocks, key_stride_bytes,
+                        value_stride_bytes, block_stride_bytes, page_stride_bytes, head_stride_bytes,
+                        as_stream(stream), "emm_reshape_and_cache_strided");
 }
 
 int emm_reshape_and_cache_paged(const void *key, const void *value, void *key_cache, void *value_cache,

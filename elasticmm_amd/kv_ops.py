@@ -321,6 +321,56 @@ def reshape_and_cache(key: torch.Tensor, value: torch.Tensor, key_cache: torch.T
         raise TypeError(f"unsupported source/cache element sizes {eb}/{ceb}")
 
 
+def reshape_and_cache_strided(keys: Sequence[torch.Tensor], values: Sequence[torch.Tensor],
+                              key_caches: Sequence[torch.Tensor], value_caches: Sequence[torch.Tensor],
+                              slot_mapping: torch.Tensor) -> None:
+    """The flash-layout append for caches that are strided views ``[NB, bs, H, D]`` (stride 1 along D),
+    such as a head-major pool ``[NB, H, bs, D]`` seen through ``permute(0, 2, 1, 3)``. Same-width copy;
+    one launch for all layers given (they must share shapes and strides)."""
+    lib = _lib.load()
+    L = len(keys)
+    if not (len(values) == len(key_caches) == len(value_caches) == L):
+        raise ValueError("per-layer lists differ in length")
+    if L == 0:
+        return
+    geom = None
+    for l in range(L):
+        k, v, kc, vc = keys[l], values[l], key_caches[l], value_caches[l]
+        for t in (k, v, kc, vc):
+            _require_gpu(t, "reshape_and_cache_strided")
+        if k.dim() != 3 or v.shape != k.shape:
+            raise ValueError("key and value must be [num_tokens, num_heads, head_size] of one shape")
+        T, H, D = (int(x) for x in k.shape)
+        if kc.dim() != 4 or tuple(kc.shape[2:]) != (H, D) or vc.shape != kc.shape or vc.stride() != kc.stride():
+            raise ValueError("caches must be [num_blocks, block_size, num_heads, head_size] views of one geometry")
+        eb = k.element_size()
+        if kc.element_size() != eb or vc.element_size() != eb or v.element_size() != eb:
+            raise TypeError("reshape_and_cache_strided copies same-width elements only")
+        if D > 1 and kc.stride(3) != 1:
+            raise ValueError("head rows of the cache must be contiguous")
+        _, _, ks = _row_geometry(k, "key")
+        _, _, vs = _row_geometry(v, "value")
+        NB, bs = int(kc.shape[0]), int(kc.shape[1])
+        g = (T, H, D, eb, NB, bs, ks, vs, kc.stride(0), kc.stride(1), kc.stride(2))
+        if geom is None:
+            geom = g
+        elif g != geom:
+            raise ValueError(f"layer {l}: geometry differs from layer 0")
+    T, H, D, eb, NB, bs, ks, vs, sb, sp, sh = geom
+    slot_mapping = _check_slot_mapping(slot_mapping, T)
+    stream = _stream_ptr(keys[0].device)
+    for l0 in range(0, L, EMM_MAX_LAYERS):
+        sl = slice(l0, l0 + EMM_MAX_LAYERS)
+        n = len(keys[sl])
+        check(lib.emm_reshape_and_cache_strided(ptr_table([t.data_ptr() for t in keys[sl]]),
+                                                ptr_table([t.data_ptr() for t in values[sl]]),
+                                                ptr_table([t.data_ptr() for t in key_caches[sl]]),
+                                                ptr_table([t.data_ptr() for t in value_caches[sl]]), n,
+                                                slot_mapping.data_ptr(), T, H, D * eb, bs, NB, ks * eb, vs * eb,
+                                                sb * eb, sp * eb, sh * eb, stream),
+              "emm_reshape_and_cache_strided")
+
+
 def _paged_geometry(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor):
     """Checks one layer of a paged-layout append; returns (T, H, D, bs, NB, ks, vs, cache_elem_bytes)."""
     for t in (key, value, key_cache, value_cache):

@@ -193,6 +193,33 @@ int emm_reshape_and_cache_fp8_layers(const void *const *key_ptrs,
                                      emm_stream_t stream);
 
 /*
+ * reshape_and_cache (flash layout, free cache strides) — the same append for a
+ * cache whose blocks, slots and heads are block_stride / page_stride /
+ * head_stride bytes apart, e.g. the head-major pool
+ * [num_blocks, num_heads, block_size, head_size] that vLLM passes to
+ * reshape_and_cache_flash as a permuted view: head h of token t goes to
+ * cache + b * block_stride + o * page_stride + h * head_stride with
+ * b, o = divmod(slot_mapping[t], block_size); head rows (head_bytes) stay
+ * contiguous. One launch for num_layers layers (HOST pointer tables as in
+ * emm_reshape_and_cache_layers; all layers share the geometry). Same-width
+ * copy only. Same call sites as emm_reshape_and_cache
+ * (elasticmm/engine/v0/worker_steps.py:281, :438).
+ */
+int emm_reshape_and_cache_strided(const void *const *key_ptrs,
+                                  const void *const *value_ptrs,
+                                  void *const *key_cache_ptrs,
+                                  void *const *value_cache_ptrs, int num_layers,
+                                  const int64_t *slot_mapping,
+                                  int64_t num_tokens, int num_heads,
+                                  int64_t head_bytes, int block_size,
+                                  int64_t num_blocks, int64_t key_stride_bytes,
+                                  int64_t value_stride_bytes,
+                                  int64_t block_stride_bytes,
+                                  int64_t page_stride_bytes,
+                                  int64_t head_stride_bytes,
+                                  emm_stream_t stream);
+
+/*
  * reshape_and_cache (paged-attention layout) — append into the transposed pool
  * of vLLM's PagedAttention backends:
  *   key_cache   [num_blocks, num_heads, head_size / x, block_size, x]

@@ -349,6 +349,44 @@ def test_append_out_of_range_slot_is_skipped():
 
 
 # ------------------------------------------------------------------ fp8
+def test_append_into_head_major_and_padded_caches():
+    """Strided cache views: a head-major pool [NB, H, bs, D] seen as [NB, bs, H, D], and a pool whose
+    blocks are padded. The oracle appends into the same views on the CPU; the whole underlying
+    storage is compared, so the padding must stay untouched."""
+    g = torch.Generator().manual_seed(41)
+    for dtype, NB, bs, H, D, T, L in ((torch.bfloat16, 48, 16, 4, 128, 500, 3), (torch.float16, 20, 8, 3, 20, 77, 1)):
+        slots = make_slots(NB * bs, T, 41, pad_frac=0.1)
+        keys = [torch.randn((T, H, D), generator=g).to(dtype) for _ in range(L)]
+        values = [torch.randn((T, H, D), generator=g).to(dtype) for _ in range(L)]
+        # head-major storage
+        store_c = [torch.full((2, NB, H, bs, D), 3.0, dtype=dtype) for _ in range(L)]
+        store_g = [t.to(DEV) for t in store_c]
+        for l in range(L):
+            kc, vc = store_g[l][0].permute(0, 2, 1, 3), store_g[l][1].permute(0, 2, 1, 3)
+            assert not kc.is_contiguous()
+            cache_ops.reshape_and_cache_flash(keys[l].to(DEV), values[l].to(DEV), kc, vc, slots.to(DEV), "auto")
+            valid = slots >= 0
+            b, o = slots[valid] // bs, slots[valid] % bs
+            store_c[l][0].permute(0, 2, 1, 3)[b, o] = keys[l][valid]
+            store_c[l][1].permute(0, 2, 1, 3)[b, o] = values[l][valid]
+            assert same_bits(store_g[l], store_c[l]), f"head-major, layer {l}"
+            # brute-force witness on a few tokens
+            t = int(valid.nonzero()[0])
+            assert torch.equal(store_g[l][0, int(slots[t]) // bs, :, int(slots[t]) % bs, :].cpu(), keys[l][t])
+        # padded blocks, all layers in one launch
+        pad_c = [torch.full((2, NB, bs + 1, H, D + 8), 5.0, dtype=dtype) for _ in range(L)]
+        pad_g = [t.to(DEV) for t in pad_c]
+        kv_ops.reshape_and_cache_strided([k.to(DEV) for k in keys], [v.to(DEV) for v in values],
+                                         [t[0, :, :bs, :, :D] for t in pad_g], [t[1, :, :bs, :, :D] for t in pad_g],
+                                         slots.to(DEV))
+        for l in range(L):
+            valid = slots >= 0
+            b, o = slots[valid] // bs, slots[valid] % bs
+            pad_c[l][0, :, :bs, :, :D][b, o] = keys[l][valid]
+            pad_c[l][1, :, :bs, :, :D][b, o] = values[l][valid]
+            assert same_bits(pad_g[l], pad_c[l]), f"padded, layer {l}"
+
+
 # ---------------------------------------------------------------- append, paged-attention layout
 def paged_slots(NB, bs, T, seed, whole_frac=0.6, pad_frac=0.05, phase=0):
     """A slot table shaped like a serving step: prompts that fill whole blocks in order (the first
