@@ -777,6 +777,132 @@ def test_cfg2_full_size_migration_properties():
     torch.cuda.empty_cache()
 
 
+def test_cfg4_full_size_fp8_properties():
+    """fp8 70B-class per-GPU shape at full size: 80 x [2,20000,16,8,128] e4m3 (52 GB per pool), 64 requests of
+    1k-8k tokens. Byte moves are checked with torch's device indexing, the conversions against the CPU oracle on
+    samples copied back."""
+    L, NB, bs, H, D = 80, 20000, 16, 8, 128
+    torch.cuda.empty_cache()
+    free, _ = torch.cuda.mem_get_info()
+    need = 2 * L * 2 * NB * bs * H * D + (16 << 30)
+    if free < need:
+        pytest.skip(f"needs {need >> 30} GiB of free HBM, have {free >> 30}")
+    say("cfg4 full size: two fp8 pools of 52 GB")
+    g = torch.Generator().manual_seed(4)
+    lens = torch.randint(1024, 8193, (64,), generator=g)
+    nblk = [(int(t) + 15) // 16 for t in lens]
+    total = sum(nblk)
+    perm_s = torch.randperm(NB, generator=g)[:total].to(DEV)
+    perm_d = torch.randperm(NB, generator=g)[:total].to(DEV)
+    k_scales = torch.rand(L, generator=g) * 0.09 + 0.01
+    v_scales = torch.rand(L, generator=g) * 0.09 + 0.01
+    src = torch.empty((L, 2, NB, bs, H, D), dtype=torch.uint8, device=DEV)
+    src.random_(0, 256)  # every byte value, NaN encodings included
+    dst = torch.full_like(src, 0x5A)
+    sp, dp = PoolView(src), PoolView(dst)
+    off = 0
+    tables = []
+    for n in nblk:
+        si, di = perm_s[off:off + n], perm_d[off:off + n]
+        tables.append((si, di))
+        kv_ops.kv_unpack(dp, di, kv_ops.kv_pack(sp, si))
+        off += n
+    torch.cuda.synchronize()
+    say(f"cfg4 full size: moved {total} blocks, checking")
+    for r, (si, di) in enumerate(tables):
+        for l in range(r % 7, L, 7):
+            ok = bool(torch.equal(dst[l][:, di], src[l][:, si]))
+            assert ok, f"request {r} layer {l}"
+    moved = torch.zeros(NB, dtype=torch.bool, device=DEV)
+    moved[perm_d] = True
+    rest = (~moved).nonzero().squeeze(1)
+    for l in range(0, L, 5):
+        ok = bool((dst[l][:, rest] == 0x5A).all())
+        assert ok, f"layer {l}: an untouched block changed"
+    del dst, dp
+    torch.cuda.empty_cache()
+    # quantising append of one step into all 80 layers with one launch
+    T = 8448
+    slots = make_slots(NB * bs, T, 4)
+    gd = torch.Generator(device=DEV).manual_seed(4)
+    keys = [(torch.randn((T, H, D), device=DEV, generator=gd) * 2).to(torch.bfloat16) for _ in range(L)]
+    values = [(torch.randn((T, H, D), device=DEV, generator=gd) * 2).to(torch.bfloat16) for _ in range(L)]
+    before = {l: src[l].cpu() for l in (0, 41, 79)}
+    cache_ops.reshape_and_cache_flash_layers(keys, values, list(src.unbind(0)), slots.to(DEV), "fp8",
+                                             k_scales.to(DEV), v_scales.to(DEV))
+    for l, ref in before.items():
+        orc.c_reshape_and_cache_fp8(keys[l].cpu(), values[l].cpu(), ref[0], ref[1], slots, float(k_scales[l]),
+                                    float(v_scales[l]))
+        assert same_bits(src[l], ref), f"fp8 append, layer {l}"
+    del keys, values, before
+    # dequantising unpack of the first 8 requests into a bf16 pool
+    dq = torch.full((L, 2, NB, bs, H, D), -3.0, dtype=torch.bfloat16, device=DEV)
+    dqp = PoolView(dq)
+    for si, di in tables[:8]:
+        kv_ops.kv_unpack_dequant_fp8(dqp, di, kv_ops.kv_pack(sp, si), k_scales, v_scales)
+    torch.cuda.synchronize()
+    for r in (0, 7):
+        si, di = tables[r]
+        for l in (0, 33, 79):
+            for kv, sc in ((0, k_scales), (1, v_scales)):
+                q = src[l][kv, si[:40]].cpu().numpy()
+                got = dq[l][kv, di[:40]].cpu().view(torch.int16).numpy().view(np.uint16)
+                want = orc.c_dequant_fp8(q, float(sc[l]), torch.bfloat16)
+                assert (got == want).all(), f"dequant-unpack request {r} layer {l} kv {kv}"
+    ok = bool((dq[17][:, rest[:2000]] == -3.0).all())
+    assert ok, "dequant-unpack touched a block outside the tables"
+    del src, sp, dq, dqp
+    torch.cuda.empty_cache()
+
+
+def test_cfg5_full_size_rebalance_properties():
+    """Elastic rebalancing at full size: a 200 GB bf16 pool in the Qwen2-7B layout, copy_blocks of half of the live
+    blocks to disjoint free blocks (54 500 pairs, 100 GB), with the vision-embedding gather of 128 images in between."""
+    L, NB, bs, H, D = 28, 218000, 16, 4, 128
+    torch.cuda.empty_cache()
+    free, _ = torch.cuda.mem_get_info()
+    need = L * 2 * NB * bs * H * D * 2 + (24 << 30)
+    if free < need:
+        pytest.skip(f"needs {need >> 30} GiB of free HBM, have {free >> 30}")
+    say("cfg5 full size: one pool of 200 GB")
+    pool = torch.empty((L, 2, NB, bs, H, D), dtype=torch.bfloat16, device=DEV)
+    gd = torch.Generator(device=DEV).manual_seed(5)
+    for l in range(L):
+        pool[l].normal_(0.0, 0.5, generator=gd)
+    g = torch.Generator().manual_seed(5)
+    perm = torch.randperm(NB, generator=g)
+    live, free_ids = perm[:NB // 2].to(DEV), perm[NB // 2:].to(DEV)
+    for l in range(L):
+        pool[l][:, free_ids] = -1.0  # canary in every free block
+    P = live.numel() // 2
+    mapping = torch.stack([live[:P], free_ids[:P]], 1).contiguous()
+    sums = [pool[l][:, live].view(torch.int16).sum(dtype=torch.int64) for l in (0, 14, 27)]
+    imgs = torch.randint(64, 2305, (128,), generator=g).tolist()
+    embeds = [torch.randn((n, 3584), device=DEV, generator=gd).to(torch.bfloat16) for n in imgs]
+    pv = PoolView(pool)
+    eighth = P // 8
+    cat = None
+    for k in range(8):  # copy_blocks in eight slices with the vision gather in between
+        hi = P if k == 7 else (k + 1) * eighth
+        kv_ops.copy_blocks(pv, mapping[k * eighth:hi])
+        if k == 3:
+            cat = kv_ops.concat_rows(embeds)
+    torch.cuda.synchronize()
+    say("cfg5 full size: checking")
+    for l in range(L):
+        ok = bool(torch.equal(pool[l][:, mapping[:, 1]], pool[l][:, mapping[:, 0]]))
+        assert ok, f"layer {l}: a destination differs from its source"
+        ok = bool((pool[l][:, free_ids[P:]] == -1.0).all())
+        assert ok, f"layer {l}: a free block outside the mapping changed"
+    for l, s0 in zip((0, 14, 27), sums):
+        ok = bool(pool[l][:, live].view(torch.int16).sum(dtype=torch.int64) == s0)
+        assert ok, f"layer {l}: a live block changed"
+    ok = bool(torch.equal(cat, torch.cat(embeds, 0)))
+    assert ok, "vision gather differs from torch.cat"
+    del pool, pv, embeds, cat
+    torch.cuda.empty_cache()
+
+
 # ------------------------------------------------------------------ prepared plan / HIP graph
 def test_layered_append_plan_reuse_and_graph_replay():
     """A prepared whole-step append is reused with new data and new slots, and the per-layer
