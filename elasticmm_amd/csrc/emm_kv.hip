@@ -1021,8 +1021,9 @@ constexpr int kPagedSeg = 256;   // row elements per tile
 // contiguous bytes per group and a whole block 16 KiB.
 // Phase 2, V: for a whole run of 16 tokens (at most one per tile) lane q gathers one 16-byte
 // piece of the run's [element][16 tokens] region from a column of the tile (8 or 16
-// element-sized LDS reads); the other owned tokens are stored one element per lane, token
-// fastest, which the memory pipeline merges where tokens have neighbouring slots.
+// element-sized LDS reads); the other owned tokens are stored one element per lane, token by
+// token (every such store is a partial write of a 32-byte sector, which is what the layout costs
+// for tokens that do not fill a block; the lane order makes no measurable difference).
 // grid: x = token tiles, y = 2 * row segments (bit 0: K | V), z = layers.
 template <int CE, int SRC_DTYPE>
 __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(const PagedParams p) {
