@@ -552,6 +552,12 @@ def extended(dev):
     med, _ = timed(lambda: kv_ops.concat_rows(embeds, out=outbuf), 10)
     out["rebalance_200GB"]["vision_concat"] = {"images": 128, "rows": sum(imgs), "ms": round(med, 4),
                                                "GBps": round(vis_bytes / (med * 1e-3) / 1e9, 1)}
+    # the same gather from segments prepared when the embeddings entered the cache (what
+    # KVWorker.gather_vision_embeddings does): the host reads two fields per image instead of the tensors
+    prepared = [kv_ops.RowSource(e) for e in embeds]
+    med, _ = timed(lambda: kv_ops.concat_row_sources(prepared, out=outbuf), 10)
+    out["rebalance_200GB"]["vision_concat"]["prepared_segments_ms"] = round(med, 4)
+    out["rebalance_200GB"]["vision_concat"]["prepared_segments_GBps"] = round(vis_bytes / (med * 1e-3) / 1e9, 1)
     med_t, _ = timed(lambda: torch.cat(embeds, 0, out=outbuf), 10)
     out["rebalance_200GB"]["vision_concat"]["torch_cat_GBps"] = round(vis_bytes / (med_t * 1e-3) / 1e9, 1)
     quarter = mapping[:P // 8]

@@ -13,7 +13,7 @@ from .build import library_path
 
 EMM_KV_ABI_VERSION = 1
 EMM_MAX_LAYERS = 96
-EMM_MAX_SEGMENTS = 96
+EMM_MAX_SEGMENTS = 128
 EMM_DTYPE_BF16 = 0
 EMM_DTYPE_F16 = 1
 

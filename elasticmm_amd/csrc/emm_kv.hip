@@ -1244,7 +1244,7 @@ int append_paged(const void *const *k, const void *const *v, void *const *kc, vo
 // ----------------------------------------------------------------------------
 // concat_rows: ragged segments -> one contiguous buffer
 // ----------------------------------------------------------------------------
-constexpr int kSegGroup = 12; // segments per group of the two-level tile -> segment search
+constexpr int kSegGroup = 16; // segments per group of the two-level tile -> segment search
 constexpr int kSegGroups = EMM_MAX_SEGMENTS / kSegGroup;
 static_assert(kSegGroups * kSegGroup == EMM_MAX_SEGMENTS, "segment table must split into whole groups");
 
@@ -1263,7 +1263,7 @@ __global__ __launch_bounds__(kThreads) void emm_concat_rows_kernel(const ConcatP
   const uint32_t w = blockIdx.x;
   // Wave-uniform search for the last segment whose first tile is <= w, as two rounds
   // of counting over small fixed tables (two dependent fetches of the argument block
-  // instead of the seven of a binary search over 96 entries).
+  // instead of the seven of a binary search over 128 entries).
   int g = -1;
 #pragma unroll
   for (int k = 0; k < kSegGroups; ++k) g += p.group_start[k] <= w ? 1 : 0;

@@ -569,6 +569,16 @@ def reshape_and_cache_layers(keys: Sequence[torch.Tensor], values: Sequence[torc
     LayeredAppend(keys, values, key_caches, value_caches, k_scales, v_scales)(slot_mapping)
 
 
+def _launch_concat(lib, ptrs, sizes, out: torch.Tensor, stream) -> None:
+    off = 0
+    for i0 in range(0, len(ptrs), EMM_MAX_SEGMENTS):
+        n = min(EMM_MAX_SEGMENTS, len(ptrs) - i0)
+        srcs = (_lib.c_void_p * n)(*ptrs[i0:i0 + n])
+        nbytes = (_lib.c_int64 * n)(*sizes[i0:i0 + n])
+        check(lib.emm_concat_rows(srcs, nbytes, n, out.data_ptr(), off, stream), "emm_concat_rows")
+        off += sum(sizes[i0:i0 + n])
+
+
 def concat_rows(tensors: Sequence[torch.Tensor], out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``torch.cat(tensors, dim=0)`` of ragged ``[rows_i, ...]`` tensors in one launch per
     EMM_MAX_SEGMENTS segments."""
@@ -577,26 +587,71 @@ def concat_rows(tensors: Sequence[torch.Tensor], out: Optional[torch.Tensor] = N
     if not tensors:
         raise ValueError("concat_rows: expected a non-empty list of tensors")
     first = tensors[0]
+    _require_gpu(first, "concat_rows")
+    tail, dtype, device = first.shape[1:], first.dtype, first.device
+    row_bytes = first.element_size()
+    for d in tail:
+        row_bytes *= int(d)
+    # one pass per tensor (the host time of this loop is what a short gather waits for)
+    ptrs, sizes, rows = [], [], 0
     for t in tensors:
-        _require_gpu(t, "concat_rows")
-        if t.shape[1:] != first.shape[1:] or t.dtype != first.dtype or t.device != first.device:
+        if t.shape[1:] != tail or t.dtype != dtype or t.device != device:
             raise ValueError("concat_rows: tensors differ in trailing shape / dtype / device")
-    tensors = [t if t.is_contiguous() else t.contiguous() for t in tensors]
-    rows = sum(int(t.shape[0]) for t in tensors)
-    shape = (rows,) + tuple(first.shape[1:])
+        if not t.is_contiguous():
+            t = t.contiguous()
+        r = t.shape[0]
+        rows += r
+        ptrs.append(t.data_ptr())
+        sizes.append(r * row_bytes)
+    shape = (rows,) + tuple(tail)
     if out is None:
-        out = torch.empty(shape, dtype=first.dtype, device=first.device)
-    elif tuple(out.shape) != shape or out.dtype != first.dtype or not out.is_contiguous():
-        raise ValueError("concat_rows: `out` has the wrong shape / dtype or is not contiguous")
-    stream = _stream_ptr(first.device)
-    off = 0
-    for i0 in range(0, len(tensors), EMM_MAX_SEGMENTS):
-        seg = tensors[i0:i0 + EMM_MAX_SEGMENTS]
-        srcs = ptr_table([t.data_ptr() for t in seg])
-        sizes = [t.numel() * t.element_size() for t in seg]
-        nbytes = (_lib.c_int64 * len(seg))(*sizes)
-        check(lib.emm_concat_rows(srcs, nbytes, len(seg), out.data_ptr(), off, stream), "emm_concat_rows")
-        off += sum(sizes)
+        out = torch.empty(shape, dtype=dtype, device=device)
+    elif tuple(out.shape) != shape or out.dtype != dtype or out.device != device or not out.is_contiguous():
+        raise ValueError("concat_rows: `out` has the wrong shape / dtype / device or is not contiguous")
+    _launch_concat(lib, ptrs, sizes, out, _stream_ptr(device))
+    return out
+
+
+class RowSource:
+    """A ``[rows, ...]`` GPU tensor prepared as a segment of ``concat_row_sources``: pointer, byte
+    count and shape signature are read once, when the tensor enters a cache, so that a gather of
+    many cached tensors costs a few dictionary lookups per tensor on the host instead of a dozen
+    tensor attribute reads. The object keeps the (contiguous) tensor alive."""
+    __slots__ = ("tensor", "ptr", "nbytes", "rows", "sig")
+
+    def __init__(self, t: torch.Tensor):
+        _require_gpu(t, "RowSource")
+        if t.dim() < 1:
+            raise ValueError("RowSource: expected [rows, ...]")
+        if not t.is_contiguous():
+            t = t.contiguous()
+        self.tensor = t
+        self.ptr = t.data_ptr()
+        self.nbytes = t.numel() * t.element_size()
+        self.rows = int(t.shape[0])
+        self.sig = (tuple(t.shape[1:]), t.dtype, t.device)
+
+
+def concat_row_sources(sources: Sequence[RowSource], out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``concat_rows`` over prepared segments."""
+    lib = _lib.load()
+    if not sources:
+        raise ValueError("concat_row_sources: expected a non-empty list")
+    sig = sources[0].sig
+    ptrs, sizes, rows = [], [], 0
+    for s in sources:
+        if s.sig is not sig and s.sig != sig:
+            raise ValueError("concat_row_sources: segments differ in trailing shape / dtype / device")
+        ptrs.append(s.ptr)
+        sizes.append(s.nbytes)
+        rows += s.rows
+    tail, dtype, device = sig
+    shape = (rows,) + tail
+    if out is None:
+        out = torch.empty(shape, dtype=dtype, device=device)
+    elif tuple(out.shape) != shape or out.dtype != dtype or out.device != device or not out.is_contiguous():
+        raise ValueError("concat_row_sources: `out` has the wrong shape / dtype / device or is not contiguous")
+    _launch_concat(lib, ptrs, sizes, out, _stream_ptr(device))
     return out
 
 

@@ -73,6 +73,7 @@ class KVWorker:
         self.block_size = block_size
         self.kv_cache: Optional[List[torch.Tensor]] = None
         self.ve_cache: Optional[Dict[str, torch.Tensor]] = None
+        self._ve_sources: Dict[str, Any] = {}
         self._pool: Optional[PoolView] = None
         self.link = link
         self.global_rank = global_rank
@@ -120,6 +121,7 @@ class KVWorker:
     def init_vecache(self, num_gpu_blocks: int = 0, num_cpu_blocks: int = 0) -> List[int]:
         """Vision embeddings are kept per request id (worker.py:431-437)."""
         self.ve_cache = {}
+        self._ve_sources = {}
         self.ve_cache_capacity = num_gpu_blocks
         return []
 
@@ -392,15 +394,33 @@ class KVWorker:
         if self.ve_cache is None:
             raise RuntimeError("Vision embedding cache not initialized")
         self.ve_cache[request_id] = ve_data
+        self._ve_sources.pop(request_id, None)
 
     def gather_vision_embeddings(self, request_ids: Sequence[str]) -> Optional[torch.Tensor]:
         """The prefill input built at worker_steps.py:252-267: embeddings of the batch's
-        requests that are cached, concatenated on dim 0 (a single tensor passes through)."""
+        requests that are cached, concatenated on dim 0 (a single tensor passes through).
+
+        ``ve_cache`` stays the plain dict of the reference (callers may assign into it); next to it
+        a prepared segment per entry is kept and revalidated by identity, so that the host cost of
+        a gather is a few dictionary lookups per request."""
         if self.ve_cache is None:
             return None
-        vision_embeds = [self.ve_cache[r] for r in request_ids if r in self.ve_cache]
-        if not vision_embeds:
+        cache, prepared = self.ve_cache, self._ve_sources
+        hits = [(r, cache[r]) for r in request_ids if r in cache]
+        if not hits:
             return None
-        if len(vision_embeds) == 1:
-            return vision_embeds[0]
-        return kv_ops.concat_rows(vision_embeds)
+        if len(hits) == 1:
+            return hits[0][1]
+        sources = []
+        for r, t in hits:
+            s = prepared.get(r)
+            if s is None or s.tensor is not t:
+                s = kv_ops.RowSource(t)
+                if s.tensor is not t:  # a non-contiguous entry: cache its contiguous copy
+                    cache[r] = s.tensor
+                prepared[r] = s
+            sources.append(s)
+        if len(prepared) > 2 * len(cache) + 64:  # entries of requests that left the cache
+            for r in [r for r in prepared if r not in cache]:
+                del prepared[r]
+        return kv_ops.concat_row_sources(sources)

@@ -40,7 +40,7 @@ extern "C" {
 
 #define EMM_KV_ABI_VERSION 1
 #define EMM_MAX_LAYERS 96   /* layer pointers carried in one kernel argument block */
-#define EMM_MAX_SEGMENTS 96  /* ragged segments carried by one emm_concat_rows launch */
+#define EMM_MAX_SEGMENTS 128 /* ragged segments carried by one emm_concat_rows launch */
 
 /* error codes */
 #define EMM_OK 0

@@ -645,6 +645,20 @@ def test_concat_rows_ragged():
         w.write_vision_blocks(f"r{i}", s.to(DEV))
     assert same_bits(w.gather_vision_embeddings(["r0", "zz", "r2"]), torch.cat([segs[0], segs[2]], 0))
     assert w.gather_vision_embeddings(["r1"]) is w.extract_vision_blocks("r1")
+    # the prepared segments follow the cache: an entry replaced through the dict itself, a non-contiguous
+    # entry, a dropped entry, and a repeated gather
+    repl = torch.randn((5, segs[0].shape[1]), generator=g).to(segs[0].dtype)
+    w.ve_cache["r0"] = repl.to(DEV)
+    wide = torch.randn((4, 2 * segs[0].shape[1]), generator=g).to(segs[0].dtype)
+    w.ve_cache["r3"] = wide.to(DEV)[:, ::2]
+    want = torch.cat([repl, segs[2], wide[:, ::2]], 0)
+    for _ in range(2):
+        assert same_bits(w.gather_vision_embeddings(["r0", "r2", "r3"]), want)
+    del w.ve_cache["r2"]
+    assert same_bits(w.gather_vision_embeddings(["r0", "r2", "r3"]), torch.cat([repl, wide[:, ::2]], 0))
+    with pytest.raises(ValueError):
+        w.ve_cache["bad"] = torch.zeros((2, 3), dtype=segs[0].dtype, device=DEV)
+        w.gather_vision_embeddings(["r0", "bad"])
 
 
 # ------------------------------------------------------------------ worker protocol
