@@ -966,6 +966,85 @@ def test_layered_append_plan_reuse_and_graph_replay():
             assert same_bits(pool_graph[l], pool_c[l]), f"graph replay {it}, layer {l}"
 
 
+def test_migration_step_replayed_from_a_hip_graph():
+    """pack -> unpack -> fused migrate -> copy_blocks -> paged append -> vision gather captured once in a HIP
+    graph over fixed buffers and device-resident tables; every replay (new tables, new data, eager work and
+    synchronisations in between) must equal the oracle."""
+    L, NB, bs, H, D, n, T = 3, 48, 16, 2, 64, 9, 40
+    g = torch.Generator().manual_seed(23)
+    src_c = cpu_pool(L, NB, bs, H, D, torch.bfloat16, 23)
+    src = to_dev(src_c)
+    dst = [torch.zeros_like(t) for t in src]
+    mig = [torch.zeros_like(t) for t in src]
+    sp, dp, mp = PoolView(src), PoolView(dst), PoolView(mig)
+    si = torch.zeros(n, dtype=torch.long, device=DEV)
+    di = torch.zeros(n, dtype=torch.long, device=DEV)
+    mapping = torch.zeros((4, 2), dtype=torch.long, device=DEV)
+    buf = torch.empty(sp.packed_shape(n), dtype=torch.bfloat16, device=DEV)
+    key = torch.zeros((T, H, D), dtype=torch.bfloat16, device=DEV)
+    value = torch.zeros_like(key)
+    slots_g = torch.zeros(T, dtype=torch.long, device=DEV)
+    kc = torch.zeros((NB, H, D // 8, bs, 8), dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros((NB, H, D, bs), dtype=torch.bfloat16, device=DEV)
+    segs = [torch.zeros((r, 24), dtype=torch.bfloat16, device=DEV) for r in (5, 1, 7)]
+    sources = [kv_ops.RowSource(t) for t in segs]
+    cat = torch.empty((13, 24), dtype=torch.bfloat16, device=DEV)
+
+    def step():
+        kv_ops.kv_pack(sp, si, out=buf)
+        kv_ops.kv_unpack(dp, di, buf)
+        kv_ops.kv_migrate(sp, si, mp, di)
+        kv_ops.copy_blocks(dp, mapping)
+        cache_ops.reshape_and_cache(key, value, kc, vc, slots_g, "auto")
+        kv_ops.concat_row_sources(sources, out=cat)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    for t in (*dst, *mig, kc, vc):
+        t.zero_()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    dst_c = [torch.zeros_like(t) for t in src_c]
+    mig_c = [torch.zeros_like(t) for t in src_c]
+    kc_c, vc_c = torch.zeros(kc.shape, dtype=torch.bfloat16), torch.zeros(vc.shape, dtype=torch.bfloat16)
+    for it in range(4):
+        perm = torch.randperm(NB, generator=g)
+        s_tab, d_tab = perm[:n], torch.randperm(NB, generator=g)[:n]
+        free = [b for b in range(NB) if b not in set(d_tab.tolist())]
+        pairs = torch.tensor([[int(d_tab[i]), free[i + it]] for i in range(4)])
+        slots = make_slots(NB * bs, T, 200 + it, pad_frac=0.1)
+        k = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+        v = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+        new_segs = [torch.randn(t.shape, generator=g).to(torch.bfloat16) for t in segs]
+        si.copy_(s_tab)
+        di.copy_(d_tab)
+        mapping.copy_(pairs)
+        slots_g.copy_(slots)
+        key.copy_(k)
+        value.copy_(v)
+        for t, c in zip(segs, new_segs):
+            t.copy_(c)
+        graph.replay()
+        torch.cuda.synchronize()
+        packed = orc.ref_extract_kv_blocks(src_c, s_tab.tolist())
+        orc.ref_write_kv_blocks(dst_c, d_tab.tolist(), packed)
+        orc.ref_write_kv_blocks(mig_c, d_tab.tolist(), packed)
+        orc.ref_copy_blocks(dst_c, pairs)
+        orc.c_reshape_and_cache_paged(k, v, kc_c, vc_c, slots)
+        assert same_bits(buf, packed), f"replay {it}: pack"
+        for l in range(L):
+            assert same_bits(dst[l], dst_c[l]), f"replay {it}: unpack + copy_blocks, layer {l}"
+            assert same_bits(mig[l], mig_c[l]), f"replay {it}: migrate, layer {l}"
+        assert same_bits(kc, kc_c) and same_bits(vc, vc_c), f"replay {it}: paged append"
+        assert same_bits(cat, torch.cat(new_segs, 0)), f"replay {it}: vision gather"
+        junk = kv_ops.kv_pack(sp, [0, 1])  # unrelated eager work between the replays
+        assert junk.shape[2] == 2
+
+
 def test_large_block_count_splits_launches():
     """More than 65 535 blocks in one call (the grid's y limit): tiny chunks keep it small."""
     NB, n = 70000, 66000
