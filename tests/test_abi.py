@@ -62,6 +62,32 @@ def test_load_and_argument_errors_without_gpu():
     assert rc == -1 and b"multiples of 16" in lib.emm_last_error()
 
 
+def test_argument_errors_of_the_layout_variants_without_gpu():
+    lib = _lib.load()
+    P = 0x1000
+    # paged-attention layout: head_size must be a multiple of x = 16 / cache element bytes
+    rc = lib.emm_reshape_and_cache_paged(P, P, P, P, P, 4, 2, 20, 16, 8, 40, 40, 0, 2, None, None, None)
+    assert rc == -1 and b"multiple of x" in lib.emm_last_error()
+    rc = lib.emm_reshape_and_cache_paged(P, P, P, P, P, 4, 2, 32, 16, 8, 64, 64, 0, 3, None, None, None)
+    assert rc == -1 and b"cache_elem_bytes" in lib.emm_last_error()
+    rc = lib.emm_reshape_and_cache_paged(P, P, P, P, P, 4, 2, 32, 16, 8, 64, 64, 0, 1, None, None, None)
+    assert rc == -1 and b"scale" in lib.emm_last_error()
+    rc = lib.emm_reshape_and_cache_paged(P, P, P, P + 8, P, 4, 2, 32, 16, 8, 64, 64, 0, 2, None, None, None)
+    assert rc == -1 and b"16-byte aligned" in lib.emm_last_error()
+    rc = lib.emm_reshape_and_cache_paged(P, P, P, P, P, 4, 2, 32, 0, 8, 64, 64, 0, 2, None, None, None)
+    assert rc == -1 and b"negative size" in lib.emm_last_error()
+    assert lib.emm_reshape_and_cache_paged(P, P, P, P, P, 0, 2, 32, 16, 8, 64, 64, 0, 2, None, None, None) == 0
+    t = _lib.ptr_table([P])
+    rc = lib.emm_reshape_and_cache_paged_layers(t, t, t, t, 97, P, 4, 2, 32, 16, 8, 64, 64, 0, 2, None, None, None)
+    assert rc == -1 and b"num_layers" in lib.emm_last_error()
+    # strided flash layout: strides must cover a head row
+    rc = lib.emm_reshape_and_cache_strided(t, t, t, t, 1, P, 4, 2, 64, 16, 8, 128, 128, 4096, 32, 64, None)
+    assert rc == -1 and b"stride smaller than a head row" in lib.emm_last_error()
+    rc = lib.emm_reshape_and_cache_strided(t, t, t, t, 1, P, 4, 2, 64, 16, 8, 100, 128, 4096, 128, 64, None)
+    assert rc == -1 and b"token stride" in lib.emm_last_error()
+    assert lib.emm_reshape_and_cache_strided(t, t, t, t, 0, P, 4, 2, 64, 16, 8, 128, 128, 4096, 128, 64, None) == 0
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "_lib", None)
     monkeypatch.setattr(_lib, "library_path", lambda: str(tmp_path / "nope.so"))
