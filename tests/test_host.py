@@ -31,6 +31,18 @@ def test_ops_refuse_cpu_tensors():
     k = torch.zeros((2, 1, 8), dtype=torch.float16)
     with pytest.raises(RuntimeError, match="GPU only"):
         kv_ops.reshape_and_cache(k, k, pool[0][0], pool[0][1], torch.tensor([0, 1]))
+    # the layout variants and the vision gather refuse them too (no CPU fallback anywhere)
+    kc = torch.zeros((4, 1, 1, 2, 8), dtype=torch.float16)
+    vc = torch.zeros((4, 1, 8, 2), dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        kv_ops.reshape_and_cache_paged(k, k, kc, vc, torch.tensor([0, 1]))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        kv_ops.reshape_and_cache_strided([k], [k], [pool[0][0].permute(0, 2, 1, 3)], [pool[0][1].permute(0, 2, 1, 3)],
+                                         torch.tensor([0, 1]))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        kv_ops.concat_rows([k, k])
+    with pytest.raises(RuntimeError, match="GPU only"):
+        kv_ops.RowSource(k)
 
 
 def test_worker_error_conventions_without_pool():
