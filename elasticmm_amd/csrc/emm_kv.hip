@@ -460,23 +460,60 @@ __device__ __forceinline__ float half_bits_to_f32(uint32_t h) {
     return f16_bits_to_f32(h);
 }
 
+// x / scale for a scale shared by a whole wave. The correctly rounded quotient is what torch's
+// cast sees, so it must be reproduced bit for bit. For 2^-30 <= |scale| <= 2^30 it is obtained
+// without the IEEE division sequence: with y = RN(1 / scale), q = RN(x * y),
+// r = fma(-q, scale, x) (exact), the result is fma(r, y, q) — checked on the device against the
+// division for every 16-bit input and 2^20 scales. Where q is not finite (x infinite or NaN, or
+// the product overflows) the correction would produce a NaN of arbitrary sign, and where q is a
+// zero it would lose the sign of -0, so q is kept in both cases.
+// Other scales take the division.
+struct Divisor {
+  float scale;
+  float recip;
+  bool exact_fast;
+};
+
+__device__ __forceinline__ Divisor make_divisor(float scale, bool allow_fast) {
+  Divisor d;
+  d.scale = scale;
+  d.recip = 1.0f / scale;
+  const float a = __builtin_fabsf(scale);
+  d.exact_fast = allow_fast && a >= 0x1p-30f && a <= 0x1p30f;
+  return d;
+}
+
+template <bool FAST>
+__device__ __forceinline__ float divide(float x, const Divisor &d) {
+  if constexpr (FAST) {
+    const float q = x * d.recip;
+    const float r = __builtin_fmaf(-q, d.scale, x);
+    const float q2 = __builtin_fmaf(r, d.recip, q);
+    // NaN, +-inf, +-0 (classes 0x267): keep q
+    return __builtin_amdgcn_classf(q, 0x267) ? q : q2;
+  } else {
+    return x / d.scale;
+  }
+}
+
 // 8 sixteen-bit values (one u32x4) -> 8 e4m3fn bytes (one u32x2), q = rne(x / scale).
-// The division is the compiler's correctly rounded IEEE sequence. A reciprocal plus one
-// fma correction step (exact for 2^-30 <= |scale| <= 2^30, verified on the device against
-// this division for every 16-bit input x 2^20 scales) was measured and gave no speed-up:
-// the kernel is bound by the 1 KiB row scatter, not by the arithmetic.
-template <int SRC_DTYPE>
-__device__ __forceinline__ u32x2 quant8(u32x4 in, float scale) {
+template <int SRC_DTYPE, bool FAST>
+__device__ __forceinline__ u32x2 quant8(u32x4 in, const Divisor &d) {
   u32x2 out;
 #pragma unroll
   for (int w = 0; w < 2; ++w) {
     const uint32_t w0 = in[w * 2], w1 = in[w * 2 + 1];
-    out[w] = f32x4_to_e4m3fn(half_bits_to_f32<SRC_DTYPE>(w0 & 0xffffu) / scale,
-                             half_bits_to_f32<SRC_DTYPE>(w0 >> 16) / scale,
-                             half_bits_to_f32<SRC_DTYPE>(w1 & 0xffffu) / scale,
-                             half_bits_to_f32<SRC_DTYPE>(w1 >> 16) / scale);
+    out[w] = f32x4_to_e4m3fn(divide<FAST>(half_bits_to_f32<SRC_DTYPE>(w0 & 0xffffu), d),
+                             divide<FAST>(half_bits_to_f32<SRC_DTYPE>(w0 >> 16), d),
+                             divide<FAST>(half_bits_to_f32<SRC_DTYPE>(w1 & 0xffffu), d),
+                             divide<FAST>(half_bits_to_f32<SRC_DTYPE>(w1 >> 16), d));
   }
   return out;
+}
+
+template <int SRC_DTYPE>
+__device__ __forceinline__ u32x2 quant8(u32x4 in, const Divisor &d) {
+  return d.exact_fast ? quant8<SRC_DTYPE, true>(in, d) : quant8<SRC_DTYPE, false>(in, d);
 }
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -600,6 +637,7 @@ struct AppendParams {
   int64_t key_stride; // bytes (copy) / elements (fp8)
   int64_t value_stride;
   int64_t num_slots;
+  int32_t fast_div; // fp8: 0 forces the IEEE division (benchmarks)
 };
 
 constexpr int kWavesPerGroup = kThreads / 64;
@@ -685,6 +723,7 @@ __global__ __launch_bounds__(kThreads) void emm_append_fp8_kernel(const AppendPa
   char *dst_base = kv == 0 ? p.key_cache[l] : p.value_cache[l];
   const int64_t stride = kv == 0 ? p.key_stride : p.value_stride;
   const float scale = kv == 0 ? p.k_scales[l] : p.v_scales[l];
+  const Divisor div = make_divisor(scale, p.fast_div != 0);
   const int64_t row = p.row_bytes; // elements
 
   int64_t slot[R];
@@ -706,8 +745,8 @@ __global__ __launch_bounds__(kThreads) void emm_append_fp8_kernel(const AppendPa
       for (int r = 0; r < R; ++r)
         if (slot[r] >= 0) {
           char *dp = dst_base + slot[r] * row;
-          const u32x2 qa = quant8<SRC_DTYPE>(a[r], scale);
-          const u32x2 qb = quant8<SRC_DTYPE>(b[r], scale);
+          const u32x2 qa = quant8<SRC_DTYPE>(a[r], div);
+          const u32x2 qb = quant8<SRC_DTYPE>(b[r], div);
           st_stream<u32x2, 1>(dp + e0, qa);
           if (e1 < row) st_stream<u32x2, 1>(dp + e1, qb);
         }
@@ -846,6 +885,7 @@ int append_fp8(const void *const *k, const void *const *v, void *const *kc, void
   p.key_stride = ks;
   p.value_stride = vs;
   p.num_slots = num_slots;
+  p.fast_div = (g_move_variant & 0x1000000) ? 0 : 1;
   const int rows = (g_append_rows == 1 || g_append_rows == 2 || g_append_rows == 4) ? g_append_rows : 1;
   dim3 grid = append_grid(num_tokens, num_layers, width == 8 ? rows : 4);
 #define EMM_FP8_LAUNCH(DT)                                                                  \
@@ -1049,6 +1089,7 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(const PagedP
 
   float scale = 1.0f;
   if constexpr (CE == 1) scale = kv == 0 ? p.k_scales[l] : p.v_scales[l];
+  const Divisor div = make_divisor(scale, true);
 
   // ---- phase 0 (wave 0): runs and the list of owned tokens ----
   if (tid < 64) {
@@ -1101,7 +1142,7 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(const PagedP
       if constexpr (CE == 2)
         *reinterpret_cast<u32x4 *>(tile + r * ROW + c * 16) = v;
       else
-        *reinterpret_cast<u32x2 *>(tile + r * ROW + c * 8) = quant8<SRC_DTYPE>(v, scale);
+        *reinterpret_cast<u32x2 *>(tile + r * ROW + c * 8) = quant8<SRC_DTYPE>(v, div);
     }
   } else {
     for (int q = tid; q < count * seg_elems; q += kThreads) {
@@ -1291,7 +1332,7 @@ int emm_abi_version(void) { return EMM_KV_ABI_VERSION; }
 
 int emm_set_move_variant(int variant) {
   const int old = g_move_variant | (g_append_rows << 12);
-  g_move_variant = variant & 0xf0fff;
+  g_move_variant = variant & 0x10f0fff;
   g_append_rows = (variant >> 12) & 0xf; // rows per wave of the append kernels
   return old;
 }

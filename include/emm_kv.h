@@ -287,7 +287,8 @@ int emm_stream_copy(const void *src, void *dst, int64_t nbytes,
 /* Tuning hook for benchmarks: 0 = library default. Bits 0-3: vectors per lane of
  * the block-move kernels (1 or 4); bits 8-11: store policy + 1 (1: non-temporal,
  * 2: sc0 sc1); bits 12-15: token rows per wave of the append kernels (1, 2, 4);
- * bits 16-19: log2 of the blocks per plane visit of pack / unpack (15 = plain order).
+ * bits 16-19: log2 of the blocks per plane visit of pack / unpack (15 = plain order);
+ * bit 24: fp8 append with the IEEE division sequence instead of the reciprocal form.
  * Process-wide, not thread-safe. Returns the previous value. */
 int emm_set_move_variant(int variant);
 

@@ -1151,6 +1151,41 @@ def test_fp8_append_scale_range_paths():
             assert (raw(vc) == want).all()
 
 
+def test_fp8_quantise_many_scales_against_the_division():
+    """The append divides through a reciprocal and one correction step wherever 2^-30 <= |scale| <= 2^30.
+    Scales whose significands are the known hard cases of that scheme (all ones, all ones minus a few ulps, one ulp
+    above a power of two, around 1.5, alternating bits) at every third exponent of the range, plus 320 random
+    scales: every bf16 and f16 input must give the byte of the oracle's correctly rounded division."""
+    import struct
+
+    def f32(bits):
+        return struct.unpack("<f", struct.pack("<I", bits))[0]
+
+    mantissas = [0, 1, 2, 3, 0x7FFFFF, 0x7FFFFE, 0x7FFFFD, 0x400000, 0x400001, 0x3FFFFF, 0x555555, 0x2AAAAA]
+    scales = [f32(((127 + e) << 23) | m) for e in range(-30, 30, 3) for m in mantissas]
+    rng = np.random.default_rng(11)
+    scales += [f32(int(b)) for b in rng.integers((127 - 30) << 23, (127 + 30) << 23, 320)]
+    scales = [s for s in scales if 2.0 ** -30 <= s <= 2.0 ** 30]
+    slots = torch.arange(64, device=DEV)
+    group = 80
+    for dtype in (torch.bfloat16, torch.float16):
+        allx = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype)
+        key = allx.view(64, 8, 128).to(DEV)
+        for g0 in range(0, len(scales), group):
+            part = scales[g0:g0 + group]
+            L = len(part)
+            pools = [torch.zeros((2, 4, 16, 8, 128), dtype=torch.uint8, device=DEV) for _ in range(L)]
+            sc = torch.tensor(part, dtype=torch.float32)
+            cache_ops.reshape_and_cache_flash_layers([key] * L, [key] * L, pools, slots, "fp8", sc, sc)
+            for l, sv in enumerate(part):
+                want = orc.c_quant_fp8(allx, float(np.float32(sv))).reshape(-1)
+                got = raw(pools[l][0])
+                bad = np.nonzero(got != want)[0]
+                assert bad.size == 0, f"{dtype} scale {sv!r}: {bad.size} mismatches, first input bits " \
+                                      f"{bad[:6].tolist()} got {got[bad[:6]].tolist()} want {want[bad[:6]].tolist()}"
+                assert (raw(pools[l][1]) == want).all()
+
+
 # ------------------------------------------------------------------ transfer manager on real workers
 def test_transfer_manager_methods_move_the_same_bytes():
     from elasticmm_amd.kv_transfer import KVTransferManager, TransferMethod
