@@ -461,13 +461,14 @@ __device__ __forceinline__ float half_bits_to_f32(uint32_t h) {
 }
 
 // x / scale for a scale shared by a whole wave. The correctly rounded quotient is what torch's
-// cast sees, so it must be reproduced bit for bit. For 2^-30 <= |scale| <= 2^30 it is obtained
+// cast sees, so it must be reproduced bit for bit. For 2^-30 <= scale <= 2^30 it is obtained
 // without the IEEE division sequence: with y = RN(1 / scale), q = RN(x * y),
-// r = fma(-q, scale, x) (exact), the result is fma(r, y, q) — checked on the device against the
-// division for every 16-bit input and 2^20 scales. Where q is not finite (x infinite or NaN, or
-// the product overflows) the correction would produce a NaN of arbitrary sign, and where q is a
-// zero it would lose the sign of -0, so q is kept in both cases.
-// Other scales take the division.
+// r = fma(-q, scale, x) (exact), the quotient is fma(r, y, q) — checked on the device against the
+// division for every 16-bit input and 2^20 scales. The correction step turns an infinite q (x
+// infinite, or the product overflows) into a NaN and loses the sign of -0, and the conversion
+// wants NaNs replaced by infinities anyway: min(|q'|, inf) maps every NaN to +inf (the IEEE
+// minimum returns its non-NaN operand) and the sign of x is put back, which is the sign of the
+// quotient for a positive scale. Other scales (and negative ones) take the division.
 struct Divisor {
   float scale;
   float recip;
@@ -478,42 +479,45 @@ __device__ __forceinline__ Divisor make_divisor(float scale, bool allow_fast) {
   Divisor d;
   d.scale = scale;
   d.recip = 1.0f / scale;
-  const float a = __builtin_fabsf(scale);
-  d.exact_fast = allow_fast && a >= 0x1p-30f && a <= 0x1p30f;
+  d.exact_fast = allow_fast && scale >= 0x1p-30f && scale <= 0x1p30f;
   return d;
 }
 
-template <bool FAST>
-__device__ __forceinline__ float divide(float x, const Divisor &d) {
-  if constexpr (FAST) {
-    const float q = x * d.recip;
-    const float r = __builtin_fmaf(-q, d.scale, x);
-    const float q2 = __builtin_fmaf(r, d.recip, q);
-    // NaN, +-inf, +-0 (classes 0x267): keep q
-    return __builtin_amdgcn_classf(q, 0x267) ? q : q2;
-  } else {
-    return x / d.scale;
-  }
+// |x / scale| with NaN -> inf, carrying the sign of x: ready for the hardware conversion
+__device__ __forceinline__ float divide_fast_nan_free(float x, const Divisor &d) {
+  const float q = x * d.recip;
+  const float r = __builtin_fmaf(-q, d.scale, x);
+  const float q2 = __builtin_fmaf(r, d.recip, q);
+  const float a = __builtin_fminf(__builtin_fabsf(q2), __builtin_inff());
+  return __uint_as_float(__float_as_uint(a) | (__float_as_uint(x) & 0x80000000u));
 }
 
 // 8 sixteen-bit values (one u32x4) -> 8 e4m3fn bytes (one u32x2), q = rne(x / scale).
-template <int SRC_DTYPE, bool FAST>
-__device__ __forceinline__ u32x2 quant8(u32x4 in, const Divisor &d) {
-  u32x2 out;
-#pragma unroll
-  for (int w = 0; w < 2; ++w) {
-    const uint32_t w0 = in[w * 2], w1 = in[w * 2 + 1];
-    out[w] = f32x4_to_e4m3fn(divide<FAST>(half_bits_to_f32<SRC_DTYPE>(w0 & 0xffffu), d),
-                             divide<FAST>(half_bits_to_f32<SRC_DTYPE>(w0 >> 16), d),
-                             divide<FAST>(half_bits_to_f32<SRC_DTYPE>(w1 & 0xffffu), d),
-                             divide<FAST>(half_bits_to_f32<SRC_DTYPE>(w1 >> 16), d));
-  }
-  return out;
-}
-
 template <int SRC_DTYPE>
 __device__ __forceinline__ u32x2 quant8(u32x4 in, const Divisor &d) {
-  return d.exact_fast ? quant8<SRC_DTYPE, true>(in, d) : quant8<SRC_DTYPE, false>(in, d);
+  u32x2 out;
+  if (d.exact_fast) {
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+      const uint32_t w0 = in[w * 2], w1 = in[w * 2 + 1];
+      int r = 0;
+      r = __builtin_amdgcn_cvt_pk_fp8_f32(divide_fast_nan_free(half_bits_to_f32<SRC_DTYPE>(w0 & 0xffffu), d),
+                                          divide_fast_nan_free(half_bits_to_f32<SRC_DTYPE>(w0 >> 16), d), r, false);
+      r = __builtin_amdgcn_cvt_pk_fp8_f32(divide_fast_nan_free(half_bits_to_f32<SRC_DTYPE>(w1 & 0xffffu), d),
+                                          divide_fast_nan_free(half_bits_to_f32<SRC_DTYPE>(w1 >> 16), d), r, true);
+      out[w] = (uint32_t)r;
+    }
+  } else {
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+      const uint32_t w0 = in[w * 2], w1 = in[w * 2 + 1];
+      out[w] = f32x4_to_e4m3fn(half_bits_to_f32<SRC_DTYPE>(w0 & 0xffffu) / d.scale,
+                               half_bits_to_f32<SRC_DTYPE>(w0 >> 16) / d.scale,
+                               half_bits_to_f32<SRC_DTYPE>(w1 & 0xffffu) / d.scale,
+                               half_bits_to_f32<SRC_DTYPE>(w1 >> 16) / d.scale);
+    }
+  }
+  return out;
 }
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
