@@ -19,6 +19,7 @@ pytestmark = pytest.mark.gpu
 from oracle import kv_oracle as orc  # noqa: E402  (test infrastructure)
 from elasticmm_amd import _lib, cache_ops, kv_ops, pool_transfer  # noqa: E402
 from elasticmm_amd.kv_ops import PoolView  # noqa: E402
+from elasticmm_amd.block_manager import BlockLocation, BlockManager  # noqa: E402
 from elasticmm_amd.worker import KVWorker, LoopbackLink  # noqa: E402
 
 DEV = "cuda:0"
@@ -1120,6 +1121,45 @@ def test_swap_blocks_out_and_in():
     fresh = KVWorker(0, DEV, bs)
     with pytest.raises(RuntimeError, match="not initialized"):
         fresh.swap_blocks(["r"], [0], [0], True)
+
+
+def test_block_manager_drives_a_swap_cycle():
+    """Requests are swapped out by the block manager, their GPU blocks are reused and overwritten by another
+    request, and after the swap-in every request's blocks hold its own data again (block ids differ)."""
+    L, NB, NBC, bs, H, D = 2, 12, 12, 16, 2, 32
+    w = KVWorker(0, DEV, bs)
+    w.init_kvcache(NB, NBC, num_layers=L, num_kv_heads=H, head_size=D, dtype=torch.float16)
+    bm = BlockManager(NB, block_size=bs, max_num_cpu_blocks=NBC, workers=[w])
+    g = torch.Generator().manual_seed(29)
+    data = {}
+
+    def fill(rid, nblocks):
+        table = bm.allocate_blocks(rid, nblocks)
+        data[rid] = torch.randn((L, 2, nblocks, bs, H, D), generator=g).to(torch.float16)
+        w.write_kv_blocks(table, data[rid].to(DEV))
+
+    def check(rid):
+        assert bm.get_location(rid) == BlockLocation.GPU
+        assert same_bits(w.extract_kv_blocks(bm.get_block_table(rid)), data[rid]), rid
+
+    fill("a", 5)
+    fill("b", 4)
+    fill("c", 3)
+    bm.swap_out_requests(["a", "b"])
+    assert bm.get_location("a") == BlockLocation.CPU and bm.get_block_table("c") == [9, 10, 11]
+    fill("d", 8)            # needs the blocks of a and b: the manager waits for the swap-out first
+    assert set(bm.get_block_table("d")) <= set(range(9))
+    check("c")
+    check("d")
+    bm.free_blocks("d")
+    bm.swap_in_requests(["b", "a"])
+    bm.wait_for_all_swap_in()
+    for rid in ("a", "b", "c"):
+        check(rid)
+    assert sorted(bm.get_block_table("a") + bm.get_block_table("b") + bm.get_block_table("c")) == \
+        sorted(set(bm.get_block_table("a") + bm.get_block_table("b") + bm.get_block_table("c")))
+    bm.clear_request_resource_batched(["a", "b"])
+    assert not w.swap_event_table
 
 
 def test_fp8_append_scale_range_paths():

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 from elasticmm_amd import kv_ops
-from elasticmm_amd.block_manager import BlockManager
+from elasticmm_amd.block_manager import BlockLocation, BlockManager, VisionBlockManager
 from elasticmm_amd.worker import KVWorker, LoopbackLink
 
 
@@ -109,6 +109,97 @@ def test_block_manager_free_list_order():
         bm.allocate_blocks("d", 5)
     ids = bm.get_block_table("b") + bm.get_block_table("c")
     assert len(set(ids)) == len(ids)
+
+
+class _Req:
+    def __init__(self, request_id, total_len, images=None):
+        self.request_id, self.total_len, self.images = request_id, total_len, images
+
+    def get_total_len(self):
+        return self.total_len
+
+
+class _SwapRecorder:
+    def __init__(self):
+        self.calls = []
+
+    def swap_blocks(self, request_ids, src, dst, is_swap_in):
+        self.calls.append(("swap_blocks", list(request_ids), list(src), list(dst), is_swap_in))
+
+    def wait_for_all_swap_in(self):
+        self.calls.append(("wait_in",))
+
+    def wait_for_all_swap_out(self):
+        self.calls.append(("wait_out",))
+
+    def clear_request_resource(self, request_id):
+        self.calls.append(("clear", request_id))
+
+
+def test_block_manager_requests_growth_and_queries():
+    bm = BlockManager(10, block_size=16, max_num_cpu_blocks=4)
+    a, b = _Req("a", 33), _Req("b", 16)
+    assert bm.get_num_blocks_needed(a) == 3 and bm.can_allocate(a)
+    assert bm.allocate_blocks(a) == [0, 1, 2]
+    bm.allocate_blocks_batched([b])
+    assert bm.get_block_table("b") == [3] and bm.get_location("b") == BlockLocation.GPU
+    a.total_len = 49                       # one decode step past a block boundary
+    assert bm.get_num_append_blocks_needed(a) == 1 and bm.can_append(a)
+    bm.append_blocks(a)
+    assert bm.get_block_table("a") == [0, 1, 2, 4]
+    bm.append_blocks(a)                    # nothing to add
+    assert bm.get_allocated_num_blocks("a") == 4
+    assert bm.expand_blocks_for_seq_len("b", 40) == [3, 5, 6]      # vision tokens spliced in
+    assert bm.expand_blocks_for_seq_len("b", 8) == [3, 5, 6]
+    with pytest.raises(ValueError, match="not allocated"):
+        bm.expand_blocks_for_seq_len("zz", 8)
+    with pytest.raises(ValueError, match="explicit num_blocks"):
+        bm.allocate_blocks("plain-id")
+    assert bm.get_max_blocks_needed([a, b, _Req("c", 100)]) == 7
+    assert not bm.can_allocate(_Req("c", 100)) and bm.can_append(_Req("d", 48))
+    assert bm.get_block_usage() == {"gpu": "70% (7/10)", "cpu": "0% (0/4)", "swap": "0 -> 0", "#req": "2"}
+    bm.free_blocks_batched([a, "b", "unknown"])
+    assert bm.get_num_avail_gpu_blocks() == 10 and bm.free_gpu_blocks_list[-7:] == [0, 1, 2, 4, 3, 5, 6]
+    vb = VisionBlockManager(100, block_size=16)
+    assert vb.get_num_blocks_needed(_Req("v", 5, images=["i0", "i1"])) == 72 and vb.get_num_blocks_needed(_Req("t", 5)) == 0
+
+
+def test_block_manager_swap_bookkeeping_and_worker_calls():
+    rec = _SwapRecorder()
+    bm = BlockManager(6, block_size=16, max_num_cpu_blocks=5, workers=[rec])
+    bm.allocate_blocks("r1", 2)
+    bm.allocate_blocks("r2", 3)
+    src, dst = bm.swap_out_requests(["r1", "r2"])
+    assert (src, dst) == ([0, 1, 2, 3, 4], [0, 1, 2, 3, 4])
+    assert rec.calls == [("swap_blocks", ["r1", "r2"], [0, 1, 2, 3, 4], [0, 1, 2, 3, 4], False)]
+    assert bm.get_location("r1") == BlockLocation.CPU and not bm.is_all_requests_on_gpu(["r1"])
+    assert bm.get_block_table("r2") == [2, 3, 4]
+    # the GPU blocks being copied out count as available but are only handed out after the workers were waited for
+    assert bm.get_num_avail_gpu_blocks() == 6 and bm.free_gpu_blocks_list == [5]
+    assert bm.get_block_usage()["swap"] == "5 -> 0"
+    assert bm.allocate_blocks("r3", 1) == [5] and rec.calls[-1][0] == "swap_blocks"
+    assert bm.allocate_blocks("r4", 2) == [0, 1] and rec.calls[-1] == ("wait_out",)
+    with pytest.raises(AssertionError, match="is on CPU"):
+        bm.allocate_blocks("r1", 3)
+    with pytest.raises(AssertionError, match="is on BlockLocation.CPU now"):
+        bm.swap_out_requests(["r1"])
+    src, dst = bm.swap_in_requests(["r2"])
+    assert (src, dst) == ([2, 3, 4], [2, 3, 4]) and rec.calls[-1] == ("swap_blocks", ["r2"], [2, 3, 4], [2, 3, 4], True)
+    assert bm.free_cpu_blocks_list == [] and bm.swapping_cpu_blocks_list == [2, 3, 4]
+    # CPU blocks parked by the swap-in are reused only after wait_for_all_swap_in
+    bm.swap_out_requests(["r3"])
+    assert rec.calls[-2] == ("wait_in",) and bm.get_block_table("r3") == [2]
+    with pytest.raises(AssertionError, match="Not enough free blocks on CPU"):
+        bm.swap_out_requests(["r2", "r4"])
+    bm.clear_request_resource_batched(["r1", "r2"])
+    assert rec.calls[-2:] == [("clear", "r1"), ("clear", "r2")]
+    bm.free_blocks("r1")
+    assert bm.free_cpu_blocks_list[-2:] == [0, 1] and bm.swap_count == 3
+    calls = []
+    bm2 = BlockManager(2, max_num_cpu_blocks=2, engine_remote_call_all_workers_async=lambda *a: calls.append(a))
+    bm2.allocate_blocks("x", 2)
+    bm2.swap_out_requests(["x"])
+    assert calls == [("swap_blocks", ["x"], [0, 1], [0, 1], False)]
 
 
 # ------------------------------------------------------------------ transfer manager (fake workers)
