@@ -162,6 +162,49 @@ class KVTransferManager:
             print(f"[KVTransferManager] device migrate failed: {e}")
             return False
 
+    # ----- migration of whole requests (backend.py:674-737) -----------------------
+    async def migrate_requests(self, request_ids: Sequence[str], src_rank: int, src_block_manager: Any,
+                               dst_rank: int, dst_block_manager: Any) -> bool:
+        return self.migrate_requests_sync(request_ids, src_rank, src_block_manager, dst_rank, dst_block_manager)
+
+    def migrate_requests_sync(self, request_ids: Sequence[str], src_rank: int, src_block_manager: Any,
+                              dst_rank: int, dst_block_manager: Any) -> bool:
+        """The KV part of the reference's ``migrate_instance`` (elasticmm/engine/v0/backend.py:674-737):
+        for every request allocate as many destination blocks as it holds on the source, move its
+        blocks, and — only once all requests have moved — free the source blocks. A request without
+        blocks is skipped. If an allocation or a transfer fails, the destination blocks taken so far
+        are freed, the source is left untouched, and False is returned."""
+        moved: List[str] = []
+
+        def roll_back() -> None:
+            for rid in moved:
+                dst_block_manager.free_blocks(rid)
+
+        for request_id in request_ids:
+            src_blocks = src_block_manager.get_block_table(request_id)
+            if not src_blocks:
+                print(f"[KVTransferManager] No blocks found for request {request_id}, skipping")
+                continue
+            try:
+                dst_block_manager.allocate_blocks(request_id, len(src_blocks))
+            except Exception as e:
+                print(f"[KVTransferManager] Failed to allocate {len(src_blocks)} blocks for {request_id}: {e}")
+                roll_back()
+                return False
+            dst_blocks = dst_block_manager.get_block_table(request_id)
+            if not self.transfer_kv_cache_sync(request_id, src_rank, dst_rank, src_blocks, dst_blocks):
+                print(f"[KVTransferManager] KV transfer failed for {request_id}")
+                dst_block_manager.free_blocks(request_id)
+                roll_back()
+                return False
+            moved.append(request_id)
+        if self.enable_batching and not self.flush_transfer_batch(src_rank, dst_rank):
+            roll_back()
+            return False
+        for request_id in moved:
+            src_block_manager.free_blocks(request_id)
+        return True
+
     # ----- batching (kv_transfer.py:341-418, :434-462) -------------------------
     def _enqueue(self, request_id, src_rank, dst_rank, src_blocks, dst_blocks) -> bool:
         key = (src_rank, dst_rank)

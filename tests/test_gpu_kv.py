@@ -1246,3 +1246,41 @@ def test_transfer_manager_methods_move_the_same_bytes():
         torch.cuda.synchronize()
         check_moved(src, dst, si, di)
         assert m.transfer_kv_cache_sync("bad", 0, 1, [999], [0]) is (True if batching else False)
+
+
+def test_migrate_requests_between_two_workers():
+    """Elastic rescheduling of whole requests: destination tables come from the destination's block manager,
+    the blocks move through each transfer method, the source blocks are freed afterwards; a destination that is
+    too small leaves both sides as they were."""
+    from elasticmm_amd.kv_transfer import KVTransferManager, TransferMethod
+
+    for method, batching in ((TransferMethod.P2P_COPY, False), (TransferMethod.NCCL, False),
+                             (TransferMethod.CUDA_IPC, False), (TransferMethod.NCCL, True)):
+        src, dst = make_pair()
+        NB = src.pool.num_blocks
+        src_bm, dst_bm = BlockManager(NB), BlockManager(NB)
+        dst_bm.allocate_blocks("resident", 5)                 # destination tables start at block 5
+        for rid, n in (("skip-me", 2), ("a", 4), ("b", 3), ("c", 6)):
+            src_bm.allocate_blocks(rid, n)
+        src_bm.free_blocks("skip-me")
+        tables = {r: list(src_bm.get_block_table(r)) for r in ("a", "b", "c")}
+        before = [t.clone() for t in src.kv_cache]
+        m = KVTransferManager(method, enable_batching=batching, batch_size=2, batch_timeout=1e9)
+        m.register_workers("prefill", [src], [0])
+        m.register_workers("decoding", [dst], [1])
+        assert m.migrate_requests_sync(["a", "skip-me", "b", "c"], 0, src_bm, 1, dst_bm) is True
+        torch.cuda.synchronize()
+        for r, si in tables.items():
+            di = dst_bm.get_block_table(r)
+            assert len(di) == len(si) and min(di) >= 5
+            for l in range(len(before)):
+                ok = bool(torch.equal(dst.kv_cache[l][:, di], before[l][:, si]))
+                assert ok, f"{method} batching={batching}: request {r} layer {l}"
+            assert src_bm.get_block_table(r) == []
+        assert src_bm.get_num_avail_gpu_blocks() == NB
+        moved = sum(len(t) for t in tables.values())
+        assert dst_bm.get_num_avail_gpu_blocks() == NB - 5 - moved
+        # too large for what is left on the destination
+        src_bm.allocate_blocks("huge", NB - 2)
+        assert m.migrate_requests_sync(["huge"], 0, src_bm, 1, dst_bm) is False
+        assert len(src_bm.get_block_table("huge")) == NB - 2 and dst_bm.get_block_table("huge") == []

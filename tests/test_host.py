@@ -5,6 +5,7 @@ import torch
 
 from elasticmm_amd import kv_ops
 from elasticmm_amd.block_manager import BlockLocation, BlockManager, VisionBlockManager
+from elasticmm_amd.kv_transfer import KVTransferManager, TransferMethod
 from elasticmm_amd.worker import KVWorker, LoopbackLink
 
 
@@ -277,3 +278,33 @@ def test_transfer_manager_dispatch_stats_and_batching():
     assert m3.get_stats()["transfer_count"] == 3 and m3.get_stats()["total_bytes_transferred"] == 500
     assert m3.transfer_kv_cache_sync("q3", 0, 1, [6], [16]) is True and len(a.calls) == 1
     assert m3.flush_all() is True and a.calls[-1] == ("send", 1, [6])
+
+
+def test_migrate_requests_allocates_moves_frees_and_rolls_back():
+    src_bm, dst_bm = BlockManager(16), BlockManager(6)
+    src_bm.allocate_blocks("a", 3)
+    src_bm.allocate_blocks("b", 2)
+    src_bm.allocate_blocks("big", 5)
+    tm = KVTransferManager(TransferMethod.P2P_COPY)
+    w0, w1 = _FakeWorker(0), _FakeWorker(1)
+    tm.register_worker(0, w0, "prefill")
+    tm.register_worker(1, w1, "decoding")
+    assert tm.migrate_requests_sync(["a", "none", "b"], 0, src_bm, 1, dst_bm)
+    assert w0.calls == [("extract", [0, 1, 2]), ("extract", [3, 4])]
+    assert [c[:2] for c in w1.calls] == [("write", [0, 1, 2]), ("write", [3, 4])]
+    assert src_bm.get_block_table("a") == [] and dst_bm.get_block_table("b") == [3, 4]
+    assert src_bm.free_gpu_blocks_list[-5:] == [0, 1, 2, 3, 4]
+    # the destination cannot hold the request: nothing moves, nothing leaks
+    assert not tm.migrate_requests_sync(["big"], 0, src_bm, 1, dst_bm)
+    assert src_bm.get_block_table("big") == [5, 6, 7, 8, 9] and dst_bm.get_num_avail_gpu_blocks() == 1
+    # a failing transfer after a successful one: the destination is rolled back, the source keeps everything
+    dst_bm.free_blocks("a")
+    src_bm.allocate_blocks("c", 1)
+    src_bm.allocate_blocks("e", 1)
+    tm.unregister_worker(1)
+    bad = _FakeWorker(1)
+    bad.write_kv_blocks = lambda blocks, data: (_ for _ in ()).throw(RuntimeError("link down")) if len(bad.calls) else bad.calls.append("first")
+    tm.register_worker(1, bad, "decoding")
+    assert not tm.migrate_requests_sync(["c", "e"], 0, src_bm, 1, dst_bm)
+    assert dst_bm.get_block_table("c") == [] and dst_bm.get_block_table("e") == []
+    assert src_bm.get_block_table("c") != [] and src_bm.get_block_table("e") != []
