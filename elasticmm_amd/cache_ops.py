@@ -10,6 +10,7 @@ from __future__ import annotations
 
 from typing import List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from . import kv_ops
@@ -103,3 +104,36 @@ def copy_blocks(kv_caches: List[torch.Tensor], block_mapping: torch.Tensor) -> N
     if len(kv_caches) == 0 or block_mapping.numel() == 0:
         return
     kv_ops.copy_blocks(PoolView(kv_caches), block_mapping)
+
+
+def compute_slot_mapping(block_tables: Sequence[Sequence[int]], context_lens: Sequence[int],
+                         query_lens: Sequence[int], block_size: int, pad_to: Optional[int] = None,
+                         device: Optional[torch.device] = None) -> torch.Tensor:
+    """The ``slot_mapping`` of one step, as vLLM's ``prepare_model_input`` derives it from the block tables the
+    reference passes in ``SequenceGroupMetadata.block_tables`` (elasticmm/engine/v0/worker_steps.py:186-218): sequence
+    i contributes ``query_lens[i]`` tokens at positions ``context_lens[i] + k``, token at position p lives in slot
+    ``block_tables[i][p // block_size] * block_size + p % block_size``. Tokens of one sequence are consecutive, so
+    a prompt yields runs of consecutive slots. The result is int64, padded with -1 up to ``pad_to`` (the padded
+    entries are skipped by the append kernels), pinned when a GPU ``device`` is given and copied there without
+    blocking."""
+    if not (len(block_tables) == len(context_lens) == len(query_lens)):
+        raise ValueError("block_tables, context_lens and query_lens differ in length")
+    total = int(sum(query_lens))
+    size = total if pad_to is None else int(pad_to)
+    if size < total:
+        raise ValueError(f"pad_to={pad_to} is smaller than the {total} tokens of the step")
+    gpu = device is not None and torch.device(device).type == "cuda"
+    out = torch.empty(size, dtype=torch.long, pin_memory=gpu)
+    slots = out.numpy()
+    slots[total:] = -1
+    pos = 0
+    for table, ctx, q in zip(block_tables, context_lens, query_lens):
+        if q == 0:
+            continue
+        p = np.arange(ctx, ctx + q, dtype=np.int64)
+        blocks = p // block_size
+        if blocks[-1] >= len(table):
+            raise IndexError(f"a sequence of {ctx + q} tokens needs {int(blocks[-1]) + 1} blocks, its table has {len(table)}")
+        slots[pos:pos + q] = np.asarray(table, dtype=np.int64)[blocks] * block_size + p % block_size
+        pos += q
+    return out.to(device, non_blocking=True) if device is not None else out

@@ -1284,3 +1284,42 @@ def test_migrate_requests_between_two_workers():
         src_bm.allocate_blocks("huge", NB - 2)
         assert m.migrate_requests_sync(["huge"], 0, src_bm, 1, dst_bm) is False
         assert len(src_bm.get_block_table("huge")) == NB - 2 and dst_bm.get_block_table("huge") == []
+
+
+def test_step_from_block_tables_to_both_cache_layouts():
+    """Block manager -> slot mapping -> append: a step of two prompts and two decode tokens lands where the
+    tables say, in the flash layout and in the paged-attention layout."""
+    NB, bs, H, D = 40, 16, 2, 64
+    bm = BlockManager(NB, block_size=bs)
+    lens = {"p0": 70, "p1": 33, "d0": 21, "d1": 48}
+    for rid, n in lens.items():
+        bm.allocate_blocks(rid, bm.get_num_blocks_needed(n))
+    bm.free_blocks("p0")
+    bm.allocate_blocks("p0", bm.get_num_blocks_needed(70))          # tables are no longer in block order
+    order = ["p0", "d0", "p1", "d1"]
+    ctx = [0, 20, 0, 47]
+    q = [70, 1, 33, 1]
+    tables = [bm.get_block_table(r) for r in order]
+    slots = cache_ops.compute_slot_mapping(tables, ctx, q, bs, pad_to=112, device=DEV)
+    T = 112
+    g = torch.Generator().manual_seed(37)
+    key = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+    value = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+    kc = torch.zeros((NB, bs, H, D), dtype=torch.bfloat16)
+    vc = torch.zeros_like(kc)
+    kc_g, vc_g = kc.to(DEV), vc.to(DEV)
+    cache_ops.reshape_and_cache_flash(key.to(DEV), value.to(DEV), kc_g, vc_g, slots, "auto")
+    orc.c_reshape_and_cache(key, value, kc, vc, slots.cpu())
+    assert same_bits(kc_g, kc) and same_bits(vc_g, vc)
+    ok = bool(torch.equal(kc_g[tables[0][4], 5].cpu(), key[69]))     # last token of p0: position 69 = block 4, offset 5
+    assert ok
+    ok = bool(torch.equal(kc_g[tables[3][2], 15].cpu(), key[104]))   # d1's token (index 70 + 1 + 33) at position 47
+    assert ok
+    assert int((slots < 0).sum()) == 7
+    kp = torch.zeros((NB, H, D // 8, bs, 8), dtype=torch.bfloat16)
+    vp = torch.zeros((NB, H, D, bs), dtype=torch.bfloat16)
+    kp_g, vp_g = kp.to(DEV), vp.to(DEV)
+    cache_ops.reshape_and_cache(key.to(DEV), value.to(DEV), kp_g, vp_g, slots, "auto")
+    orc.c_reshape_and_cache_paged(key, value, kp, vp, slots.cpu())
+    assert same_bits(kp_g, kp) and same_bits(vp_g, vp)
+    assert same_bits(kp_g, kc_g.view(NB, bs, H, D // 8, 8).permute(0, 2, 3, 1, 4).contiguous())

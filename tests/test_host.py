@@ -308,3 +308,25 @@ def test_migrate_requests_allocates_moves_frees_and_rolls_back():
     assert not tm.migrate_requests_sync(["c", "e"], 0, src_bm, 1, dst_bm)
     assert dst_bm.get_block_table("c") == [] and dst_bm.get_block_table("e") == []
     assert src_bm.get_block_table("c") != [] and src_bm.get_block_table("e") != []
+
+
+def test_compute_slot_mapping_matches_the_definition():
+    from elasticmm_amd import cache_ops
+
+    tables = [[7, 2, 9], [4], [5, 0]]
+    ctx, q, bs = [0, 3, 17], [40, 1, 2], 16
+    got = cache_ops.compute_slot_mapping(tables, ctx, q, bs, pad_to=48)
+    want = []
+    for t, c, n in zip(tables, ctx, q):
+        for p in range(c, c + n):
+            want.append(t[p // bs] * bs + p % bs)
+    assert got.dtype == torch.long and got.tolist() == want + [-1] * 5
+    assert got[:16].tolist() == list(range(7 * 16, 8 * 16))          # a prompt fills its blocks in order
+    assert cache_ops.compute_slot_mapping([], [], [], 16).numel() == 0
+    assert cache_ops.compute_slot_mapping([[1]], [0], [0], 16, pad_to=3).tolist() == [-1, -1, -1]
+    with pytest.raises(IndexError, match="needs 3 blocks"):
+        cache_ops.compute_slot_mapping([[1, 2]], [0], [33], 16)
+    with pytest.raises(ValueError, match="pad_to"):
+        cache_ops.compute_slot_mapping([[1, 2]], [0], [20], 16, pad_to=8)
+    with pytest.raises(ValueError, match="differ in length"):
+        cache_ops.compute_slot_mapping([[1]], [0, 1], [1], 16)
