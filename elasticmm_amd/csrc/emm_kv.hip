@@ -1182,21 +1182,30 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(const PagedP
     const int64_t blk = s_blk[whole];
     const int off0 = s_off[whole];
     const char *rows = tile + whole * ROW;
-    for (int q = tid; q < seg_elems * CE; q += kThreads) {
-      uint32_t w[4];
-      int e;
-      if constexpr (CE == 2) {
-        e = q >> 1;
-        const char *col = rows + (q & 1) * 8 * ROW + e * 2;
+    if constexpr (CE == 2) {
+      // Lanes 0-31 of a wave gather tokens 0-7 of 32 consecutive elements, lanes 32-63 tokens 8-15 of
+      // the same elements: the two half-waves read different tile rows at the same column (the same
+      // LDS banks) in different passes, and one store instruction still covers the 32 elements'
+      // 1 KiB of output completely.
+      const int lane = tid & 63, half = lane >> 5;
+      for (int q0 = (tid >> 6) * 32; q0 < seg_elems; q0 += (kThreads >> 6) * 32) {
+        const int e = q0 + (lane & 31);
+        if (e >= seg_elems) continue;
+        const char *col = rows + half * 8 * ROW + e * 2;
+        uint32_t w[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const uint32_t lo = *reinterpret_cast<const uint16_t *>(col + (2 * i) * ROW);
           const uint32_t hi = *reinterpret_cast<const uint16_t *>(col + (2 * i + 1) * ROW);
           w[i] = lo | (hi << 16);
         }
-      } else {
-        e = q;
+        char *dst = cache + ((blk * p.row_elems + e0 + e) * bs + off0) * 2 + half * 16;
+        st_stream<u32x4, 1>(dst, u32x4{w[0], w[1], w[2], w[3]});
+      }
+    } else {
+      for (int e = tid; e < seg_elems; e += kThreads) {
         const char *col = rows + e;
+        uint32_t w[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           uint32_t x = 0;
@@ -1205,9 +1214,9 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(const PagedP
             x |= (uint32_t) * reinterpret_cast<const uint8_t *>(col + (4 * i + k) * ROW) << (8 * k);
           w[i] = x;
         }
+        char *dst = cache + ((blk * p.row_elems + e0 + e) * bs + off0);
+        st_stream<u32x4, 1>(dst, u32x4{w[0], w[1], w[2], w[3]});
       }
-      char *dst = cache + ((blk * p.row_elems + e0 + e) * bs + off0) * CE + (CE == 2 ? (q & 1) * 16 : 0);
-      st_stream<u32x4, 1>(dst, u32x4{w[0], w[1], w[2], w[3]});
     }
   }
   // ---- V, the other owned tokens: one element per lane, element fastest ----
