@@ -42,6 +42,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements (append, batched, copy)")
     ap.add_argument("--variant", type=int, default=0, help="block-move launch variant (tuning)")
+    ap.add_argument("--spread", type=int, default=4,
+                    help="stripes per pool: each pool's layers are allocated in this many pieces spread over the "
+                         "free device memory (0 or 1: one allocation per pool)")
     ap.add_argument("--extended", action="store_true",
                     help="after the headline, free its pools and measure the fp8 70B-class shape and the ~200 GB "
                          "rebalancing shape at full size (adds about a minute)")
@@ -135,8 +138,10 @@ def main():
     tables, total_blocks = make_requests(args.requests, NB, seed=2)
 
     src_w, dst_w = KVWorker(0, "cuda:0", bs), KVWorker(1, "cuda:0", bs)
-    src_w.init_kvcache(NB, num_layers=L, num_kv_heads=H, head_size=D, dtype=dtype, monolithic=True)
-    dst_w.init_kvcache(NB, num_layers=L, num_kv_heads=H, head_size=D, dtype=dtype, monolithic=True)
+    src_w.init_kvcache(NB, num_layers=L, num_kv_heads=H, head_size=D, dtype=dtype, monolithic=True,
+                       spread_stripes=args.spread)
+    dst_w.init_kvcache(NB, num_layers=L, num_kv_heads=H, head_size=D, dtype=dtype, monolithic=True,
+                       spread_stripes=args.spread)
     g = torch.Generator(device=dev).manual_seed(2)
     for t in src_w.kv_cache:
         t.normal_(0.0, 0.5, generator=g)
@@ -247,6 +252,8 @@ def main():
                         % (NB, len(tables), total_blocks, payload / 1e9),
             "num_layers": L, "num_blocks": NB, "block_size": bs, "kv_heads": H, "head_dim": D,
             "requests": len(tables), "blocks_moved": total_blocks, "algorithmic_bytes_per_step": bytes_per_step,
+            "pool_allocation": ("each pool allocated on its own, layers in %d stripes spread over the free device "
+                                "memory" % args.spread) if args.spread > 1 else "each pool one allocation",
         },
         "roofline": roofline,
         "extra": extra,

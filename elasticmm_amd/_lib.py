@@ -65,6 +65,12 @@ def load() -> ctypes.CDLL:
         raise RuntimeError(
             f"{path} is missing: the HIP library has not been built "
             "(run `python -m elasticmm_amd.build`). There is no CPU fallback.")
+    # torch carries its own copy of the HIP runtime and exports its symbols globally. Streams and device pointers
+    # come from torch, so the library has to bind to that copy: torch is loaded before the library is.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = ctypes.CDLL(path)
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError if the symbol is not exported

@@ -63,6 +63,65 @@ class LoopbackLink:
         return len(self._queues[(src, dst, tag)])
 
 
+def _hip_runtime():
+    """The HIP runtime torch itself uses (torch ships its own copy next to its libraries)."""
+    import ctypes
+    import os
+
+    bundled = os.path.join(os.path.dirname(torch.__file__), "lib", "libamdhip64.so")
+    rt = ctypes.CDLL(bundled if os.path.exists(bundled) else "libamdhip64.so")
+    rt.hipMalloc.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t]
+    rt.hipMalloc.restype = ctypes.c_int
+    rt.hipFree.argtypes = [ctypes.c_void_p]
+    rt.hipFree.restype = ctypes.c_int
+    rt.hipGetLastError.restype = ctypes.c_int
+    return rt, ctypes
+
+
+def allocate_layers_spread(num_layers: int, layer_shape: Sequence[int], dtype: torch.dtype, device: torch.device,
+                           stripes: int = 4, reserve_bytes: int = 8 << 30) -> List[torch.Tensor]:
+    """Allocate the L layer tensors of a pool in ``stripes`` allocations that lie far apart in device memory;
+    layer l goes to stripe ``l % stripes``, so consecutive layers are far apart as well.
+
+    Why: on MI355X the scattered 16 KiB writes of unpack / copy_blocks run at 5.4 TB/s when a launch's
+    destinations all lie in one large region of device memory and at 6.3 TB/s when they reach more than one
+    (the regions are tens of GiB long; a pool of about 50 GiB allocated in one piece often lies inside a single
+    one). A pool that fills most of the device spans them anyway; for a smaller pool the stripes are pushed
+    apart by allocating a temporary spacer after each stripe (the free memory divided by the number of stripes)
+    and releasing the spacers at the end. Nothing is shared with other pools: every pool is allocated by its
+    own call. With too little free memory for spacers the stripes are simply allocated one after the other."""
+    device = torch.device(device)
+    stripes = max(1, min(int(stripes), num_layers))
+    layer_elems = 1
+    for d in layer_shape:
+        layer_elems *= int(d)
+    elem = torch.empty((), dtype=dtype).element_size()
+    need = num_layers * layer_elems * elem
+    counts = [len(range(s, num_layers, stripes)) for s in range(stripes)]
+    with torch.cuda.device(device):
+        free, _ = torch.cuda.mem_get_info()
+        gap = max(0, (free - need - reserve_bytes) // stripes)
+        gap -= gap % (2 << 20)
+        rt, ctypes = _hip_runtime()
+        spacers, parts = [], []
+        try:
+            for s in range(stripes):
+                parts.append(torch.empty(counts[s] * layer_elems, dtype=dtype, device=device))
+                if gap > 0 and s + 1 < stripes:
+                    ptr = ctypes.c_void_p()
+                    if rt.hipMalloc(ctypes.byref(ptr), gap) != 0:
+                        rt.hipGetLastError()  # clear it: the next launch check must not see this failure
+                        break  # no room for this spacer: the remaining stripes follow directly
+                    spacers.append(ptr)
+        finally:
+            for ptr in spacers:
+                rt.hipFree(ptr)
+    while len(parts) < stripes:
+        parts.append(torch.empty(counts[len(parts)] * layer_elems, dtype=dtype, device=device))
+    return [parts[l % stripes][(l // stripes) * layer_elems:(l // stripes + 1) * layer_elems].view(tuple(layer_shape))
+            for l in range(num_layers)]
+
+
 class KVWorker:
     """Owns one block pool on one GPU and moves blocks in and out of it."""
 
@@ -90,13 +149,18 @@ class KVWorker:
 
     # ----- pool -----------------------------------------------------------
     def init_kvcache(self, num_gpu_blocks: int, num_cpu_blocks: int = 0, *, num_layers: int, num_kv_heads: int,
-                     head_size: int, dtype: torch.dtype = torch.bfloat16, monolithic: bool = True) -> List[int]:
+                     head_size: int, dtype: torch.dtype = torch.bfloat16, monolithic: bool = True,
+                     spread_stripes: int = 0) -> List[int]:
         """Allocate the pool: L tensors ``[2, num_gpu_blocks, block_size, num_kv_heads, head_size]``
         (worker.py:388-394). With ``monolithic`` the L tensors are views of one
         allocation, which keeps the list API and lets the whole pool be one HBM
-        region; otherwise each layer is its own allocation as vLLM's CacheEngine does."""
+        region; otherwise each layer is its own allocation as vLLM's CacheEngine does.
+        ``spread_stripes = k > 1`` places the layers in k allocations spread over the device's
+        free memory (see ``allocate_layers_spread``)."""
         shape = (2, num_gpu_blocks, self.block_size, num_kv_heads, head_size)
-        if monolithic:
+        if spread_stripes > 1:
+            layers = allocate_layers_spread(num_layers, shape, dtype, self.device, spread_stripes)
+        elif monolithic:
             whole = torch.empty((num_layers,) + shape, dtype=dtype, device=self.device)
             layers = list(whole.unbind(0))
         else:

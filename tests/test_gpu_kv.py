@@ -1323,3 +1323,36 @@ def test_step_from_block_tables_to_both_cache_layouts():
     orc.c_reshape_and_cache_paged(key, value, kp, vp, slots.cpu())
     assert same_bits(kp_g, kp) and same_bits(vp_g, vp)
     assert same_bits(kp_g, kc_g.view(NB, bs, H, D // 8, 8).permute(0, 2, 3, 1, 4).contiguous())
+
+
+def test_spread_allocation_of_a_pool():
+    """A pool whose layers are allocated in stripes spread over the device memory: same list API, layers
+    disjoint, consecutive layers in different stripes (where the stripes land physically cannot be seen from here), and the kernels give the oracle's bytes on it."""
+    from elasticmm_amd.worker import allocate_layers_spread
+
+    L, NB, bs, H, D = 7, 4096, 16, 2, 64       # 32 MiB per layer: large enough to be allocations of their own
+    torch.cuda.empty_cache()
+    w = KVWorker(0, DEV, bs)
+    w.init_kvcache(NB, num_layers=L, num_kv_heads=H, head_size=D, dtype=torch.bfloat16, spread_stripes=3)
+    assert len(w.kv_cache) == L and all(tuple(t.shape) == (2, NB, bs, H, D) and t.is_contiguous() for t in w.kv_cache)
+    nbytes = w.kv_cache[0].numel() * 2
+    spans = sorted((t.data_ptr(), t.data_ptr() + nbytes) for t in w.kv_cache)
+    assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:])), "layers overlap"
+    p = [t.data_ptr() for t in w.kv_cache]
+    assert p[3] - p[0] == nbytes and p[6] - p[3] == nbytes and p[4] - p[1] == nbytes     # stripe = layers l, l+3, l+6
+    src_c = cpu_pool(L, NB, bs, H, D, torch.bfloat16, 51)
+    for t, c in zip(w.kv_cache, src_c):
+        t.copy_(c)
+    si, di = [3, 4095, 0, 1717, 8], [1, 2, 3000, 31, 5]
+    buf = w.extract_kv_blocks(si)
+    assert same_bits(buf, orc.ref_extract_kv_blocks(src_c, si))
+    w.write_kv_blocks(di, buf)
+    orc.ref_write_kv_blocks(src_c, di, orc.ref_extract_kv_blocks(src_c, si))
+    for l in range(L):
+        assert same_bits(w.kv_cache[l], src_c[l]), f"layer {l}"
+    # more stripes than layers, and no room for spacers
+    layers = allocate_layers_spread(2, (2, 4, 16, 1, 8), torch.float16, torch.device(DEV), stripes=5,
+                                    reserve_bytes=1 << 50)
+    assert len(layers) == 2 and layers[0].data_ptr() != layers[1].data_ptr()
+    kv_ops.kv_pack(PoolView(layers), [0, 3])
+    torch.cuda.synchronize()
