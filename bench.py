@@ -200,9 +200,9 @@ def main():
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4),
         # HBM bytes per launch: rocprofv3 FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 (factors from a plain
-        # 1 GiB copy in the same profile run) came to 1.0006 x the algorithmic bytes for this kernel on this
+        # 1 GiB copy in the same profile run) came to 1.0004 x the algorithmic bytes for this kernel on this
         # workload (profiles/block_move_qwen2_7b_migrate_pmc.txt); the figure is that ratio, not a live counter
-        "traffic": int(kern_bytes / launches * 1.0006),
+        "traffic": int(kern_bytes / launches * 1.0004),
         "launches": launches,
         "avg_launch_us": round((pack_ms + unpack_ms) * 1e3 / launches, 2),
         "avg_bytes_per_launch": int(kern_bytes / launches),
