@@ -230,7 +230,7 @@ def main():
         src_w._pool = dst_w._pool = None
         dev_tables = None
         torch.cuda.empty_cache()
-        extra["extended"] = extended(dev)
+        extra["extended"] = extended(dev, args.spread)
 
     result = {
         "metric": "KV pack+unpack GB/s",
@@ -437,7 +437,7 @@ def append_bench(kv, NB, bs, H, D, cache_dtype_name, k_scales, v_scales, dev, T=
     return res
 
 
-def extended(dev):
+def extended(dev, spread=4):
     """The two other target shapes at full size (run with --extended; needs the whole GPU):
     the fp8-e4m3 70B-class per-GPU shape and the elastic rebalancing of a ~200 GB pool."""
     from elasticmm_amd import kv_ops
@@ -455,9 +455,20 @@ def extended(dev):
     perm_d = torch.randperm(NB, generator=g)[:total].to(dev)
     k_scales = (torch.rand(L, generator=g) * 0.09 + 0.01).to(dev)
     v_scales = (torch.rand(L, generator=g) * 0.09 + 0.01).to(dev)
-    src = torch.empty((L, 2, NB, bs, H, D), dtype=torch.uint8, device=dev)
-    src.random_(0, 0x78)  # finite positive e4m3 bytes
-    dst = torch.zeros_like(src)
+    from elasticmm_amd.worker import allocate_layers_spread
+
+    def make_pool(dtype):
+        shape = (2, NB, bs, H, D)
+        if spread > 1:
+            return allocate_layers_spread(L, shape, dtype, dev, spread)
+        return list(torch.empty((L,) + shape, dtype=dtype, device=dev).unbind(0))
+
+    src = make_pool(torch.uint8)
+    dst = make_pool(torch.uint8)
+    for t in src:
+        t.random_(0, 0x78)  # finite positive e4m3 bytes
+    for t in dst:
+        t.zero_()
     sp, dp = PoolView(src), PoolView(dst)
     off, ts_pack, ts_unpack, payload = 0, 0.0, 0.0, 0
     for n in nblk:  # per-request staging buffers (the whole batch would be 45 GiB)
@@ -474,11 +485,13 @@ def extended(dev):
                             "payload_GB": round(payload / 1e9, 2),
                             "pack_GBps": round(2 * payload / (ts_pack * 1e-3) / 1e9, 1),
                             "unpack_GBps": round(2 * payload / (ts_unpack * 1e-3) / 1e9, 1)}
-    out["fp8_70b_shape"]["append"] = append_bench(list(src.unbind(0)), NB, bs, H, D, "fp8", k_scales, v_scales, dev)
+    out["fp8_70b_shape"]["append"] = append_bench(src, NB, bs, H, D, "fp8", k_scales, v_scales, dev)
     del dst, dp
     torch.cuda.empty_cache()
     # dequantising unpack into a bf16 pool (first 16 requests)
-    dq = torch.zeros((L, 2, NB, bs, H, D), dtype=torch.bfloat16, device=dev)
+    dq = make_pool(torch.bfloat16)
+    for t in dq:
+        t.zero_()
     dqp = PoolView(dq)
     off, t_dq, pay = 0, 0.0, 0
     for n in nblk[:16]:
