@@ -127,9 +127,10 @@ def main():
     from elasticmm_amd.kv_ops import PoolView
     from elasticmm_amd.worker import KVWorker
 
-    lib = _lib.load()
     if args.variant:
-        lib.emm_set_move_variant(args.variant)
+        # launch variants exist only in the hooks build of the library: route this process through it
+        _lib.use_hooks_build().emm_hook_set_move_variant(args.variant)
+    lib = _lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     L, bs, H, D, dtype = 28, 16, 4, 128, torch.bfloat16

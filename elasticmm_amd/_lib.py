@@ -9,13 +9,14 @@ import ctypes
 import os
 from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p, POINTER
 
-from .build import library_path
+from .build import hooks_library_path, library_path
 
-EMM_KV_ABI_VERSION = 1
+EMM_KV_ABI_VERSION = 2
 EMM_MAX_LAYERS = 96
 EMM_MAX_SEGMENTS = 128
 EMM_DTYPE_BF16 = 0
 EMM_DTYPE_F16 = 1
+EMM_FP8_SATURATE = 0x100
 
 _P = c_void_p
 _PP = POINTER(c_void_p)
@@ -25,7 +26,6 @@ _I64P = POINTER(c_int64)
 SIGNATURES = {
     "emm_last_error": (c_char_p, []),
     "emm_abi_version": (c_int, []),
-    "emm_set_move_variant": (c_int, [c_int]),
     "emm_kv_pack": (c_int, [_PP, c_int, c_int, c_int64, c_int64, _P, c_int64, _P, _P]),
     "emm_kv_unpack": (c_int, [_PP, c_int, c_int, c_int64, c_int64, _P, c_int64, _P, _P]),
     "emm_copy_blocks": (c_int, [_PP, c_int, c_int, c_int64, c_int64, _P, c_int64, _P]),
@@ -48,7 +48,16 @@ SIGNATURES = {
     "emm_stream_copy": (c_int, [_P, _P, c_int64, _P]),
 }
 
+# libemm_kv_hooks.so only (csrc/emm_kv_hooks.h): benchmark / test hooks, absent from the product library
+HOOK_SIGNATURES = {
+    "emm_hook_set_move_variant": (c_int, [c_int]),
+    "emm_hook_probe": (c_int, [_PP, c_int, c_int, c_int64, c_int64, _P, c_int64, _P, _P, _P]),
+    "emm_hook_fp8_quotient_sweep": (c_int, [c_int, c_int, ctypes.c_uint32, ctypes.c_uint32, _P, _P]),
+}
+EMM_PROBE_SEQ_READ, EMM_PROBE_SEQ_WRITE, EMM_PROBE_GATHER_READ, EMM_PROBE_SCATTER_WRITE = 0, 1, 2, 3
+
 _lib = None
+_hooks = None
 
 
 class EmmError(RuntimeError):
@@ -81,6 +90,35 @@ def load() -> ctypes.CDLL:
         raise RuntimeError(f"libemm_kv.so ABI version {ver}, expected {EMM_KV_ABI_VERSION}")
     _lib = lib
     return lib
+
+
+def load_hooks() -> ctypes.CDLL:
+    """Load libemm_kv_hooks.so (bench.py and tests only): the product ABI plus the hooks."""
+    global _hooks
+    if _hooks is not None:
+        return _hooks
+    path = hooks_library_path()
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing (run `python -m elasticmm_amd.build`)")
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
+    lib = ctypes.CDLL(path)
+    for name, (res, args) in {**SIGNATURES, **HOOK_SIGNATURES}.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _hooks = lib
+    return lib
+
+
+def use_hooks_build() -> ctypes.CDLL:
+    """Route every later call of this process through libemm_kv_hooks.so, so that a benchmark can switch
+    launch variants (``emm_hook_set_move_variant``). Never called by the package itself."""
+    global _lib
+    _lib = load_hooks()
+    return _lib
 
 
 def check(rc: int, what: str) -> None:

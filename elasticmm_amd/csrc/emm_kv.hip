@@ -21,6 +21,7 @@
 #include <stdio.h>
 #include <stdarg.h>
 #include <string.h>
+#include <type_traits>
 
 #include "emm_kv.h"
 
@@ -162,177 +163,163 @@ __device__ __forceinline__ void copy_tile(const char *__restrict__ src, char *__
 }
 
 // ----------------------------------------------------------------------------
-// block move: pack / unpack / copy_blocks / migrate / plain copy
+// block move: pack / unpack / copy_blocks / migrate
 // ----------------------------------------------------------------------------
 // One side of a move is either a block pool (one base pointer per (layer, K|V)
 // plane, block chosen through an int64 index array) or a linear transfer
 // buffer [planes, n, chunk].
+//
+// What bounds these kernels is not instruction issue but the length of the chain of
+// dependent memory round trips a wave goes through before its data load is in flight
+// (measured: with the pool side read at random the memory system is not saturated — its
+// queues report 15x fewer stalls for lack of DRAM credits than for a sequential copy —
+// so every round trip a wave waits for shows up as lost throughput). The chain is kept
+// at its minimum of two:
+//   1. block id (scalar load through the index pointer) and plane base (scalar load from
+//      the table in the argument block), issued together and waited for once;
+//   2. the data.
+// To that end the scalar arguments are explicit kernel parameters in the order in which
+// they are needed, so that the hardware preloads them into scalar registers before the
+// wave starts (kernarg preload, -mllvm -amdgpu-kernarg-preload-count): no round trip is
+// spent on fetching them. Loads from a linear source depend on no id and are issued
+// before that single wait. Launch-order variants and tail handling are template
+// parameters, so the common path carries no branch and no extra argument.
 constexpr int kMaxPlanes = 2 * EMM_MAX_LAYERS;
 constexpr int kMaxGridY = 65535;
 constexpr int kRun = 16; // blocks per plane visit in the pool-to-pool order
 
-struct MoveParams {
-  const char *src_planes[kMaxPlanes]; // pool source: base of each (layer, kv) plane
-  char *dst_planes[kMaxPlanes];       // pool destination
-  const char *src_linear;             // linear source base
-  char *dst_linear;                   // linear destination base
-  const int64_t *src_idx;             // block ids on the source side
-  const int64_t *dst_idx;             // block ids on the destination side
-  int64_t idx_stride;                 // elements between consecutive ids
-  int64_t src_num_blocks;
-  int64_t dst_num_blocks;
-  int64_t chunk_bytes;
-  int64_t n;      // blocks per plane of the linear buffer
-  int64_t j0;     // first block of this launch
-  int64_t j_end;  // one past the last block of this launch
-  int32_t group_log2; // grouped order for moves with a linear side (0 = off)
-  int64_t plane0; // first plane of this launch (linear side)
+struct PlaneTable {
+  char *base[kMaxPlanes]; // base of each (layer, kv) plane
+};
+template <int N>
+struct PlaneTables {
+  PlaneTable t[N]; // pack: source; unpack: destination; pool-to-pool: source, destination
 };
 
-// grid: x = tiles of one chunk, y = blocks (at most kMaxGridY per launch),
-// z = planes. Dispatch order (x fastest, then y, then z) walks the transfer
-// buffer linearly; no integer division is needed to find a workgroup's tile.
-//
-// When both sides are pools (copy_blocks, migrate) the order is different: runs
-// of kRun consecutive blocks per plane, planes next, runs last (y = plane * kRun
-// + position in the run, z = run), so that the workgroups in flight at any moment
-// touch every plane of the pool instead of one plane's window, while a table of
-// consecutive block ids still gives sequential runs. Measured on MI355X this is
-// about 12 % faster for scattered pool-to-pool moves; with a linear side it is
-// slower (the linear buffer would be read as one stream per plane).
-template <typename V, int T, int U, bool SRC_POOL, bool DST_POOL, int POLICY>
-__global__ __launch_bounds__(T) void emm_block_move_kernel(const MoveParams p) {
-  constexpr int64_t TILE = (int64_t)U * T * sizeof(V);
-  constexpr bool PLANE_FASTEST = SRC_POOL && DST_POOL;
-  uint32_t pl;
-  int64_t j;
-  if constexpr (PLANE_FASTEST) {
-    // y = plane * kRun + position in a run of kRun consecutive blocks, z = run
+constexpr int kPack = 0, kUnpack = 1, kPoolToPool = 2;
+// Launch orders (grid x is always the tile inside a chunk):
+//  plain    y = block, z = plane: walks the transfer buffer linearly.
+//  grouped  y = plane * 2^g + position, z = group: groups of 2^g blocks per plane visit. Used for
+//           long scatters: visiting a plane for thousands of blocks in a row keeps all writes inside
+//           that plane's address window, which this memory system serves about 12 % slower than
+//           writes spread over the whole pool.
+//  runs     y = plane * kRun + position in a run of kRun consecutive blocks, z = run, every plane
+//           starting at its own run: the workgroups in flight at any moment touch every plane of
+//           the pool, while a table of consecutive ids still gives sequential runs. Used when both
+//           sides are pools (about 12 % faster there; slower with a linear side, which would be
+//           read as one stream per plane).
+constexpr int kOrderPlain = 0, kOrderGrouped = 1, kOrderRuns = 2;
+
+// idx_a / idx_b: source / destination ids (PAIRS: idx_a holds (src, dst) pairs, idx_b unused).
+// `n` = blocks of this launch (ids and linear buffer already offset to its first block),
+// `order_arg` = log2 of the group size (grouped) or the per-plane rotation of the runs (runs).
+template <typename V, int U, int KIND, int ORDER, bool FULL, bool PAIRS, int POLICY>
+__global__ __launch_bounds__(kThreads) void emm_block_move_kernel(
+    const int64_t *__restrict__ idx_a, const int64_t *__restrict__ idx_b, char *lin,
+    int64_t lin_plane_stride, int64_t chunk, uint32_t src_nb, uint32_t dst_nb, uint32_t n,
+    uint32_t order_arg, const PlaneTables<KIND == kPoolToPool ? 2 : 1> tables) {
+  constexpr int64_t TILE = (int64_t)U * kThreads * sizeof(V);
+  constexpr bool SRC_POOL = KIND != kUnpack, DST_POOL = KIND != kPack;
+  uint32_t pl, j;
+  if constexpr (ORDER == kOrderRuns) {
     pl = blockIdx.y / kRun;
-    // every plane starts at its own run: planes whose bases differ by a highly
-    // aligned stride then do not hit the same memory channels at the same time
-    uint32_t run = blockIdx.z + pl * (gridDim.z / (gridDim.y / kRun));
-    if (run >= gridDim.z) run -= gridDim.z;
-    j = p.j0 + (int64_t)run * kRun + (blockIdx.y % kRun);
-    if (j >= p.j_end) return;
-  } else if (p.group_log2 > 0) {
-    // groups of 2^group_log2 blocks per plane visit (y = plane * G + position, z = group)
-    const uint32_t G = 1u << p.group_log2;
-    pl = blockIdx.y >> p.group_log2;
-    j = p.j0 + ((int64_t)blockIdx.z << p.group_log2) + (blockIdx.y & (G - 1));
-    if (j >= p.j_end) return;
+    const uint32_t runs = (n + kRun - 1) / kRun;
+    uint32_t run = blockIdx.z + pl * order_arg; // order_arg = runs / planes
+    if (run >= runs) run -= runs;
+    j = run * kRun + (blockIdx.y % kRun);
+    if (j >= n) return;
+  } else if constexpr (ORDER == kOrderGrouped) {
+    pl = blockIdx.y >> order_arg;
+    j = (blockIdx.z << order_arg) + (blockIdx.y & ((1u << order_arg) - 1u));
+    if (j >= n) return;
   } else {
     pl = blockIdx.z;
-    j = p.j0 + blockIdx.y;
+    j = blockIdx.y;
   }
-  const int64_t chunk = p.chunk_bytes;
-  const int64_t tile_off = (int64_t)blockIdx.x * TILE;
-  const int64_t linear_off = ((p.plane0 + pl) * p.n + j) * chunk + tile_off;
-
-  const int64_t limit = chunk - tile_off;
-  // The scalar work of a workgroup is a chain of dependent fetches (arguments ->
-  // block ids -> data). The empty asm statements below pin values in scalar
-  // registers at the point where they stand, which keeps the chain at its
-  // minimum: (1) plane bases arrive with the first batch of argument loads,
-  // (2) both block ids are fetched together and waited for once, and (3) loads
-  // from a linear source, which depend on no id, are issued before that wait.
+  // round trip 1: ids and plane bases, all issued before the one wait below
+  int64_t sb = 0, db = 0;
+  if constexpr (PAIRS) {
+    sb = idx_a[2 * (uint64_t)j];
+    db = idx_a[2 * (uint64_t)j + 1];
+  } else {
+    if constexpr (SRC_POOL) sb = idx_a[j];
+    if constexpr (DST_POOL) db = idx_b[j];
+  }
   const char *src_plane = nullptr;
   char *dst_plane = nullptr;
-  if constexpr (SRC_POOL) {
-    src_plane = p.src_planes[pl];
-    asm volatile("" : "+s"(src_plane));
-  }
-  if constexpr (DST_POOL) {
-    dst_plane = p.dst_planes[pl];
-    asm volatile("" : "+s"(dst_plane));
-  }
-  int64_t sb = 0, db = 0;
-  if constexpr (SRC_POOL) sb = p.src_idx[j * p.idx_stride];
-  if constexpr (DST_POOL) db = p.dst_idx[j * p.idx_stride];
+  if constexpr (SRC_POOL) src_plane = tables.t[0].base[pl];
+  if constexpr (DST_POOL) dst_plane = tables.t[KIND == kPoolToPool ? 1 : 0].base[pl];
+
+  const int64_t tile_off = (int64_t)blockIdx.x * TILE;
+  const int64_t limit = FULL ? TILE : chunk - tile_off;
+  char *linp = nullptr;
+  if constexpr (KIND != kPoolToPool) linp = lin + (int64_t)pl * lin_plane_stride + (int64_t)j * chunk + tile_off;
   V v[U];
-  if constexpr (!SRC_POOL) load_tile<V, T, U, POLICY>(v, p.src_linear + linear_off, limit);
-  sb = uniform64(sb);
-  db = uniform64(db);
-  asm volatile("" : "+s"(sb), "+s"(db) : : "memory");
+  if constexpr (!SRC_POOL) load_tile<V, kThreads, U, POLICY>(v, linp, limit); // needs no id
+  asm volatile("" : "+s"(sb), "+s"(db), "+s"(src_plane), "+s"(dst_plane) : : "memory");
   if constexpr (SRC_POOL) {
-    if ((uint64_t)sb >= (uint64_t)p.src_num_blocks) return; // padding / invalid
-    load_tile<V, T, U, POLICY>(v, src_plane + sb * chunk + tile_off, limit);
+    if ((uint64_t)sb >= (uint64_t)src_nb) return; // padding (negative) / out of range: skipped
+    load_tile<V, kThreads, U, POLICY>(v, src_plane + sb * chunk + tile_off, limit); // round trip 2
   }
   char *dst;
   if constexpr (DST_POOL) {
-    if ((uint64_t)db >= (uint64_t)p.dst_num_blocks) return;
+    if ((uint64_t)db >= (uint64_t)dst_nb) return;
     dst = dst_plane + db * chunk + tile_off;
   } else {
-    dst = p.dst_linear + linear_off;
+    dst = linp;
   }
-  store_tile<V, T, U, POLICY>(v, dst, limit);
+  store_tile<V, kThreads, U, POLICY>(v, dst, limit);
 }
 
-// Launch variant of the 16-byte path (benchmarks only): bits 0-3 vectors per lane
-// (1 or 4), bits 8-11 cache policy + 1 (policy 0: nt stores, 1: sc0 sc1 stores).
-// 0 selects the default: one vector per lane, sc0 sc1 stores. The sweep that chose
-// it also covered 64-thread workgroups, two vectors per lane and the sc0 sc1 nt /
-// plain policies; none was faster and they are no longer instantiated.
+// Plain device-to-device copy with the same tile shape (the yardstick of the block moves).
+template <typename V, int U, int POLICY>
+__global__ __launch_bounds__(kThreads) void emm_stream_copy_kernel(const char *__restrict__ src,
+                                                                   char *__restrict__ dst, int64_t nbytes) {
+  constexpr int64_t TILE = (int64_t)U * kThreads * sizeof(V);
+  const int64_t off = (int64_t)blockIdx.x * TILE;
+  copy_tile<V, kThreads, U, POLICY>(src + off, dst + off, nbytes - off);
+}
+
+#ifdef EMM_BENCH_HOOKS
+// Benchmark builds only (libemm_kv_hooks.so): launch variants selectable at run time.
 int g_move_variant = 0;
+inline int move_variant() { return g_move_variant; }
+#else
+constexpr int move_variant() { return 0; }
+#endif
 
 bool aligned(const void *p, int a) { return ((uintptr_t)p & (uintptr_t)(a - 1)) == 0; }
 
-template <typename V, int U, bool SP, bool DP>
-void launch_move_policy(const MoveParams &p, dim3 grid, int policy, hipStream_t s) {
-  if (policy == 1 && sizeof(V) == 16)
-    emm_block_move_kernel<V, kThreads, U, SP, DP, 1><<<grid, kThreads, 0, s>>>(p);
+struct MoveArgs {
+  const int64_t *idx_a;
+  const int64_t *idx_b;
+  char *lin;
+  int64_t lin_plane_stride;
+  int64_t chunk;
+  uint32_t src_nb, dst_nb;
+};
+
+template <typename V, int U, int KIND, int ORDER, bool PAIRS, int POLICY>
+void launch_move_full(const MoveArgs &a, uint32_t n, uint32_t order_arg, dim3 grid, bool full,
+                      const PlaneTables<KIND == kPoolToPool ? 2 : 1> &t, hipStream_t s) {
+  if (full)
+    emm_block_move_kernel<V, U, KIND, ORDER, true, PAIRS, POLICY><<<grid, kThreads, 0, s>>>(
+        a.idx_a, a.idx_b, a.lin, a.lin_plane_stride, a.chunk, a.src_nb, a.dst_nb, n, order_arg, t);
   else
-    emm_block_move_kernel<V, kThreads, U, SP, DP, 0><<<grid, kThreads, 0, s>>>(p);
+    emm_block_move_kernel<V, U, KIND, ORDER, false, PAIRS, POLICY><<<grid, kThreads, 0, s>>>(
+        a.idx_a, a.idx_b, a.lin, a.lin_plane_stride, a.chunk, a.src_nb, a.dst_nb, n, order_arg, t);
 }
 
-template <bool SP, bool DP>
-int launch_move(MoveParams &p, int planes, int min_align, hipStream_t s, const char *what) {
-  if (p.n == 0 || planes == 0 || p.chunk_bytes == 0) return EMM_OK;
-  // widest lane access that divides the chunk and every base address
-  int vec = 16;
-  while (vec > 1 && (p.chunk_bytes % vec != 0 || min_align % vec != 0)) vec >>= 1;
-  if (vec == 8) vec = 4; // 8-byte lanes are not instantiated
-  int unroll = 1, policy = 1;
-  if (vec == 16 && g_move_variant > 0) {
-    if ((g_move_variant & 0xf) == 4) unroll = 4;
-    const int pc = (g_move_variant >> 8) & 0xf;
-    if (pc == 1 || pc == 2) policy = pc - 1;
-  }
-  if (vec != 16) { unroll = 4; policy = 0; } // rare unaligned shapes: narrower lanes, four per lane
-  const int64_t tile_bytes = (int64_t)unroll * kThreads * vec;
-  const int64_t tpc = (p.chunk_bytes + tile_bytes - 1) / tile_bytes;
-  if (tpc > 0x7fffffffLL)
-    return fail(EMM_EINVAL, "%s: chunk of %lld bytes needs too many tiles", what, (long long)p.chunk_bytes);
-
-  const int64_t j_begin = p.j0, j_end = p.j0 + p.n;
-  for (int64_t j0 = j_begin; j0 < j_end; j0 += kMaxGridY) {
-    const int64_t ny = (j_end - j0 < kMaxGridY) ? (j_end - j0) : kMaxGridY;
-    MoveParams q = p;
-    q.j0 = j0;
-    q.j_end = j0 + ny;
-    dim3 grid((uint32_t)tpc, (uint32_t)ny, (uint32_t)planes);
-    if (SP && DP) grid = dim3((uint32_t)tpc, (uint32_t)(planes * kRun), (uint32_t)((ny + kRun - 1) / kRun));
-    // Scatter from a linear buffer (unpack): visiting a plane for thousands of blocks in a row
-    // keeps all writes inside that plane's address window, which this memory system serves
-    // about 12 % slower than writes spread over the whole pool. Long tables are therefore
-    // walked in groups of 128 blocks per plane visit (y = plane * 128 + position, z = group);
-    // short tables already leave a plane after a few hundred blocks. Gathers (pack) measured
-    // faster in the plain order and keep it.
-    int glog = (!SP && DP && ny >= 1024) ? 7 : 0;
-    if ((g_move_variant >> 16) & 0xf) glog = ((g_move_variant >> 16) & 0xf) == 0xf ? 0 : (g_move_variant >> 16) & 0xf;
-    if (!(SP && DP) && glog > 0 && (planes << glog) <= kMaxGridY) {
-      q.group_log2 = glog;
-      grid = dim3((uint32_t)tpc, (uint32_t)(planes << glog), (uint32_t)((ny + (1 << glog) - 1) >> glog));
-    }
-    if (vec == 16 && unroll == 1) launch_move_policy<u32x4, 1, SP, DP>(q, grid, policy, s);
-    else if (vec == 16) launch_move_policy<u32x4, 4, SP, DP>(q, grid, policy, s);
-    else if (vec == 4) launch_move_policy<uint32_t, 4, SP, DP>(q, grid, 0, s);
-    else if (vec == 2) launch_move_policy<uint16_t, 4, SP, DP>(q, grid, 0, s);
-    else launch_move_policy<uint8_t, 4, SP, DP>(q, grid, 0, s);
-    const int rc = check_launch(what);
-    if (rc != EMM_OK) return rc;
-  }
-  return EMM_OK;
+template <int KIND, int ORDER, bool PAIRS>
+void launch_move_vec(const MoveArgs &a, uint32_t n, uint32_t order_arg, dim3 grid, int vec, int policy, bool full,
+                     const PlaneTables<KIND == kPoolToPool ? 2 : 1> &t, hipStream_t s) {
+  // 16-byte lanes: one vector per lane, sc0 sc1 stores (nt stores in benchmark builds on request);
+  // rare unaligned shapes: narrower lanes, four per lane, nt stores
+  if (vec == 16 && policy == 1) launch_move_full<u32x4, 1, KIND, ORDER, PAIRS, 1>(a, n, order_arg, grid, full, t, s);
+  else if (vec == 16) launch_move_full<u32x4, 1, KIND, ORDER, PAIRS, 0>(a, n, order_arg, grid, full, t, s);
+  else if (vec == 4) launch_move_full<uint32_t, 4, KIND, ORDER, PAIRS, 0>(a, n, order_arg, grid, false, t, s);
+  else if (vec == 2) launch_move_full<uint16_t, 4, KIND, ORDER, PAIRS, 0>(a, n, order_arg, grid, false, t, s);
+  else launch_move_full<uint8_t, 4, KIND, ORDER, PAIRS, 0>(a, n, order_arg, grid, false, t, s);
 }
 
 int common_align(int a, const void *p) {
@@ -348,6 +335,8 @@ int check_pool_args(const char *what, const void *const *layer_ptrs, int num_lay
   if (num_kv < 0 || num_blocks < 0 || chunk_bytes < 0 || n < 0)
     return fail(EMM_EINVAL, "%s: negative size (num_kv=%d num_blocks=%lld chunk_bytes=%lld n=%lld)",
                 what, num_kv, (long long)num_blocks, (long long)chunk_bytes, (long long)n);
+  if (num_blocks > 0x7fffffffLL)
+    return fail(EMM_EINVAL, "%s: num_blocks=%lld exceeds 2^31-1", what, (long long)num_blocks);
   if (num_layers > 0 && !layer_ptrs) return fail(EMM_EINVAL, "%s: layer_ptrs is null", what);
   for (int l = 0; l < num_layers; ++l)
     if (!layer_ptrs[l] && n > 0 && num_blocks > 0)
@@ -355,43 +344,76 @@ int check_pool_args(const char *what, const void *const *layer_ptrs, int num_lay
   return EMM_OK;
 }
 
-// Build the plane tables for groups of at most kMaxPlanes (layer, kv) planes and
-// launch. A null layer table means that side is the linear buffer.
-template <bool SP, bool DP>
+// Build the plane tables for groups of at most kMaxPlanes (layer, kv) planes and launch, at most
+// kMaxGridY blocks per launch. A null layer table means that side is the linear buffer
+// [planes, n, chunk]. `pairs`: idx_a holds (src, dst) pairs (copy_blocks).
+template <int KIND>
 int move_planes(const void *const *src_layers, int64_t src_nb, void *const *dst_layers,
                 int64_t dst_nb, int num_layers, int num_kv, int64_t chunk,
-                const int64_t *src_idx, const int64_t *dst_idx, int64_t idx_stride, int64_t n,
-                const void *src_linear, void *dst_linear, hipStream_t s, const char *what) {
+                const int64_t *idx_a, const int64_t *idx_b, bool pairs, int64_t n,
+                const void *linear, hipStream_t s, const char *what) {
+  constexpr bool SP = KIND != kUnpack, DP = KIND != kPack;
+  if (n == 0 || num_layers == 0 || num_kv == 0 || chunk == 0) return EMM_OK;
   int al = 16;
-  if (!SP) al = common_align(al, src_linear);
-  if (!DP) al = common_align(al, dst_linear);
+  if (KIND != kPoolToPool) al = common_align(al, linear);
   for (int l = 0; l < num_layers; ++l) {
     if (SP) al = common_align(al, src_layers[l]);
     if (DP) al = common_align(al, dst_layers[l]);
   }
+  // widest lane access that divides the chunk and every base address
+  int vec = 16;
+  while (vec > 1 && (chunk % vec != 0 || al % vec != 0)) vec >>= 1;
+  if (vec == 8) vec = 4; // 8-byte lanes are not instantiated
+  int policy = 1;
+  if (vec == 16 && ((move_variant() >> 8) & 0xf) == 1) policy = 0;
+  const int64_t tile_bytes = (int64_t)(vec == 16 ? 1 : 4) * kThreads * vec;
+  const int64_t tpc = (chunk + tile_bytes - 1) / tile_bytes;
+  if (tpc > 0x7fffffffLL)
+    return fail(EMM_EINVAL, "%s: chunk of %lld bytes needs too many tiles", what, (long long)chunk);
+  const bool full = chunk % tile_bytes == 0;
+
   const int64_t planes = (int64_t)num_layers * num_kv;
   for (int64_t pl0 = 0; pl0 < planes; pl0 += kMaxPlanes) {
     const int cnt = (int)((planes - pl0 < kMaxPlanes) ? (planes - pl0) : kMaxPlanes);
-    MoveParams p;
-    memset(&p, 0, sizeof(p));
+    PlaneTables<KIND == kPoolToPool ? 2 : 1> t;
     for (int i = 0; i < cnt; ++i) {
       const int64_t l = (pl0 + i) / num_kv, kv = (pl0 + i) % num_kv;
-      if (SP) p.src_planes[i] = (const char *)src_layers[l] + kv * src_nb * chunk;
-      if (DP) p.dst_planes[i] = (char *)dst_layers[l] + kv * dst_nb * chunk;
+      if (SP) t.t[0].base[i] = (char *)src_layers[l] + kv * src_nb * chunk;
+      if (DP) t.t[KIND == kPoolToPool ? 1 : 0].base[i] = (char *)dst_layers[l] + kv * dst_nb * chunk;
     }
-    p.src_linear = (const char *)src_linear;
-    p.dst_linear = (char *)dst_linear;
-    p.src_idx = src_idx;
-    p.dst_idx = dst_idx;
-    p.idx_stride = idx_stride;
-    p.src_num_blocks = src_nb;
-    p.dst_num_blocks = dst_nb;
-    p.chunk_bytes = chunk;
-    p.n = n;
-    p.j0 = 0;
-    p.plane0 = pl0;
-    const int rc = launch_move<SP, DP>(p, cnt, al, s, what);
-    if (rc != EMM_OK) return rc;
+    for (int64_t j0 = 0; j0 < n; j0 += kMaxGridY) {
+      const int64_t ny = (n - j0 < kMaxGridY) ? (n - j0) : kMaxGridY;
+      MoveArgs a;
+      a.idx_a = idx_a ? idx_a + (pairs ? 2 * j0 : j0) : nullptr;
+      a.idx_b = idx_b ? idx_b + j0 : nullptr;
+      a.lin = linear ? (char *)linear + (pl0 * n + j0) * chunk : nullptr;
+      a.lin_plane_stride = n * chunk;
+      a.chunk = chunk;
+      a.src_nb = (uint32_t)src_nb;
+      a.dst_nb = (uint32_t)dst_nb;
+      if constexpr (KIND == kPoolToPool) {
+        const uint32_t runs = (uint32_t)((ny + kRun - 1) / kRun);
+        const dim3 grid((uint32_t)tpc, (uint32_t)(cnt * kRun), runs);
+        if (pairs) launch_move_vec<KIND, kOrderRuns, true>(a, (uint32_t)ny, runs / cnt, grid, vec, policy, full, t, s);
+        else launch_move_vec<KIND, kOrderRuns, false>(a, (uint32_t)ny, runs / cnt, grid, vec, policy, full, t, s);
+      } else {
+        // long scatters (unpack) are walked in groups of 128 blocks per plane visit; short tables
+        // already leave a plane after a few hundred blocks, and gathers (pack) measured faster in
+        // the plain order
+        int glog = (KIND == kUnpack && ny >= 1024) ? 7 : 0;
+        const int forced = (move_variant() >> 16) & 0xf;
+        if (forced) glog = forced == 0xf ? 0 : forced;
+        if (glog > 0 && ((int64_t)cnt << glog) <= kMaxGridY) {
+          const dim3 grid((uint32_t)tpc, (uint32_t)(cnt << glog), (uint32_t)((ny + (1 << glog) - 1) >> glog));
+          launch_move_vec<KIND, kOrderGrouped, false>(a, (uint32_t)ny, (uint32_t)glog, grid, vec, policy, full, t, s);
+        } else {
+          const dim3 grid((uint32_t)tpc, (uint32_t)ny, (uint32_t)cnt);
+          launch_move_vec<KIND, kOrderPlain, false>(a, (uint32_t)ny, 0, grid, vec, policy, full, t, s);
+        }
+      }
+      const int rc = check_launch(what);
+      if (rc != EMM_OK) return rc;
+    }
   }
   return EMM_OK;
 }
@@ -413,32 +435,35 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
 // fp32 -> e4m3fn with the rule of torch's cast: round to nearest even, no
 // saturation; what rounds past 448 (464 is the tie that still gives 448), +-inf
 // and NaN give sign|0x7F. gfx950's v_cvt_pk_fp8_f32 (OCP e4m3, overflow mode off)
-// implements exactly this for every non-NaN fp32 input — checked against the
-// integer formulation below over all 2^32 bit patterns on the device — and
-// returns 0xFF for every NaN, so NaN inputs are first replaced by the infinity of
-// their sign.
-__device__ __forceinline__ float nan_to_signed_inf(float f) {
-  const uint32_t u = __float_as_uint(f);
-  uint32_t a = u & 0x7fffffffu;
-  a = a < 0x7f800000u ? a : 0x7f800000u;
-  return __uint_as_float(a | (u & 0x80000000u));
+// implements this for every non-NaN fp32 input and returns 0xFF for every NaN, so NaNs
+// are first replaced by the infinity of their sign (the GPU tests compare the conversion
+// with the oracle for every 16-bit input at many scales).
+//
+// Two overflow modes:
+//   SAT = false  torch's x.to(float8_e4m3fn): overflow, +-inf and NaN -> sign|0x7F;
+//   SAT = true   clamp(q, -448, 448) first (vLLM's fp8 KV-cache convention): overflow and
+//                +-inf -> sign|0x7E (448), NaN stays NaN (sign|0x7F).
+// finish_quotient prepares a quotient for the hardware conversion: |q| limited to inf
+// (SAT: to 448) with one IEEE minimum — which also maps a NaN q to the limit, because the
+// minimum returns its non-NaN operand —, `is_nan` (SAT only) puts the NaN back as an
+// infinity, and the sign is taken from `sign_bits`.
+template <bool SAT>
+__device__ __forceinline__ float finish_quotient(float q, bool is_nan, uint32_t sign_bits) {
+  float a = __builtin_fminf(__builtin_fabsf(q), SAT ? 448.0f : __builtin_inff());
+  if constexpr (SAT) a = is_nan ? __builtin_inff() : a;
+  return __uint_as_float(__float_as_uint(a) | (sign_bits & 0x80000000u));
 }
 
-// four fp32 -> four e4m3fn bytes in one dword (byte k = value k)
-__device__ __forceinline__ uint32_t f32x4_to_e4m3fn(float q0, float q1, float q2, float q3) {
-  int r = 0;
-  r = __builtin_amdgcn_cvt_pk_fp8_f32(nan_to_signed_inf(q0), nan_to_signed_inf(q1), r, false);
-  r = __builtin_amdgcn_cvt_pk_fp8_f32(nan_to_signed_inf(q2), nan_to_signed_inf(q3), r, true);
-  return (uint32_t)r;
-}
+__device__ __forceinline__ bool is_nan_bits(float f) { return (__float_as_uint(f) & 0x7fffffffu) > 0x7f800000u; }
 
-// The same rule in integer arithmetic, one value at a time (element-wise path).
+// The rule in integer arithmetic, one value at a time (element-wise path); `f` has been
+// through finish_quotient (no NaN).
 __device__ __forceinline__ uint32_t f32_to_e4m3fn(float f) {
   const uint32_t u = __float_as_uint(f);
   const uint32_t sign = (u >> 24) & 0x80u;
   uint32_t a = u & 0x7fffffffu;
   uint32_t r;
-  if (a >= 0x43f00000u) { // >= 480, inf, NaN
+  if (a >= 0x43f00000u) { // >= 480, inf
     r = 0x7fu;
   } else if (a < 0x3c800000u) { // below 2^-6: subnormal grid of 2^-9
     // |f| * 2^9 is exact; rintf rounds to nearest even; 8 encodes 2^-6
@@ -460,15 +485,18 @@ __device__ __forceinline__ float half_bits_to_f32(uint32_t h) {
     return f16_bits_to_f32(h);
 }
 
-// x / scale for a scale shared by a whole wave. The correctly rounded quotient is what torch's
-// cast sees, so it must be reproduced bit for bit. For 2^-30 <= scale <= 2^30 it is obtained
-// without the IEEE division sequence: with y = RN(1 / scale), q = RN(x * y),
-// r = fma(-q, scale, x) (exact), the quotient is fma(r, y, q) — checked on the device against the
-// division for every 16-bit input and 2^20 scales. The correction step turns an infinite q (x
-// infinite, or the product overflows) into a NaN and loses the sign of -0, and the conversion
-// wants NaNs replaced by infinities anyway: min(|q'|, inf) maps every NaN to +inf (the IEEE
-// minimum returns its non-NaN operand) and the sign of x is put back, which is the sign of the
-// quotient for a positive scale. Other scales (and negative ones) take the division.
+// x / scale for a scale shared by a whole wave. The correctly rounded fp32 quotient is what
+// torch's cast sees, so it must be reproduced bit for bit. For 2^-30 <= scale <= 2^30 it is
+// obtained without the IEEE division sequence: with y = RN(1 / scale), q = RN(x * y),
+// r = fma(-q, scale, x), the quotient is q' = fma(r, y, q). That q' equals RN(x / scale) for
+// every input with at most 11 significant bits (all f16 and bf16 values) and every scale is
+// established by exhaustion: the three operations commute with powers of two as long as nothing
+// leaves the normal range, so the identity only depends on the two significands, and the GPU test
+// suite checks all 2^10 x 2^23 significand pairs against the division (and, for what leaves the
+// normal range, that the result still converts to the same byte). The correction step turns an
+// infinite q (x infinite, or the product overflows) into a NaN and loses the sign of -0;
+// finish_quotient repairs both, the sign of x being the sign of the quotient for a positive
+// scale. Other scales (and negative ones) take the division.
 struct Divisor {
   float scale;
   float recip;
@@ -483,17 +511,27 @@ __device__ __forceinline__ Divisor make_divisor(float scale, bool allow_fast) {
   return d;
 }
 
-// |x / scale| with NaN -> inf, carrying the sign of x: ready for the hardware conversion
-__device__ __forceinline__ float divide_fast_nan_free(float x, const Divisor &d) {
+// the bare fast quotient (may be NaN where the division gives +-inf, see above)
+__device__ __forceinline__ float divide_fast_raw(float x, const Divisor &d) {
   const float q = x * d.recip;
   const float r = __builtin_fmaf(-q, d.scale, x);
-  const float q2 = __builtin_fmaf(r, d.recip, q);
-  const float a = __builtin_fminf(__builtin_fabsf(q2), __builtin_inff());
-  return __uint_as_float(__float_as_uint(a) | (__float_as_uint(x) & 0x80000000u));
+  return __builtin_fmaf(r, d.recip, q);
+}
+
+// x / scale, ready for the hardware conversion (no NaN, limited as the mode demands)
+template <bool SAT>
+__device__ __forceinline__ float divide_fast(float x, const Divisor &d) {
+  return finish_quotient<SAT>(divide_fast_raw(x, d), is_nan_bits(x), __float_as_uint(x));
+}
+
+template <bool SAT>
+__device__ __forceinline__ float divide_ieee(float x, float scale) {
+  const float q = x / scale;
+  return finish_quotient<SAT>(q, is_nan_bits(q), __float_as_uint(q));
 }
 
 // 8 sixteen-bit values (one u32x4) -> 8 e4m3fn bytes (one u32x2), q = rne(x / scale).
-template <int SRC_DTYPE>
+template <int SRC_DTYPE, bool SAT>
 __device__ __forceinline__ u32x2 quant8(u32x4 in, const Divisor &d) {
   u32x2 out;
   if (d.exact_fast) {
@@ -501,23 +539,31 @@ __device__ __forceinline__ u32x2 quant8(u32x4 in, const Divisor &d) {
     for (int w = 0; w < 2; ++w) {
       const uint32_t w0 = in[w * 2], w1 = in[w * 2 + 1];
       int r = 0;
-      r = __builtin_amdgcn_cvt_pk_fp8_f32(divide_fast_nan_free(half_bits_to_f32<SRC_DTYPE>(w0 & 0xffffu), d),
-                                          divide_fast_nan_free(half_bits_to_f32<SRC_DTYPE>(w0 >> 16), d), r, false);
-      r = __builtin_amdgcn_cvt_pk_fp8_f32(divide_fast_nan_free(half_bits_to_f32<SRC_DTYPE>(w1 & 0xffffu), d),
-                                          divide_fast_nan_free(half_bits_to_f32<SRC_DTYPE>(w1 >> 16), d), r, true);
+      r = __builtin_amdgcn_cvt_pk_fp8_f32(divide_fast<SAT>(half_bits_to_f32<SRC_DTYPE>(w0 & 0xffffu), d),
+                                          divide_fast<SAT>(half_bits_to_f32<SRC_DTYPE>(w0 >> 16), d), r, false);
+      r = __builtin_amdgcn_cvt_pk_fp8_f32(divide_fast<SAT>(half_bits_to_f32<SRC_DTYPE>(w1 & 0xffffu), d),
+                                          divide_fast<SAT>(half_bits_to_f32<SRC_DTYPE>(w1 >> 16), d), r, true);
       out[w] = (uint32_t)r;
     }
   } else {
 #pragma unroll
     for (int w = 0; w < 2; ++w) {
       const uint32_t w0 = in[w * 2], w1 = in[w * 2 + 1];
-      out[w] = f32x4_to_e4m3fn(half_bits_to_f32<SRC_DTYPE>(w0 & 0xffffu) / d.scale,
-                               half_bits_to_f32<SRC_DTYPE>(w0 >> 16) / d.scale,
-                               half_bits_to_f32<SRC_DTYPE>(w1 & 0xffffu) / d.scale,
-                               half_bits_to_f32<SRC_DTYPE>(w1 >> 16) / d.scale);
+      int r = 0;
+      r = __builtin_amdgcn_cvt_pk_fp8_f32(divide_ieee<SAT>(half_bits_to_f32<SRC_DTYPE>(w0 & 0xffffu), d.scale),
+                                          divide_ieee<SAT>(half_bits_to_f32<SRC_DTYPE>(w0 >> 16), d.scale), r, false);
+      r = __builtin_amdgcn_cvt_pk_fp8_f32(divide_ieee<SAT>(half_bits_to_f32<SRC_DTYPE>(w1 & 0xffffu), d.scale),
+                                          divide_ieee<SAT>(half_bits_to_f32<SRC_DTYPE>(w1 >> 16), d.scale), r, true);
+      out[w] = (uint32_t)r;
     }
   }
   return out;
+}
+
+// one value, element-wise paths (always the division)
+template <int SRC_DTYPE, bool SAT>
+__device__ __forceinline__ uint8_t quant1(uint32_t h, float scale) {
+  return (uint8_t)f32_to_e4m3fn(divide_ieee<SAT>(half_bits_to_f32<SRC_DTYPE>(h), scale));
 }
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -628,165 +674,144 @@ __global__ __launch_bounds__(kThreads) void emm_unpack_dequant_fp8_kernel(const 
 // ----------------------------------------------------------------------------
 // reshape_and_cache: row scatter by slot_mapping
 // ----------------------------------------------------------------------------
-struct AppendParams {
+// Per-layer pointer tables of the whole-step launches (one launch for all layers).
+struct AppendTables {
   const char *key[EMM_MAX_LAYERS];
   const char *value[EMM_MAX_LAYERS];
   char *key_cache[EMM_MAX_LAYERS];
   char *value_cache[EMM_MAX_LAYERS];
-  const int64_t *slot_mapping;
-  const float *k_scales; // fp8 only
-  const float *v_scales;
-  int64_t num_tokens;
-  int64_t row_bytes;  // source row bytes (copy) / source row elements (fp8)
-  int64_t key_stride; // bytes (copy) / elements (fp8)
-  int64_t value_stride;
-  int64_t num_slots;
-  int32_t fast_div; // fp8: 0 forces the IEEE division (benchmarks)
 };
+struct NoTables {};
 
 constexpr int kWavesPerGroup = kThreads / 64;
 
-// Rows per wave of the append kernels: 0 = default. Set through the tuning hook.
-int g_append_rows = 0;
-
-// Fetch the slots of R consecutive tokens. The loads are only issued here (one
-// address for all lanes); resolve_slots() waits for them, moves the values to
-// scalar registers and turns padding (< 0) and out-of-range slots into -1.
-template <int R>
-__device__ __forceinline__ void fetch_slots(int64_t (&s)[R], const int64_t *slot_mapping, int64_t t0,
-                                            int64_t num_tokens) {
+// One wave moves R token rows, K and V both: the slot of a token is fetched once (a scalar load: the
+// token index is wave-uniform) and 2 R sixteen-byte loads per lane are in flight before the first
+// store. The source rows do not depend on the slots, so their loads are issued before the slots are
+// waited for (rows of padded tokens are read and dropped). A model forward calls this once per layer
+// with some tens of megabytes, where the time of a launch is its ramp: every scalar argument is an
+// explicit kernel parameter, ordered by first use, so that the hardware has preloaded it into scalar
+// registers when the wave starts (kernarg preload) and the first loads go out at once; small
+// workgroups (one wave) start and drain fastest. TABLES: the four tensor pointers come from
+// per-layer tables in the argument block instead (grid z = layer), one more scalar round trip.
+// grid: x = groups of WAVES * R tokens, z = layers (TABLES) or 1.
+template <typename V, int R, int WAVES, int POLICY, bool TABLES>
+__global__ __launch_bounds__(WAVES * 64) void emm_append_kernel(
+    const int64_t *__restrict__ slot_mapping, const char *key, const char *value, char *key_cache,
+    char *value_cache, uint32_t num_tokens, uint32_t row_bytes, uint32_t key_stride, uint32_t value_stride,
+    int64_t num_slots, const std::conditional_t<TABLES, AppendTables, NoTables> tables) {
+  // (the 14 dwords up to value_stride are preloaded; num_slots is fetched while the loads are in flight)
+  constexpr uint32_t VB = sizeof(V);
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = WAVES == 1 ? 0u : (uint32_t)__builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t t0 = (blockIdx.x * WAVES + wave) * R;
+  if (t0 >= num_tokens) return;
+  if constexpr (TABLES) {
+    const uint32_t l = blockIdx.z;
+    key = tables.key[l];
+    value = tables.value[l];
+    key_cache = tables.key_cache[l];
+    value_cache = tables.value_cache[l];
+  }
+  int64_t slot[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) slot[r] = t0 + r < num_tokens ? slot_mapping[t0 + r] : -1;
+  uint32_t off = lane * VB;
+  V a[R], b[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const int64_t t = t0 + r;
-    s[r] = -1;
-    if (t < num_tokens) s[r] = ld<int64_t, false>((const char *)(slot_mapping + t));
+    const uint32_t t = t0 + r < num_tokens ? t0 + r : num_tokens - 1; // tail: re-read the last row, dropped below
+    const uint32_t o = off < row_bytes ? off : 0;
+    a[r] = ld_stream<V, POLICY>(key + (uint64_t)t * key_stride + o);
+    b[r] = ld_stream<V, POLICY>(value + (uint64_t)t * value_stride + o);
   }
-}
-
-template <int R>
-__device__ __forceinline__ void resolve_slots(int64_t (&s)[R], int64_t num_slots) {
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    s[r] = uniform64(s[r]);
-    if ((uint64_t)s[r] >= (uint64_t)num_slots) s[r] = -1;
+    asm volatile("" : "+s"(slot[r]) : : "memory");
+    if ((uint64_t)slot[r] >= (uint64_t)num_slots) slot[r] = -1; // padding (< 0) and out-of-range slots: skipped
   }
-}
-
-// One wave moves R token rows of K or V: grid x = groups of 4 * R tokens,
-// y = 2 (K, V), z = layers. The source rows do not depend on the slots, so their
-// first loads are issued before the slots are waited for (rows of padded tokens
-// are read and dropped).
-template <typename V, int R, int POLICY>
-__global__ __launch_bounds__(kThreads) void emm_append_kernel(const AppendParams p) {
-  constexpr int64_t VB = sizeof(V);
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const uint32_t kv = blockIdx.y, l = blockIdx.z;
-  const int64_t t0 = ((int64_t)blockIdx.x * kWavesPerGroup + wave) * R;
-  if (t0 >= p.num_tokens) return;
-  const char *src_base = kv == 0 ? p.key[l] : p.value[l];
-  char *dst_base = kv == 0 ? p.key_cache[l] : p.value_cache[l];
-  const int64_t stride = kv == 0 ? p.key_stride : p.value_stride;
-  const int64_t row_bytes = p.row_bytes;
-
-  int64_t slot[R];
-  fetch_slots<R>(slot, p.slot_mapping, t0, p.num_tokens);
-  int64_t off = (int64_t)lane * VB;
-  V v[R];
-#pragma unroll
-  for (int r = 0; r < R; ++r)
-    if (t0 + r < p.num_tokens && off < row_bytes)
-      v[r] = ld_stream<V, POLICY>(src_base + (t0 + r) * stride + off);
-  resolve_slots<R>(slot, p.num_slots);
-#pragma unroll
-  for (int r = 0; r < R; ++r)
-    if (slot[r] >= 0 && off < row_bytes) st_stream<V, POLICY>(dst_base + slot[r] * row_bytes + off, v[r]);
-  for (off += 64 * VB; off < row_bytes; off += 64 * VB) {
+  if (off < row_bytes) {
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      if (slot[r] >= 0) v[r] = ld_stream<V, POLICY>(src_base + (t0 + r) * stride + off);
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-      if (slot[r] >= 0) st_stream<V, POLICY>(dst_base + slot[r] * row_bytes + off, v[r]);
-  }
-}
-
-// fp8 append. VEC_ELEMS = 8: a wave converts a row in pieces of 1024 elements; lane i
-// loads elements [8i, 8i+8) and [512+8i, 512+8i+8) of the piece (two 16-byte loads, each
-// instruction 1 KiB contiguous) and stores the two 8-byte results at those element offsets
-// (each instruction 512 contiguous bytes of whole cache lines). VEC_ELEMS = 1:
-// element-wise path for rows that are not a multiple of 8 elements or misaligned bases.
-template <int SRC_DTYPE, int VEC_ELEMS, int R>
-__global__ __launch_bounds__(kThreads) void emm_append_fp8_kernel(const AppendParams p) {
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const uint32_t kv = blockIdx.y, l = blockIdx.z;
-  const int64_t t0 = ((int64_t)blockIdx.x * kWavesPerGroup + wave) * R;
-  if (t0 >= p.num_tokens) return;
-  const char *src_base = kv == 0 ? p.key[l] : p.value[l];
-  char *dst_base = kv == 0 ? p.key_cache[l] : p.value_cache[l];
-  const int64_t stride = kv == 0 ? p.key_stride : p.value_stride;
-  const float scale = kv == 0 ? p.k_scales[l] : p.v_scales[l];
-  const Divisor div = make_divisor(scale, p.fast_div != 0);
-  const int64_t row = p.row_bytes; // elements
-
-  int64_t slot[R];
-  fetch_slots<R>(slot, p.slot_mapping, t0, p.num_tokens);
-  if constexpr (VEC_ELEMS == 8) {
-    int64_t e0 = (int64_t)lane * 8, e1 = e0 + 512;
-    u32x4 a[R], b[R];
-    // first piece: issued before the slots are waited for (rows of padded tokens are read and dropped)
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-      if (t0 + r < p.num_tokens) {
-        const char *sp = src_base + (t0 + r) * stride * 2;
-        a[r] = ld<u32x4, true>(sp + (e0 < row ? e0 : 0) * 2);
-        b[r] = ld<u32x4, true>(sp + (e1 < row ? e1 : 0) * 2);
+      if (slot[r] >= 0) {
+        st_stream<V, POLICY>(key_cache + slot[r] * (int64_t)row_bytes + off, a[r]);
+        st_stream<V, POLICY>(value_cache + slot[r] * (int64_t)row_bytes + off, b[r]);
       }
-    resolve_slots<R>(slot, p.num_slots);
-    while (e0 < row) {
+  }
+  for (off += 64 * VB; off < row_bytes; off += 64 * VB) { // rows longer than 64 vectors
 #pragma unroll
-      for (int r = 0; r < R; ++r)
-        if (slot[r] >= 0) {
-          char *dp = dst_base + slot[r] * row;
-          const u32x2 qa = quant8<SRC_DTYPE>(a[r], div);
-          const u32x2 qb = quant8<SRC_DTYPE>(b[r], div);
-          st_stream<u32x2, 1>(dp + e0, qa);
-          if (e1 < row) st_stream<u32x2, 1>(dp + e1, qb);
-        }
+    for (int r = 0; r < R; ++r)
+      if (slot[r] >= 0) {
+        a[r] = ld_stream<V, POLICY>(key + (uint64_t)(t0 + r) * key_stride + off);
+        b[r] = ld_stream<V, POLICY>(value + (uint64_t)(t0 + r) * value_stride + off);
+      }
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (slot[r] >= 0) {
+        st_stream<V, POLICY>(key_cache + slot[r] * (int64_t)row_bytes + off, a[r]);
+        st_stream<V, POLICY>(value_cache + slot[r] * (int64_t)row_bytes + off, b[r]);
+      }
+  }
+}
+
+// fp8 append: one wave quantises one token row of K or V (grid y = 2). VEC_ELEMS = 8: the row is
+// converted in pieces of 1024 elements; lane i loads elements [8i, 8i+8) and [512+8i, 512+8i+8) of the
+// piece (two 16-byte loads, each instruction 1 KiB contiguous) and stores the two 8-byte results at
+// those element offsets (each instruction 512 contiguous bytes of whole cache lines). VEC_ELEMS = 1:
+// element-wise path for rows that are not a multiple of 8 elements or misaligned bases. Scalar
+// arguments are explicit and ordered by first use, as in emm_append_kernel. Strides and rows in
+// elements. grid: x = groups of 4 tokens, y = 2 (K, V), z = layers (TABLES) or 1.
+template <int SRC_DTYPE, int VEC_ELEMS, bool SAT, bool TABLES>
+__global__ __launch_bounds__(kThreads) void emm_append_fp8_kernel(
+    const int64_t *__restrict__ slot_mapping, const char *key, const char *value, uint32_t num_tokens,
+    uint32_t row, uint32_t key_stride, uint32_t value_stride, const float *__restrict__ k_scales,
+    const float *__restrict__ v_scales, char *key_cache, char *value_cache, int64_t num_slots, int32_t fast_div,
+    const std::conditional_t<TABLES, AppendTables, NoTables> tables) {
+  // (the 14 dwords up to v_scales are preloaded: everything the first loads need)
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t kv = blockIdx.y, l = TABLES ? blockIdx.z : 0;
+  const uint32_t t = blockIdx.x * kWavesPerGroup + wave;
+  if (t >= num_tokens) return;
+  if constexpr (TABLES) {
+    key = tables.key[l];
+    value = tables.value[l];
+    key_cache = tables.key_cache[l];
+    value_cache = tables.value_cache[l];
+  }
+  const char *src = (kv == 0 ? key : value) + (uint64_t)t * (kv == 0 ? key_stride : value_stride) * 2;
+  char *dst_base = kv == 0 ? key_cache : value_cache;
+  int64_t slot = slot_mapping[t];
+  const float scale = kv == 0 ? k_scales[l] : v_scales[l];
+
+  if constexpr (VEC_ELEMS == 8) {
+    uint32_t e0 = lane * 8, e1 = e0 + 512;
+    // first piece: issued before slot and scale are waited for (rows of padded tokens are read and dropped)
+    u32x4 a = ld<u32x4, true>(src + (e0 < row ? e0 : 0) * 2);
+    u32x4 b = ld<u32x4, true>(src + (e1 < row ? e1 : 0) * 2);
+    asm volatile("" : "+s"(slot) : : "memory");
+    if ((uint64_t)slot >= (uint64_t)num_slots) return;
+    const Divisor div = make_divisor(scale, fast_div != 0);
+    char *dp = dst_base + slot * (int64_t)row;
+    while (e0 < row) {
+      const u32x2 qa = quant8<SRC_DTYPE, SAT>(a, div);
+      const u32x2 qb = quant8<SRC_DTYPE, SAT>(b, div);
+      st_stream<u32x2, 1>(dp + e0, qa);
+      if (e1 < row) st_stream<u32x2, 1>(dp + e1, qb);
       e0 += 1024;
       e1 += 1024;
       if (e0 < row) {
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-          if (slot[r] >= 0) {
-            const char *sp = src_base + (t0 + r) * stride * 2;
-            a[r] = ld<u32x4, true>(sp + e0 * 2);
-            b[r] = ld<u32x4, true>(sp + (e1 < row ? e1 : e0) * 2);
-          }
+        a = ld<u32x4, true>(src + e0 * 2);
+        b = ld<u32x4, true>(src + (e1 < row ? e1 : e0) * 2);
       }
     }
   } else {
-    resolve_slots<R>(slot, p.num_slots);
-    for (int64_t e = lane; e < row; e += 64) {
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        if (slot[r] >= 0) {
-          const uint16_t h = ld<uint16_t, false>(src_base + ((t0 + r) * stride + e) * 2);
-          const float x = half_bits_to_f32<SRC_DTYPE>(h) / scale;
-          st<uint8_t, false>(dst_base + slot[r] * row + e, (uint8_t)f32_to_e4m3fn(x));
-        }
-      }
+    if ((uint64_t)slot >= (uint64_t)num_slots) return;
+    for (uint32_t e = lane; e < row; e += 64) {
+      const uint16_t h = ld<uint16_t, false>(src + (int64_t)e * 2);
+      st<uint8_t, false>(dst_base + slot * (int64_t)row + e, quant1<SRC_DTYPE, SAT>(h, scale));
     }
   }
-}
-
-// A walk that cycles through the planes in short runs of tokens (as the long unpack does with
-// blocks) was measured for the whole-step launch and made no difference: a plane is left after
-// 8 MiB of rows anyway.
-dim3 append_grid(int64_t num_tokens, int num_layers, int rows_per_wave) {
-  const int64_t rows_per_group = (int64_t)kWavesPerGroup * rows_per_wave;
-  return dim3((uint32_t)((num_tokens + rows_per_group - 1) / rows_per_group), 2, (uint32_t)num_layers);
 }
 
 int check_append_args(const char *what, const void *const *k, const void *const *v,
@@ -805,100 +830,125 @@ int check_append_args(const char *what, const void *const *k, const void *const 
       return fail(EMM_EINVAL, "%s: null tensor pointer at layer %d", what, l);
   if (ks < row || vs < row)
     return fail(EMM_EINVAL, "%s: token stride smaller than the row", what);
-  if ((num_tokens + 15) / 16 > 0x7fffffffLL) return fail(EMM_EINVAL, "%s: too many tokens", what);
+  if (num_tokens > 0x7fffffffLL) return fail(EMM_EINVAL, "%s: too many tokens", what);
+  if (row > 0x7fffffffLL || ks > 0x7fffffffLL || vs > 0x7fffffffLL)
+    return fail(EMM_EINVAL, "%s: row / token stride of 2 GiB or more", what);
   return EMM_OK;
+}
+
+void fill_tables(AppendTables &t, const void *const *k, const void *const *v, void *const *kc, void *const *vc,
+                 int num_layers) {
+  for (int l = 0; l < num_layers; ++l) {
+    t.key[l] = (const char *)k[l];
+    t.value[l] = (const char *)v[l];
+    t.key_cache[l] = (char *)kc[l];
+    t.value_cache[l] = (char *)vc[l];
+  }
+}
+
+// launch shapes of the 16-byte copy append: (token rows per wave, waves per workgroup)
+template <typename V, int R, int WAVES, int POLICY>
+void launch_append(bool tables, const AppendTables &t, const int64_t *slot_mapping, int64_t num_tokens,
+                   int64_t row_bytes, int64_t ks, int64_t vs, int64_t num_slots, int num_layers, hipStream_t s) {
+  const int64_t per_group = (int64_t)R * WAVES;
+  const uint32_t gx = (uint32_t)((num_tokens + per_group - 1) / per_group);
+  if (tables)
+    emm_append_kernel<V, R, WAVES, POLICY, true><<<dim3(gx, 1, (uint32_t)num_layers), WAVES * 64, 0, s>>>(
+        slot_mapping, nullptr, nullptr, nullptr, nullptr, (uint32_t)num_tokens, (uint32_t)row_bytes, (uint32_t)ks,
+        (uint32_t)vs, num_slots, t);
+  else
+    emm_append_kernel<V, R, WAVES, POLICY, false><<<dim3(gx), WAVES * 64, 0, s>>>(
+        slot_mapping, t.key[0], t.value[0], t.key_cache[0], t.value_cache[0], (uint32_t)num_tokens,
+        (uint32_t)row_bytes, (uint32_t)ks, (uint32_t)vs, num_slots, NoTables{});
 }
 
 int append_copy(const void *const *k, const void *const *v, void *const *kc, void *const *vc,
                 int num_layers, const int64_t *slot_mapping, int64_t num_tokens,
                 int64_t row_bytes, int64_t ks, int64_t vs, int64_t num_slots,
-                hipStream_t s, const char *what) {
+                bool tables, hipStream_t s, const char *what) {
   int rc = check_append_args(what, k, v, kc, vc, num_layers, slot_mapping, num_tokens,
                              row_bytes, ks, vs, num_slots);
   if (rc != EMM_OK) return rc;
   if (num_tokens == 0 || num_layers == 0 || row_bytes == 0) return EMM_OK;
-  AppendParams p;
-  memset(&p, 0, sizeof(p));
+  AppendTables t;
+  fill_tables(t, k, v, kc, vc, num_layers);
   int al = 16;
   for (int l = 0; l < num_layers; ++l) {
-    p.key[l] = (const char *)k[l];
-    p.value[l] = (const char *)v[l];
-    p.key_cache[l] = (char *)kc[l];
-    p.value_cache[l] = (char *)vc[l];
     al = common_align(al, k[l]);
     al = common_align(al, v[l]);
     al = common_align(al, kc[l]);
     al = common_align(al, vc[l]);
   }
-  p.slot_mapping = slot_mapping;
-  p.num_tokens = num_tokens;
-  p.row_bytes = row_bytes;
-  p.key_stride = ks;
-  p.value_stride = vs;
-  p.num_slots = num_slots;
   int vec = al;
   while (vec > 1 && (row_bytes % vec || ks % vec || vs % vec)) vec >>= 1;
-  const int rows = (g_append_rows == 1 || g_append_rows == 2 || g_append_rows == 4) ? g_append_rows : 1;
-  dim3 grid = append_grid(num_tokens, num_layers, vec == 16 ? rows : 4);
   if (vec == 16) {
-    switch (rows) {
-    case 4: emm_append_kernel<u32x4, 4, 1><<<grid, kThreads, 0, s>>>(p); break;
-    case 2: emm_append_kernel<u32x4, 2, 1><<<grid, kThreads, 0, s>>>(p); break;
-    default: emm_append_kernel<u32x4, 1, 1><<<grid, kThreads, 0, s>>>(p); break;
+    // one wave per two tokens in workgroups of one wave: the fastest start and drain of a per-layer
+    // launch; the other shapes exist for benchmark builds
+    switch ((move_variant() >> 12) & 0xf) {
+    case 1: launch_append<u32x4, 1, 4, 1>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
+    case 2: launch_append<u32x4, 2, 4, 1>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
+    case 3: launch_append<u32x4, 4, 1, 1>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
+    case 4: launch_append<u32x4, 1, 1, 1>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
+    default: launch_append<u32x4, 2, 1, 1>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
     }
   } else {
     switch (vec) {
-    case 8: emm_append_kernel<u32x2, 4, 0><<<grid, kThreads, 0, s>>>(p); break;
-    case 4: emm_append_kernel<uint32_t, 4, 0><<<grid, kThreads, 0, s>>>(p); break;
-    case 2: emm_append_kernel<uint16_t, 4, 0><<<grid, kThreads, 0, s>>>(p); break;
-    default: emm_append_kernel<uint8_t, 4, 0><<<grid, kThreads, 0, s>>>(p); break;
+    case 8: launch_append<u32x2, 2, 4, 0>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
+    case 4: launch_append<uint32_t, 2, 4, 0>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
+    case 2: launch_append<uint16_t, 2, 4, 0>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
+    default: launch_append<uint8_t, 2, 4, 0>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
     }
   }
   return check_launch(what);
 }
 
+template <int DT, int VEC, bool SAT>
+void launch_append_fp8(bool tables, const AppendTables &t, const int64_t *slot_mapping, const float *k_scales,
+                       const float *v_scales, int64_t num_tokens, int64_t row, int64_t ks, int64_t vs,
+                       int64_t num_slots, int fast_div, int num_layers, hipStream_t s) {
+  const uint32_t gx = (uint32_t)((num_tokens + kWavesPerGroup - 1) / kWavesPerGroup);
+  if (tables)
+    emm_append_fp8_kernel<DT, VEC, SAT, true><<<dim3(gx, 2, (uint32_t)num_layers), kThreads, 0, s>>>(
+        slot_mapping, nullptr, nullptr, (uint32_t)num_tokens, (uint32_t)row, (uint32_t)ks, (uint32_t)vs, k_scales,
+        v_scales, nullptr, nullptr, num_slots, fast_div, t);
+  else
+    emm_append_fp8_kernel<DT, VEC, SAT, false><<<dim3(gx, 2), kThreads, 0, s>>>(
+        slot_mapping, t.key[0], t.value[0], (uint32_t)num_tokens, (uint32_t)row, (uint32_t)ks, (uint32_t)vs,
+        k_scales, v_scales, t.key_cache[0], t.value_cache[0], num_slots, fast_div, NoTables{});
+}
+
 int append_fp8(const void *const *k, const void *const *v, void *const *kc, void *const *vc,
                int num_layers, const int64_t *slot_mapping, int64_t num_tokens,
                int64_t row_elems, int64_t ks, int64_t vs, int64_t num_slots,
-               const float *k_scales, const float *v_scales, int src_dtype,
+               const float *k_scales, const float *v_scales, int src_dtype, bool tables,
                hipStream_t s, const char *what) {
   int rc = check_append_args(what, k, v, kc, vc, num_layers, slot_mapping, num_tokens,
                              row_elems, ks, vs, num_slots);
   if (rc != EMM_OK) return rc;
-  if (src_dtype != EMM_DTYPE_BF16 && src_dtype != EMM_DTYPE_F16)
+  const bool sat = (src_dtype & EMM_FP8_SATURATE) != 0;
+  const int dt = src_dtype & ~EMM_FP8_SATURATE;
+  if (dt != EMM_DTYPE_BF16 && dt != EMM_DTYPE_F16)
     return fail(EMM_EINVAL, "%s: unknown src_dtype %d", what, src_dtype);
   if (num_tokens == 0 || num_layers == 0 || row_elems == 0) return EMM_OK;
   if (!k_scales || !v_scales) return fail(EMM_EINVAL, "%s: scale pointer is null", what);
-  AppendParams p;
-  memset(&p, 0, sizeof(p));
+  AppendTables t;
+  fill_tables(t, k, v, kc, vc, num_layers);
   int width = (row_elems % 8 || ks % 8 || vs % 8) ? 1 : 8;
   for (int l = 0; l < num_layers; ++l) {
-    p.key[l] = (const char *)k[l];
-    p.value[l] = (const char *)v[l];
-    p.key_cache[l] = (char *)kc[l];
-    p.value_cache[l] = (char *)vc[l];
     if (!aligned(k[l], 2) || !aligned(v[l], 2))
       return fail(EMM_EINVAL, "%s: 16-bit source not 2-byte aligned at layer %d", what, l);
     if (!aligned(k[l], 16) || !aligned(v[l], 16) || !aligned(kc[l], 8) || !aligned(vc[l], 8)) width = 1;
   }
-  p.slot_mapping = slot_mapping;
-  p.k_scales = k_scales;
-  p.v_scales = v_scales;
-  p.num_tokens = num_tokens;
-  p.row_bytes = row_elems;
-  p.key_stride = ks;
-  p.value_stride = vs;
-  p.num_slots = num_slots;
-  p.fast_div = (g_move_variant & 0x1000000) ? 0 : 1;
-  const int rows = (g_append_rows == 1 || g_append_rows == 2 || g_append_rows == 4) ? g_append_rows : 1;
-  dim3 grid = append_grid(num_tokens, num_layers, width == 8 ? rows : 4);
-#define EMM_FP8_LAUNCH(DT)                                                                  \
-  if (width == 8) {                                                                         \
-    if (rows == 4) emm_append_fp8_kernel<DT, 8, 4><<<grid, kThreads, 0, s>>>(p);            \
-    else if (rows == 2) emm_append_fp8_kernel<DT, 8, 2><<<grid, kThreads, 0, s>>>(p);       \
-    else emm_append_fp8_kernel<DT, 8, 1><<<grid, kThreads, 0, s>>>(p);                      \
-  } else emm_append_fp8_kernel<DT, 1, 4><<<grid, kThreads, 0, s>>>(p);
-  if (src_dtype == EMM_DTYPE_BF16) { EMM_FP8_LAUNCH(EMM_DTYPE_BF16) } else { EMM_FP8_LAUNCH(EMM_DTYPE_F16) }
+  const int fast_div = (move_variant() & 0x1000000) ? 0 : 1;
+#define EMM_FP8_LAUNCH(DT, VEC, SAT) \
+  launch_append_fp8<DT, VEC, SAT>(tables, t, slot_mapping, k_scales, v_scales, num_tokens, row_elems, ks, vs, num_slots, fast_div, num_layers, s)
+  if (dt == EMM_DTYPE_BF16) {
+    if (width == 8) { if (sat) EMM_FP8_LAUNCH(EMM_DTYPE_BF16, 8, true); else EMM_FP8_LAUNCH(EMM_DTYPE_BF16, 8, false); }
+    else { if (sat) EMM_FP8_LAUNCH(EMM_DTYPE_BF16, 1, true); else EMM_FP8_LAUNCH(EMM_DTYPE_BF16, 1, false); }
+  } else {
+    if (width == 8) { if (sat) EMM_FP8_LAUNCH(EMM_DTYPE_F16, 8, true); else EMM_FP8_LAUNCH(EMM_DTYPE_F16, 8, false); }
+    else { if (sat) EMM_FP8_LAUNCH(EMM_DTYPE_F16, 1, true); else EMM_FP8_LAUNCH(EMM_DTYPE_F16, 1, false); }
+  }
 #undef EMM_FP8_LAUNCH
   return check_launch(what);
 }
@@ -1069,7 +1119,7 @@ constexpr int kPagedSeg = 256;   // row elements per tile
 // token (every such store is a partial write of a 32-byte sector, which is what the layout costs
 // for tokens that do not fill a block; the lane order makes no measurable difference).
 // grid: x = token tiles, y = 2 * row segments (bit 0: K | V), z = layers.
-template <int CE, int SRC_DTYPE>
+template <int CE, int SRC_DTYPE, bool SAT>
 __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(const PagedParams p) {
   constexpr int X = 16 / CE;               // elements per 16-byte piece of the cache
   constexpr int ROW = kPagedSeg * CE + 16; // LDS row stride in bytes
@@ -1146,7 +1196,7 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(const PagedP
       if constexpr (CE == 2)
         *reinterpret_cast<u32x4 *>(tile + r * ROW + c * 16) = v;
       else
-        *reinterpret_cast<u32x2 *>(tile + r * ROW + c * 8) = quant8<SRC_DTYPE>(v, div);
+        *reinterpret_cast<u32x2 *>(tile + r * ROW + c * 8) = quant8<SRC_DTYPE, SAT>(v, div);
     }
   } else {
     for (int q = tid; q < count * seg_elems; q += kThreads) {
@@ -1155,8 +1205,7 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(const PagedP
       if constexpr (CE == 2)
         *reinterpret_cast<uint16_t *>(tile + r * ROW + c * 2) = h;
       else
-        *reinterpret_cast<uint8_t *>(tile + r * ROW + c) =
-            (uint8_t)f32_to_e4m3fn(half_bits_to_f32<SRC_DTYPE>(h) / scale);
+        *reinterpret_cast<uint8_t *>(tile + r * ROW + c) = quant1<SRC_DTYPE, SAT>(h, scale);
     }
   }
   __syncthreads();
@@ -1248,6 +1297,8 @@ int append_paged(const void *const *k, const void *const *v, void *const *kc, vo
   if (cache_elem_bytes != 1 && cache_elem_bytes != 2)
     return fail(EMM_EINVAL, "%s: cache_elem_bytes=%d, expected 2 (16-bit cache) or 1 (fp8 cache)", what,
                 cache_elem_bytes);
+  const bool sat = (src_dtype & EMM_FP8_SATURATE) != 0;
+  src_dtype &= ~EMM_FP8_SATURATE;
   if (src_dtype != EMM_DTYPE_BF16 && src_dtype != EMM_DTYPE_F16)
     return fail(EMM_EINVAL, "%s: unknown src_dtype %d", what, src_dtype);
   const int x = 16 / cache_elem_bytes;
@@ -1287,11 +1338,15 @@ int append_paged(const void *const *k, const void *const *v, void *const *kc, vo
   p.block_size = block_size;
   const dim3 grid((uint32_t)tiles, (uint32_t)(segs * 2), (uint32_t)num_layers);
   if (cache_elem_bytes == 2)
-    emm_append_paged_kernel<2, EMM_DTYPE_BF16><<<grid, kThreads, 0, s>>>(p);
+    emm_append_paged_kernel<2, EMM_DTYPE_BF16, false><<<grid, kThreads, 0, s>>>(p);
+  else if (src_dtype == EMM_DTYPE_BF16 && !sat)
+    emm_append_paged_kernel<1, EMM_DTYPE_BF16, false><<<grid, kThreads, 0, s>>>(p);
   else if (src_dtype == EMM_DTYPE_BF16)
-    emm_append_paged_kernel<1, EMM_DTYPE_BF16><<<grid, kThreads, 0, s>>>(p);
+    emm_append_paged_kernel<1, EMM_DTYPE_BF16, true><<<grid, kThreads, 0, s>>>(p);
+  else if (!sat)
+    emm_append_paged_kernel<1, EMM_DTYPE_F16, false><<<grid, kThreads, 0, s>>>(p);
   else
-    emm_append_paged_kernel<1, EMM_DTYPE_F16><<<grid, kThreads, 0, s>>>(p);
+    emm_append_paged_kernel<1, EMM_DTYPE_F16, true><<<grid, kThreads, 0, s>>>(p);
   return check_launch(what);
 }
 
@@ -1343,13 +1398,6 @@ extern "C" {
 const char *emm_last_error(void) { return g_last_error; }
 int emm_abi_version(void) { return EMM_KV_ABI_VERSION; }
 
-int emm_set_move_variant(int variant) {
-  const int old = g_move_variant | (g_append_rows << 12);
-  g_move_variant = variant & 0x10f0fff;
-  g_append_rows = (variant >> 12) & 0xf; // rows per wave of the append kernels
-  return old;
-}
-
 int emm_kv_pack(const void *const *layer_ptrs, int num_layers, int num_kv,
                 int64_t num_blocks, int64_t chunk_bytes, const int64_t *block_idx,
                 int64_t n, void *packed, emm_stream_t stream) {
@@ -1357,9 +1405,8 @@ int emm_kv_pack(const void *const *layer_ptrs, int num_layers, int num_kv,
   if (rc != EMM_OK) return rc;
   if (n == 0 || num_layers == 0 || num_kv == 0 || chunk_bytes == 0) return EMM_OK;
   if (!block_idx || !packed) return fail(EMM_EINVAL, "emm_kv_pack: null block_idx / packed");
-  return move_planes<true, false>(layer_ptrs, num_blocks, nullptr, 0, num_layers, num_kv, chunk_bytes,
-                                  block_idx, nullptr, 1, n, nullptr, packed, as_stream(stream),
-                                  "emm_kv_pack");
+  return move_planes<kPack>(layer_ptrs, num_blocks, nullptr, 0, num_layers, num_kv, chunk_bytes,
+                            block_idx, nullptr, false, n, packed, as_stream(stream), "emm_kv_pack");
 }
 
 int emm_kv_unpack(void *const *layer_ptrs, int num_layers, int num_kv,
@@ -1370,9 +1417,8 @@ int emm_kv_unpack(void *const *layer_ptrs, int num_layers, int num_kv,
   if (rc != EMM_OK) return rc;
   if (n == 0 || num_layers == 0 || num_kv == 0 || chunk_bytes == 0) return EMM_OK;
   if (!block_idx || !packed) return fail(EMM_EINVAL, "emm_kv_unpack: null block_idx / packed");
-  return move_planes<false, true>(nullptr, 0, layer_ptrs, num_blocks, num_layers, num_kv, chunk_bytes,
-                                  nullptr, block_idx, 1, n, packed, nullptr, as_stream(stream),
-                                  "emm_kv_unpack");
+  return move_planes<kUnpack>(nullptr, 0, layer_ptrs, num_blocks, num_layers, num_kv, chunk_bytes,
+                              nullptr, block_idx, false, n, packed, as_stream(stream), "emm_kv_unpack");
 }
 
 int emm_copy_blocks(void *const *layer_ptrs, int num_layers, int num_kv,
@@ -1383,9 +1429,9 @@ int emm_copy_blocks(void *const *layer_ptrs, int num_layers, int num_kv,
   if (rc != EMM_OK) return rc;
   if (num_pairs == 0 || num_layers == 0 || num_kv == 0 || chunk_bytes == 0) return EMM_OK;
   if (!block_mapping) return fail(EMM_EINVAL, "emm_copy_blocks: null block_mapping");
-  return move_planes<true, true>((const void *const *)layer_ptrs, num_blocks, layer_ptrs, num_blocks,
-                                 num_layers, num_kv, chunk_bytes, block_mapping, block_mapping + 1, 2,
-                                 num_pairs, nullptr, nullptr, as_stream(stream), "emm_copy_blocks");
+  return move_planes<kPoolToPool>((const void *const *)layer_ptrs, num_blocks, layer_ptrs, num_blocks,
+                                  num_layers, num_kv, chunk_bytes, block_mapping, nullptr, true,
+                                  num_pairs, nullptr, as_stream(stream), "emm_copy_blocks");
 }
 
 int emm_kv_migrate(const void *const *src_layer_ptrs, int64_t src_num_blocks,
@@ -1400,17 +1446,32 @@ int emm_kv_migrate(const void *const *src_layer_ptrs, int64_t src_num_blocks,
   if (rc != EMM_OK) return rc;
   if (n == 0 || num_layers == 0 || num_kv == 0 || chunk_bytes == 0) return EMM_OK;
   if (!src_idx || !dst_idx) return fail(EMM_EINVAL, "emm_kv_migrate: null index array");
-  return move_planes<true, true>(src_layer_ptrs, src_num_blocks, dst_layer_ptrs, dst_num_blocks,
-                                 num_layers, num_kv, chunk_bytes, src_idx, dst_idx, 1, n, nullptr,
-                                 nullptr, as_stream(stream), "emm_kv_migrate");
+  return move_planes<kPoolToPool>(src_layer_ptrs, src_num_blocks, dst_layer_ptrs, dst_num_blocks,
+                                  num_layers, num_kv, chunk_bytes, src_idx, dst_idx, false, n, nullptr,
+                                  as_stream(stream), "emm_kv_migrate");
 }
 
 int emm_stream_copy(const void *src, void *dst, int64_t nbytes, emm_stream_t stream) {
   if (nbytes < 0) return fail(EMM_EINVAL, "emm_stream_copy: negative size");
   if (nbytes == 0) return EMM_OK;
   if (!src || !dst) return fail(EMM_EINVAL, "emm_stream_copy: null pointer");
-  return move_planes<false, false>(nullptr, 0, nullptr, 0, 1, 1, nbytes, nullptr, nullptr, 1, 1, src,
-                                   dst, as_stream(stream), "emm_stream_copy");
+  int vec = common_align(common_align(16, src), dst);
+  while (vec > 1 && nbytes % vec) vec >>= 1;
+  if (vec == 8) vec = 4;
+  const int64_t tile = (int64_t)(vec == 16 ? 1 : 4) * kThreads * vec;
+  const int64_t tiles = (nbytes + tile - 1) / tile;
+  if (tiles > 0x7fffffffLL) return fail(EMM_EINVAL, "emm_stream_copy: %lld bytes need too many tiles", (long long)nbytes);
+  const dim3 grid((uint32_t)tiles);
+  hipStream_t s = as_stream(stream);
+  const char *a = (const char *)src;
+  char *b = (char *)dst;
+  switch (vec) {
+  case 16: emm_stream_copy_kernel<u32x4, 1, 1><<<grid, kThreads, 0, s>>>(a, b, nbytes); break;
+  case 4: emm_stream_copy_kernel<uint32_t, 4, 0><<<grid, kThreads, 0, s>>>(a, b, nbytes); break;
+  case 2: emm_stream_copy_kernel<uint16_t, 4, 0><<<grid, kThreads, 0, s>>>(a, b, nbytes); break;
+  default: emm_stream_copy_kernel<uint8_t, 4, 0><<<grid, kThreads, 0, s>>>(a, b, nbytes); break;
+  }
+  return check_launch("emm_stream_copy");
 }
 
 int emm_kv_unpack_dequant_fp8(void *const *layer_ptrs, int num_layers, int64_t num_blocks,
@@ -1471,7 +1532,7 @@ int emm_reshape_and_cache(const void *key, const void *value, void *key_cache,
                           int64_t num_tokens, int64_t row_bytes, int64_t key_stride_bytes,
                           int64_t value_stride_bytes, int64_t num_slots, emm_stream_t stream) {
   return append_copy(&key, &value, &key_cache, &value_cache, 1, slot_mapping, num_tokens,
-                     row_bytes, key_stride_bytes, value_stride_bytes, num_slots,
+                     row_bytes, key_stride_bytes, value_stride_bytes, num_slots, false,
                      as_stream(stream), "emm_reshape_and_cache");
 }
 
@@ -1483,7 +1544,7 @@ int emm_reshape_and_cache_layers(const void *const *key_ptrs, const void *const 
                                  int64_t num_slots, emm_stream_t stream) {
   return append_copy(key_ptrs, value_ptrs, key_cache_ptrs, value_cache_ptrs, num_layers,
                      slot_mapping, num_tokens, row_bytes, key_stride_bytes, value_stride_bytes,
-                     num_slots, as_stream(stream), "emm_reshape_and_cache_layers");
+                     num_slots, true, as_stream(stream), "emm_reshape_and_cache_layers");
 }
 
 int emm_reshape_and_cache_fp8(const void *key, const void *value, void *key_cache,
@@ -1494,7 +1555,7 @@ int emm_reshape_and_cache_fp8(const void *key, const void *value, void *key_cach
                               emm_stream_t stream) {
   return append_fp8(&key, &value, &key_cache, &value_cache, 1, slot_mapping, num_tokens,
                     row_elems, key_stride_elems, value_stride_elems, num_slots, k_scale, v_scale,
-                    src_dtype, as_stream(stream), "emm_reshape_and_cache_fp8");
+                    src_dtype, false, as_stream(stream), "emm_reshape_and_cache_fp8");
 }
 
 int emm_reshape_and_cache_fp8_layers(const void *const *key_ptrs, const void *const *value_ptrs,
@@ -1506,7 +1567,7 @@ int emm_reshape_and_cache_fp8_layers(const void *const *key_ptrs, const void *co
                                      const float *v_scales, int src_dtype, emm_stream_t stream) {
   return append_fp8(key_ptrs, value_ptrs, key_cache_ptrs, value_cache_ptrs, num_layers,
                     slot_mapping, num_tokens, row_elems, key_stride_elems, value_stride_elems,
-                    num_slots, k_scales, v_scales, src_dtype, as_stream(stream),
+                    num_slots, k_scales, v_scales, src_dtype, true, as_stream(stream),
                     "emm_reshape_and_cache_fp8_layers");
 }
 
@@ -1598,3 +1659,143 @@ int emm_concat_rows(const void *const *srcs, const int64_t *nbytes, int n, void 
 }
 
 } // extern "C"
+
+// ============================================================================
+// Benchmark / test hooks — compiled only with -DEMM_BENCH_HOOKS into
+// libemm_kv_hooks.so, never into the product library (csrc/emm_kv_hooks.h)
+// ============================================================================
+#ifdef EMM_BENCH_HOOKS
+#include "emm_kv_hooks.h"
+
+namespace {
+
+// Memory-system yardsticks with the geometry of pack / unpack: grid (tiles per chunk, n, planes),
+// one 16-byte vector per lane. READ kinds fold what they load into a value that is (practically)
+// never equal to the magic word, so the loads cannot be dropped and nothing is written.
+template <int KIND>
+__global__ __launch_bounds__(kThreads) void emm_probe_kernel(const int64_t *__restrict__ idx, char *lin,
+                                                            int64_t lin_plane_stride, int64_t chunk, uint32_t nb,
+                                                            uint32_t *sink, const PlaneTables<1> tables) {
+  const uint32_t pl = blockIdx.z, j = blockIdx.y;
+  const int64_t tile_off = (int64_t)blockIdx.x * (kThreads * 16) + threadIdx.x * 16;
+  if (tile_off >= chunk) return;
+  char *p;
+  if constexpr (KIND == EMM_PROBE_GATHER_READ || KIND == EMM_PROBE_SCATTER_WRITE) {
+    int64_t b = idx[j];
+    char *plane = tables.t[0].base[pl];
+    asm volatile("" : "+s"(b), "+s"(plane) : : "memory");
+    if ((uint64_t)b >= (uint64_t)nb) return;
+    p = plane + b * chunk + tile_off;
+  } else {
+    p = lin + (int64_t)pl * lin_plane_stride + (int64_t)j * chunk + tile_off;
+  }
+  if constexpr (KIND == EMM_PROBE_SEQ_READ || KIND == EMM_PROBE_GATHER_READ) {
+    const u32x4 v = ld_stream<u32x4, 1>(p);
+    if ((v[0] ^ v[1] ^ v[2] ^ v[3]) == 0x9e3779b9u && sink) sink[threadIdx.x] = v[0];
+  } else {
+    st_stream<u32x4, 1>(p, u32x4{j, pl, 2u, 3u});
+  }
+}
+
+// The fast quotient against the division for one exponent pair and a range of scale significands:
+// thread = one scale significand, loop over all 2^10 x significands (the 11 significant bits of an
+// f16; bf16 values are the subset with 3 more trailing zeros) and both signs.
+// counters[0] raw fp32 quotients that differ from RN(x / s) (counted where the division's result is
+// a normal number), [1] differing e4m3fn bytes (torch mode), [2] differing bytes (saturating mode),
+// [3] pairs checked, [4] (x bits << 32 | s bits) of one differing pair.
+__global__ __launch_bounds__(kThreads) void emm_quotient_sweep_kernel(int x_exp, int s_exp, uint32_t s_begin,
+                                                                      uint32_t s_end,
+                                                                      unsigned long long *counters) {
+  const uint32_t ms = s_begin + blockIdx.x * kThreads + threadIdx.x;
+  if (ms >= s_end) return;
+  const uint32_t sbits = ((uint32_t)(s_exp + 127) << 23) | ms;
+  const float s = __uint_as_float(sbits);
+  const Divisor d = make_divisor(s, true);
+  unsigned long long bad_raw = 0, bad_byte = 0, bad_sat = 0, bad_pair = 0;
+  for (uint32_t mx = 0; mx < 2048; ++mx) {
+    const uint32_t xbits = ((mx & 1024u) << 21) | ((uint32_t)(x_exp + 127) << 23) | ((mx & 1023u) << 13);
+    const float x = __uint_as_float(xbits);
+    const float ref = x / s;
+    const float fast = d.exact_fast ? divide_fast_raw(x, d) : ref;
+    const uint32_t rb = __float_as_uint(ref), fb = __float_as_uint(fast);
+    const bool normal = (rb & 0x7f800000u) != 0 && (rb & 0x7f800000u) != 0x7f800000u;
+    if (normal && rb != fb) {
+      ++bad_raw;
+      bad_pair = ((unsigned long long)xbits << 32) | sbits;
+    }
+    const float f0 = d.exact_fast ? divide_fast<false>(x, d) : divide_ieee<false>(x, s);
+    const float f1 = d.exact_fast ? divide_fast<true>(x, d) : divide_ieee<true>(x, s);
+    const float r0 = divide_ieee<false>(x, s), r1 = divide_ieee<true>(x, s);
+    const int b0 = __builtin_amdgcn_cvt_pk_fp8_f32(f0, f0, 0, false) & 0xff;
+    const int c0 = __builtin_amdgcn_cvt_pk_fp8_f32(r0, r0, 0, false) & 0xff;
+    const int b1 = __builtin_amdgcn_cvt_pk_fp8_f32(f1, f1, 0, false) & 0xff;
+    const int c1 = __builtin_amdgcn_cvt_pk_fp8_f32(r1, r1, 0, false) & 0xff;
+    if (b0 != c0) {
+      ++bad_byte;
+      bad_pair = ((unsigned long long)xbits << 32) | sbits;
+    }
+    if (b1 != c1) ++bad_sat;
+  }
+  if (bad_raw) atomicAdd(&counters[0], bad_raw);
+  if (bad_byte) atomicAdd(&counters[1], bad_byte);
+  if (bad_sat) atomicAdd(&counters[2], bad_sat);
+  atomicAdd(&counters[3], 2048ull);
+  if (bad_pair) atomicMax(&counters[4], bad_pair);
+}
+
+} // namespace
+
+extern "C" {
+
+int emm_hook_set_move_variant(int variant) {
+  const int old = g_move_variant;
+  g_move_variant = variant & 0x10fff00;
+  return old;
+}
+
+int emm_hook_probe(int kind, void *const *layer_ptrs, int num_layers, int num_kv, int64_t num_blocks,
+                   int64_t chunk_bytes, const int64_t *block_idx, int64_t n, void *linear, uint32_t *sink,
+                   emm_stream_t stream) {
+  const char *what = "emm_hook_probe";
+  const bool pool = kind == EMM_PROBE_GATHER_READ || kind == EMM_PROBE_SCATTER_WRITE;
+  if (kind < 0 || kind > 3) return fail(EMM_EINVAL, "%s: unknown kind %d", what, kind);
+  if (num_layers <= 0 || num_layers > EMM_MAX_LAYERS || num_kv <= 0 || n <= 0 || n > kMaxGridY || chunk_bytes <= 0 ||
+      chunk_bytes % 16)
+    return fail(EMM_EINVAL, "%s: bad geometry", what);
+  if (pool && (!layer_ptrs || !block_idx || num_blocks <= 0 || num_blocks > 0x7fffffffLL))
+    return fail(EMM_EINVAL, "%s: pool kinds need layer_ptrs, block_idx and num_blocks", what);
+  if (!pool && (!linear || !aligned(linear, 16))) return fail(EMM_EINVAL, "%s: linear kinds need a 16-byte aligned buffer", what);
+  PlaneTables<1> t;
+  const int planes = num_layers * num_kv;
+  if (pool)
+    for (int i = 0; i < planes; ++i) {
+      if (!layer_ptrs[i / num_kv] || !aligned(layer_ptrs[i / num_kv], 16)) return fail(EMM_EINVAL, "%s: bad layer pointer", what);
+      t.t[0].base[i] = (char *)layer_ptrs[i / num_kv] + (int64_t)(i % num_kv) * num_blocks * chunk_bytes;
+    }
+  const dim3 grid((uint32_t)((chunk_bytes + kThreads * 16 - 1) / (kThreads * 16)), (uint32_t)n, (uint32_t)planes);
+  hipStream_t s = as_stream(stream);
+  char *lin = (char *)linear;
+  const int64_t stride = n * chunk_bytes;
+  switch (kind) {
+  case EMM_PROBE_SEQ_READ: emm_probe_kernel<EMM_PROBE_SEQ_READ><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
+  case EMM_PROBE_SEQ_WRITE: emm_probe_kernel<EMM_PROBE_SEQ_WRITE><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
+  case EMM_PROBE_GATHER_READ: emm_probe_kernel<EMM_PROBE_GATHER_READ><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
+  default: emm_probe_kernel<EMM_PROBE_SCATTER_WRITE><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
+  }
+  return check_launch(what);
+}
+
+int emm_hook_fp8_quotient_sweep(int x_exp, int s_exp, uint32_t s_begin, uint32_t s_end, uint64_t *counters,
+                                emm_stream_t stream) {
+  const char *what = "emm_hook_fp8_quotient_sweep";
+  if (x_exp < -126 || x_exp > 127 || s_exp < -126 || s_exp > 127) return fail(EMM_EINVAL, "%s: exponent out of range", what);
+  if (s_begin >= s_end || s_end > (1u << 23)) return fail(EMM_EINVAL, "%s: bad significand range", what);
+  if (!counters) return fail(EMM_EINVAL, "%s: null counters", what);
+  const uint32_t blocks = (s_end - s_begin + kThreads - 1) / kThreads;
+  emm_quotient_sweep_kernel<<<blocks, kThreads, 0, as_stream(stream)>>>(x_exp, s_exp, s_begin, s_end,
+                                                                        (unsigned long long *)counters);
+  return check_launch(what);
+}
+
+} // extern "C"
+#endif // EMM_BENCH_HOOKS

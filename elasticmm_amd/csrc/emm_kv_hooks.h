@@ -1,0 +1,51 @@
+/*
+ * emm_kv_hooks.h — entry points that exist only in libemm_kv_hooks.so, the build of
+ * emm_kv.hip with -DEMM_BENCH_HOOKS used by bench.py and the GPU tests. The product
+ * library libemm_kv.so (include/emm_kv.h) exports none of them and carries no
+ * run-time switch. The hooks library also exports the whole product ABI, so a
+ * benchmark can route its calls through it and select launch variants.
+ */
+#ifndef EMM_KV_HOOKS_H
+#define EMM_KV_HOOKS_H
+
+#include <stdint.h>
+
+#include "emm_kv.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Launch variants of the hooks library's own kernels: 0 = the product's defaults.
+ * bits 8-11: 1 = non-temporal stores in the 16-byte block moves (default: sc0 sc1);
+ * bits 12-15: shape of the 16-byte copy append (token rows per wave, waves per workgroup):
+ *   0 = (2, 1) default, 1 = (1, 4), 2 = (2, 4), 3 = (4, 1), 4 = (1, 1);
+ * bits 16-19: log2 of the blocks per plane visit of pack / unpack (15 = plain order);
+ * bit 24: fp8 append with the IEEE division instead of the reciprocal form.
+ * Process-wide, not thread-safe. Returns the previous value. */
+int emm_hook_set_move_variant(int variant);
+
+/* Memory-system yardsticks with the grid of pack / unpack (one 4 KiB tile per workgroup):
+ * sequential kinds touch `linear` [num_layers * num_kv, n, chunk]; pool kinds touch the
+ * n blocks block_idx[] of every plane of the pool. Reads write nothing (sink may be null). */
+#define EMM_PROBE_SEQ_READ 0
+#define EMM_PROBE_SEQ_WRITE 1
+#define EMM_PROBE_GATHER_READ 2
+#define EMM_PROBE_SCATTER_WRITE 3
+int emm_hook_probe(int kind, void *const *layer_ptrs, int num_layers, int num_kv, int64_t num_blocks,
+                   int64_t chunk_bytes, const int64_t *block_idx, int64_t n, void *linear, uint32_t *sink,
+                   emm_stream_t stream);
+
+/* Exhaustive check of the fp8 append's reciprocal-form quotient: for x = +-1.m * 2^x_exp over all
+ * 2^10 ten-bit m and scale = 1.f * 2^s_exp for f in [s_begin, s_end) (23-bit significand fields),
+ * compare with the IEEE division. counters (DEVICE, 5 x uint64, zeroed by the caller):
+ * [0] differing fp32 quotients (where the division gives a normal number), [1] differing e4m3fn
+ * bytes in torch mode, [2] in saturating mode, [3] pairs checked, [4] one differing pair
+ * (x bits << 32 | scale bits). */
+int emm_hook_fp8_quotient_sweep(int x_exp, int s_exp, uint32_t s_begin, uint32_t s_end, uint64_t *counters,
+                                emm_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EMM_KV_HOOKS_H */

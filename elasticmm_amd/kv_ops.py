@@ -593,12 +593,16 @@ def concat_rows(tensors: Sequence[torch.Tensor], out: Optional[torch.Tensor] = N
     for d in tail:
         row_bytes *= int(d)
     # one pass per tensor (the host time of this loop is what a short gather waits for)
-    ptrs, sizes, rows = [], [], 0
+    # `alive` holds the contiguous copies made here until the launch has been queued: a copy that
+    # is dropped earlier goes back to the caching allocator, and the next copy (or `out`) may be
+    # handed the same memory before the kernel has read it.
+    ptrs, sizes, rows, alive = [], [], 0, []
     for t in tensors:
         if t.shape[1:] != tail or t.dtype != dtype or t.device != device:
             raise ValueError("concat_rows: tensors differ in trailing shape / dtype / device")
         if not t.is_contiguous():
             t = t.contiguous()
+            alive.append(t)
         r = t.shape[0]
         rows += r
         ptrs.append(t.data_ptr())
@@ -609,6 +613,7 @@ def concat_rows(tensors: Sequence[torch.Tensor], out: Optional[torch.Tensor] = N
     elif tuple(out.shape) != shape or out.dtype != dtype or out.device != device or not out.is_contiguous():
         raise ValueError("concat_rows: `out` has the wrong shape / dtype / device or is not contiguous")
     _launch_concat(lib, ptrs, sizes, out, _stream_ptr(device))
+    del alive  # queued on the stream the copies were made on: the allocator may reuse them now
     return out
 
 

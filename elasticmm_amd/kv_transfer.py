@@ -11,9 +11,18 @@ What is different: workers are ``KVWorker`` objects in this process, not Ray act
 are plain method calls. The reference's batching path is disabled in the product and its enqueue
 code refers to undefined names (:439); here the queue is keyed by (src_rank, dst_rank) and a flush
 moves the merged tables with one pack launch and one unpack launch.
+
+The coroutines (``transfer_kv_cache``, ``transfer_vision_embeddings``, ``migrate_requests``) hand
+the blocking work — kernel launches followed by the device synchronisation the workers perform, as
+the reference's do (worker.py:684, :724) — to one worker thread of the manager and await it, so the
+event loop that calls them (the reference's is stage_engine.py:1506) keeps serving other coroutines
+while a transfer runs. Transfers of one manager run one after the other in that thread. The
+``*_sync`` forms do the same work on the calling thread.
 """
 from __future__ import annotations
 
+import asyncio
+import concurrent.futures
 import time
 from enum import Enum
 from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
@@ -46,6 +55,21 @@ class KVTransferManager:
         self.total_transfer_time = 0.0
         self.total_bytes_transferred = 0
         self.first_transfer_done = False
+        self._executor: Optional[concurrent.futures.ThreadPoolExecutor] = None
+
+    def _transfer_thread(self) -> concurrent.futures.ThreadPoolExecutor:
+        if self._executor is None:
+            self._executor = concurrent.futures.ThreadPoolExecutor(max_workers=1, thread_name_prefix="kv-transfer")
+        return self._executor
+
+    async def _off_loop(self, fn, *args):
+        """Run blocking transfer work on the manager's thread and await its result."""
+        return await asyncio.get_running_loop().run_in_executor(self._transfer_thread(), fn, *args)
+
+    def close(self) -> None:
+        if self._executor is not None:
+            self._executor.shutdown(wait=True)
+            self._executor = None
 
     # ----- registry (kv_transfer.py:113-168) ---------------------------------
     def register_workers(self, stage: str, workers: Sequence[Any], global_ranks: Sequence[int]) -> None:
@@ -70,7 +94,38 @@ class KVTransferManager:
     # ----- transfer (kv_transfer.py:224-262) ----------------------------------
     async def transfer_kv_cache(self, request_id: str, src_rank: int, dst_rank: int, src_blocks: List[int],
                                 dst_blocks: List[int]) -> bool:
-        return self.transfer_kv_cache_sync(request_id, src_rank, dst_rank, src_blocks, dst_blocks)
+        return await self._off_loop(self.transfer_kv_cache_sync, request_id, src_rank, dst_rank, src_blocks,
+                                    dst_blocks)
+
+    # ----- vision embeddings (kv_transfer.py:264-301, 've' branch of :724-728) ----
+    async def transfer_vision_embeddings(self, request_id: str, src_rank: int, src_blocks: List[int],
+                                         dst_rank: int, dst_blocks: List[int]) -> bool:
+        return await self._off_loop(self.transfer_vision_embeddings_sync, request_id, src_rank, src_blocks,
+                                    dst_rank, dst_blocks)
+
+    def transfer_vision_embeddings_sync(self, request_id: str, src_rank: int, src_blocks: List[int],
+                                        dst_rank: int, dst_blocks: List[int]) -> bool:
+        """Move a request's vision embeddings from the source worker's cache to the destination's.
+
+        The reference routes every method but CUDA_IPC (a placeholder there) to the 've' branch of
+        ``_transfer_via_p2p_copy``: ``extract_vision_blocks(request_id)`` on the source,
+        ``write_vision_blocks(request_id, data)`` on the destination; the block lists are carried for
+        logging only. Its signature still names (stage, worker_id) pairs although its body hands them
+        on as ranks (and two arguments too many); here the arguments are the ranks the registry is
+        keyed by."""
+        src_worker, dst_worker = self._workers(src_rank, dst_rank)
+        if src_worker is None:
+            return False
+        try:
+            start_time = time.perf_counter()
+            ve_data = src_worker.extract_vision_blocks(request_id)
+            dst_worker.write_vision_blocks(request_id, ve_data)
+            _ = time.perf_counter() - start_time
+            self.transfer_count += 1  # counted, but not reported to the metrics callback (kv only, :743)
+            return True
+        except Exception as e:
+            print(f"[KVTransferManager] P2P copy failed: {e}")
+            return False
 
     def transfer_kv_cache_sync(self, request_id: str, src_rank: int, dst_rank: int, src_blocks: List[int],
                                dst_blocks: List[int]) -> bool:
@@ -165,7 +220,8 @@ class KVTransferManager:
     # ----- migration of whole requests (backend.py:674-737) -----------------------
     async def migrate_requests(self, request_ids: Sequence[str], src_rank: int, src_block_manager: Any,
                                dst_rank: int, dst_block_manager: Any) -> bool:
-        return self.migrate_requests_sync(request_ids, src_rank, src_block_manager, dst_rank, dst_block_manager)
+        return await self._off_loop(self.migrate_requests_sync, request_ids, src_rank, src_block_manager,
+                                    dst_rank, dst_block_manager)
 
     def migrate_requests_sync(self, request_ids: Sequence[str], src_rank: int, src_block_manager: Any,
                               dst_rank: int, dst_block_manager: Any) -> bool:
@@ -177,6 +233,10 @@ class KVTransferManager:
         moved: List[str] = []
 
         def roll_back() -> None:
+            # with batching the moved requests may still sit in the queue: take them out before
+            # their destination blocks go back to the free list, or a later flush would scatter
+            # into blocks that belong to nobody (or to another request by then)
+            self._purge_queued((src_rank, dst_rank), moved)
             for rid in moved:
                 dst_block_manager.free_blocks(rid)
 
@@ -219,6 +279,17 @@ class KVTransferManager:
             return self.flush_transfer_batch(src_rank, dst_rank)
         return True  # queued, flushed later
 
+    def _purge_queued(self, key: Tuple[int, int], request_ids: Sequence[str]) -> int:
+        """Remove the queued (not yet flushed) transfers of `request_ids` from the batch queue."""
+        queue = self._transfer_queue.get(key)
+        if not queue or not request_ids:
+            return 0
+        gone = set(request_ids)
+        kept = [t for t in queue if t[0] not in gone]
+        removed = len(queue) - len(kept)
+        self._transfer_queue[key] = kept
+        return removed
+
     def flush_transfer_batch(self, src_rank: int, dst_rank: int) -> bool:
         """Merge the queued requests' tables and move them with one send / one receive."""
         key = (src_rank, dst_rank)
@@ -241,6 +312,10 @@ class KVTransferManager:
                 return False
             recv_result = dst_worker.p2p_recv_kv(src_rank, all_dst_blocks)
             if "error" in recv_result:
+                # the send went through: nothing of it may stay on the link for the next transfer
+                link = getattr(src_worker, "link", None)
+                if link is not None:
+                    link.drop_pending(src_rank, dst_rank)
                 return False
             elapsed = time.perf_counter() - start_time
             nbytes = recv_result.get("bytes", 0)

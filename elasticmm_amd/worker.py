@@ -42,25 +42,68 @@ _DTYPES = {
 class LoopbackLink:
     """Same-device stand-in for the global NCCL group: per (src, dst, tag) FIFOs of
     device tensors. ``send`` enqueues a tensor, ``recv`` dequeues it; both sides run
-    on the same HIP stream order, so no extra synchronisation is needed."""
+    on the same HIP stream order, so no extra synchronisation is needed.
+
+    Every message may carry the id of the transfer it belongs to (one id for the L
+    per-layer messages of one send). A receiver that gives up in the middle of a
+    transfer (deadline, shape mismatch) discards the transfer's remaining messages by
+    that id, so that the next transfer between the same ranks does not start with
+    stale layers."""
 
     def __init__(self, world_size: int = 2):
         self.world_size = world_size
-        self._queues: Dict[Tuple[int, int, int], Deque[torch.Tensor]] = collections.defaultdict(collections.deque)
+        self._queues: Dict[Tuple[int, int, int], Deque[Tuple[Optional[int], torch.Tensor]]] = \
+            collections.defaultdict(collections.deque)
+        self._next_transfer_id = 0
 
-    def send(self, tensor: torch.Tensor, src: int, dst: int, tag: int = 0) -> None:
+    def new_transfer_id(self) -> int:
+        self._next_transfer_id += 1
+        return self._next_transfer_id
+
+    def send(self, tensor: torch.Tensor, src: int, dst: int, tag: int = 0, transfer_id: Optional[int] = None) -> None:
         if not (0 <= dst < self.world_size):
             raise ValueError(f"Invalid dst rank: {dst} (world_size={self.world_size})")
-        self._queues[(src, dst, tag)].append(tensor)
+        self._queues[(src, dst, tag)].append((transfer_id, tensor))
 
-    def recv(self, src: int, dst: int, tag: int = 0) -> torch.Tensor:
+    def recv_with_id(self, src: int, dst: int, tag: int = 0) -> Tuple[Optional[int], torch.Tensor]:
         q = self._queues[(src, dst, tag)]
         if not q:
             raise RuntimeError(f"no message pending from rank {src} to rank {dst} (tag {tag})")
         return q.popleft()
 
+    def recv(self, src: int, dst: int, tag: int = 0) -> torch.Tensor:
+        return self.recv_with_id(src, dst, tag)[1]
+
+    def head_id(self, src: int, dst: int, tag: int = 0) -> Optional[int]:
+        """Transfer id of the next message of this FIFO (None if it is empty or the message has none)."""
+        q = self._queues[(src, dst, tag)]
+        return q[0][0] if q else None
+
     def pending(self, src: int, dst: int, tag: int = 0) -> int:
         return len(self._queues[(src, dst, tag)])
+
+    def discard(self, src: int, dst: int, transfer_id: Optional[int]) -> int:
+        """Drop every queued message of transfer ``transfer_id`` from ``src`` to ``dst`` (all tags).
+        Returns the number of messages dropped."""
+        if transfer_id is None:
+            return 0
+        dropped = 0
+        for (s, d, _), q in self._queues.items():
+            if s == src and d == dst and q:
+                kept = [m for m in q if m[0] != transfer_id]
+                dropped += len(q) - len(kept)
+                q.clear()
+                q.extend(kept)
+        return dropped
+
+    def drop_pending(self, src: int, dst: int) -> int:
+        """Drop everything queued from ``src`` to ``dst`` (all tags, all transfers)."""
+        dropped = 0
+        for (s, d, _), q in self._queues.items():
+            if s == src and d == dst:
+                dropped += len(q)
+                q.clear()
+        return dropped
 
 
 def _hip_runtime():
@@ -244,10 +287,15 @@ class KVWorker:
         try:
             packed = kv_ops.kv_pack(self.pool, block_indices)
             total_bytes = 0
-            for l in range(self.pool.num_layers):
-                layer_data = packed[l]
-                self.link.send(layer_data, src=self.global_rank, dst=dst_rank)
-                total_bytes += layer_data.numel() * layer_data.element_size()
+            transfer_id = self.link.new_transfer_id()
+            try:
+                for l in range(self.pool.num_layers):
+                    layer_data = packed[l]
+                    self.link.send(layer_data, src=self.global_rank, dst=dst_rank, transfer_id=transfer_id)
+                    total_bytes += layer_data.numel() * layer_data.element_size()
+            except Exception:
+                self.link.discard(self.global_rank, dst_rank, transfer_id)  # no half-sent transfer stays queued
+                raise
             torch.cuda.synchronize(self.device)
             return {"bytes": total_bytes, "blocks": len(block_indices)}
         except Exception as e:  # transport failures are reported, not raised (worker.py:686-691)
@@ -262,13 +310,26 @@ class KVWorker:
         n = len(block_indices)
         layer_shape = (pool.num_kv, n) + pool.block_shape
         msgs: List[torch.Tensor] = []
-        for layer_idx in range(pool.num_layers):
-            if deadline is not None and time.time() - deadline[0] > deadline[1]:
-                return layer_idx
-            m = self.link.recv(src=src_rank, dst=self.global_rank, tag=layer_idx if tagged else 0)
-            if tuple(m.shape) != layer_shape:
-                raise RuntimeError(f"layer {layer_idx}: received {tuple(m.shape)}, expected {layer_shape}")
-            msgs.append(m)
+        # the transfer this call consumes: on any early exit its remaining per-layer messages are
+        # dropped from the link, so that the next receive does not scatter stale layers
+        transfer_id = self.link.head_id(src_rank, self.global_rank, 0)
+        complete = False
+        try:
+            for layer_idx in range(pool.num_layers):
+                if deadline is not None and time.time() - deadline[0] > deadline[1]:
+                    return layer_idx
+                tid, m = self.link.recv_with_id(src=src_rank, dst=self.global_rank, tag=layer_idx if tagged else 0)
+                if layer_idx == 0:
+                    transfer_id = tid
+                elif tid != transfer_id:
+                    raise RuntimeError(f"layer {layer_idx}: message of transfer {tid} inside transfer {transfer_id}")
+                if tuple(m.shape) != layer_shape:
+                    raise RuntimeError(f"layer {layer_idx}: received {tuple(m.shape)}, expected {layer_shape}")
+                msgs.append(m)
+            complete = True
+        finally:
+            if not complete:
+                self.link.discard(src_rank, self.global_rank, transfer_id)
         total_bytes = sum(m.numel() * m.element_size() for m in msgs)
         step = self._layer_bytes(n)
         whole = msgs[0]._base if msgs else None
@@ -357,9 +418,11 @@ class KVWorker:
         n = int(block_idx.numel())
         packed = kv_ops.kv_pack(self.pool, block_idx)
         total_bytes = 0
+        transfer_id = self.link.new_transfer_id()
         for layer_idx in range(self.pool.num_layers):
             layer_data = packed[layer_idx]
-            self.link.send(layer_data, src=self.global_rank, dst=requester_rank, tag=layer_idx)
+            self.link.send(layer_data, src=self.global_rank, dst=requester_rank, tag=layer_idx,
+                           transfer_id=transfer_id)
             total_bytes += layer_data.numel() * layer_data.element_size()
         torch.cuda.synchronize(self.device)
         return {"bytes": total_bytes, "blocks": n}

@@ -27,7 +27,8 @@
  *     fixed-size request convention, elasticmm/engine/v0/worker.py:924-925); an
  *     index >= num_blocks is never dereferenced (skipped), the Python layer
  *     raises IndexError for it before launch when indices arrive as a list;
- *   - no allocation, no global mutable state; re-entrant from any host thread.
+ *   - no allocation, no global mutable state; re-entrant from any host thread
+ *     (the only per-thread state is the text behind emm_last_error()).
  */
 #ifndef EMM_KV_H
 #define EMM_KV_H
@@ -38,7 +39,7 @@
 extern "C" {
 #endif
 
-#define EMM_KV_ABI_VERSION 1
+#define EMM_KV_ABI_VERSION 2
 #define EMM_MAX_LAYERS 96   /* layer pointers carried in one kernel argument block */
 #define EMM_MAX_SEGMENTS 128 /* ragged segments carried by one emm_concat_rows launch */
 
@@ -50,6 +51,9 @@ extern "C" {
 /* element types of the 16-bit side of the fp8 kernels */
 #define EMM_DTYPE_BF16 0
 #define EMM_DTYPE_F16 1
+/* or-ed into the src_dtype of the fp8 appends: clamp the quotient to +-448 before the
+ * cast (see emm_reshape_and_cache_fp8) */
+#define EMM_FP8_SATURATE 0x100
 
 typedef void *emm_stream_t; /* hipStream_t */
 
@@ -164,10 +168,17 @@ int emm_reshape_and_cache_layers(const void *const *key_ptrs,
 /*
  * fp8 append — as emm_reshape_and_cache with a 16-bit source (src_dtype) and an
  * fp8-e4m3fn cache: q = e4m3fn_rne(float(x) / scale) with a correctly rounded
- * fp32 division, round-to-nearest-even, ties at 464 -> 448 and at 2^-10 -> 0,
- * |x/scale| >= 465, inf and NaN -> sign|0x7F (no saturation) — the rule of
- * torch's .to(torch.float8_e4m3fn). k_scale / v_scale are DEVICE pointers to
- * one float each (per-layer per-tensor scale). Strides in elements.
+ * fp32 division, round-to-nearest-even, ties at 464 -> 448 and at 2^-10 -> 0.
+ * Overflow follows src_dtype:
+ *   EMM_DTYPE_BF16 / EMM_DTYPE_F16: |x/scale| >= 465, inf and NaN -> sign|0x7F (no
+ *     saturation) — the rule of torch's (x.float() / scale).to(torch.float8_e4m3fn);
+ *   the same or-ed with EMM_FP8_SATURATE: the quotient is clamped to [-448, 448]
+ *     first, so overflow and +-inf give sign|0x7E and only NaN gives sign|0x7F —
+ *     torch.clamp(x.float() / scale, -448, 448).to(torch.float8_e4m3fn), the
+ *     convention of vLLM's fp8 KV cache (the cache_dtype the reference leaves open
+ *     at elasticmm/engine/v0/worker.py:194). Never the default.
+ * scale must be finite and non-zero. k_scale / v_scale are DEVICE pointers to one
+ * float each (per-layer per-tensor scale). Strides in elements.
  */
 int emm_reshape_and_cache_fp8(const void *key, const void *value,
                               void *key_cache, void *value_cache,
@@ -283,14 +294,6 @@ int emm_concat_rows(const void *const *srcs, const int64_t *nbytes, int n,
  */
 int emm_stream_copy(const void *src, void *dst, int64_t nbytes,
                     emm_stream_t stream);
-
-/* Tuning hook for benchmarks: 0 = library default. Bits 0-3: vectors per lane of
- * the block-move kernels (1 or 4); bits 8-11: store policy + 1 (1: non-temporal,
- * 2: sc0 sc1); bits 12-15: token rows per wave of the append kernels (1, 2, 4);
- * bits 16-19: log2 of the blocks per plane visit of pack / unpack (15 = plain order);
- * bit 24: fp8 append with the IEEE division sequence instead of the reciprocal form.
- * Process-wide, not thread-safe. Returns the previous value. */
-int emm_set_move_variant(int variant);
 
 #ifdef __cplusplus
 }

@@ -662,6 +662,22 @@ def test_concat_rows_ragged():
         w.gather_vision_embeddings(["r0", "bad"])
 
 
+def test_concat_rows_non_contiguous_segments():
+    say("vision concat: several non-contiguous segments of equal size (their contiguous copies must stay alive)")
+    g = torch.Generator().manual_seed(15)
+    wide = [torch.randn((256, 2 * 3584), generator=g).to(torch.bfloat16) for _ in range(6)]
+    views = [w.to(DEV)[:, ::2] for w in wide]
+    assert not views[0].is_contiguous()
+    want = torch.cat([w[:, ::2] for w in wide], 0)
+    for _ in range(3):
+        got = kv_ops.concat_rows(views)
+        assert same_bits(got, want)
+        del got
+    mixed = [views[0], wide[1].to(DEV)[:, :3584].contiguous(), views[2], views[3]]
+    assert same_bits(kv_ops.concat_rows(mixed), torch.cat([wide[0][:, ::2], wide[1][:, :3584], wide[2][:, ::2],
+                                                            wide[3][:, ::2]], 0))
+
+
 # ------------------------------------------------------------------ worker protocol
 def make_pair(L=3, NB=32, bs=16, H=2, D=64, dtype=torch.bfloat16):
     link = LoopbackLink(world_size=2)
