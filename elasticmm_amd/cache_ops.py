@@ -16,6 +16,13 @@ import torch
 from . import kv_ops
 from .kv_ops import PoolView
 
+# kv_cache_dtype strings of the fp8 KV cache. "fp8" / "fp8_e4m3" is the cast torch performs,
+# (x.float() / scale).to(torch.float8_e4m3fn): what overflows becomes NaN (0x7F / 0xFF). The "_sat"
+# names clamp the quotient to [-448, 448] first, the convention of a cache written by vLLM's own fp8
+# kernels (the variants the reference leaves open at elasticmm/engine/v0/worker.py:194); it has to be
+# asked for by name.
+_FP8_MODES = {"fp8": False, "fp8_e4m3": False, "fp8_sat": True, "fp8_e4m3_sat": True}
+
 
 def reshape_and_cache_flash(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor,
                             value_cache: torch.Tensor, slot_mapping: torch.Tensor, kv_cache_dtype: str = "auto",
@@ -24,8 +31,9 @@ def reshape_and_cache_flash(key: torch.Tensor, value: torch.Tensor, key_cache: t
     ``[num_blocks, block_size, num_heads, head_size]`` (contiguous, or for "auto" a strided view with
     contiguous head rows such as a permuted head-major pool); ``slot_mapping`` int64
     ``[num_tokens]`` with -1 for padded tokens. ``kv_cache_dtype`` is "auto" (cache
-    dtype == key dtype, bit copy) or "fp8" / "fp8_e4m3" (cache is 1 byte wide and
-    is written as ``e4m3fn(float(x) / scale)``)."""
+    dtype == key dtype, bit copy), "fp8" / "fp8_e4m3" (cache is 1 byte wide and
+    is written as ``e4m3fn(float(x) / scale)``, torch's cast) or "fp8_sat" / "fp8_e4m3_sat" (the
+    same with the quotient clamped to [-448, 448] first)."""
     if kv_cache_dtype == "auto":
         if key_cache.element_size() != key.element_size():
             raise ValueError("kv_cache_dtype='auto' needs a cache of the key's element size")
@@ -33,10 +41,11 @@ def reshape_and_cache_flash(key: torch.Tensor, value: torch.Tensor, key_cache: t
             kv_ops.reshape_and_cache(key, value, key_cache, value_cache, slot_mapping)
         else:  # e.g. the head-major pool [NB, H, bs, D] passed as a permuted view
             kv_ops.reshape_and_cache_strided([key], [value], [key_cache], [value_cache], slot_mapping)
-    elif kv_cache_dtype in ("fp8", "fp8_e4m3"):
+    elif kv_cache_dtype in _FP8_MODES:
         if key_cache.element_size() != 1:
             raise ValueError("fp8 KV cache must be a 1-byte tensor (float8_e4m3fn or uint8)")
-        kv_ops.reshape_and_cache(key, value, key_cache, value_cache, slot_mapping, k_scale, v_scale)
+        kv_ops.reshape_and_cache(key, value, key_cache, value_cache, slot_mapping, k_scale, v_scale,
+                                 saturate=_FP8_MODES[kv_cache_dtype])
     else:
         raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
 
@@ -51,10 +60,11 @@ def reshape_and_cache(key: torch.Tensor, value: torch.Tensor, key_cache: torch.T
         if key_cache.element_size() != key.element_size():
             raise ValueError("kv_cache_dtype='auto' needs a cache of the key's element size")
         kv_ops.reshape_and_cache_paged(key, value, key_cache, value_cache, slot_mapping)
-    elif kv_cache_dtype in ("fp8", "fp8_e4m3"):
+    elif kv_cache_dtype in _FP8_MODES:
         if key_cache.element_size() != 1:
             raise ValueError("fp8 KV cache must be a 1-byte tensor (float8_e4m3fn or uint8)")
-        kv_ops.reshape_and_cache_paged(key, value, key_cache, value_cache, slot_mapping, k_scale, v_scale)
+        kv_ops.reshape_and_cache_paged(key, value, key_cache, value_cache, slot_mapping, k_scale, v_scale,
+                                       saturate=_FP8_MODES[kv_cache_dtype])
     else:
         raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
 
@@ -67,8 +77,9 @@ def reshape_and_cache_flash_layers(keys: Sequence[torch.Tensor], values: Sequenc
     value_caches = [c[1] for c in kv_caches]
     if kv_cache_dtype == "auto":
         kv_ops.reshape_and_cache_layers(keys, values, key_caches, value_caches, slot_mapping)
-    elif kv_cache_dtype in ("fp8", "fp8_e4m3"):
-        kv_ops.reshape_and_cache_layers(keys, values, key_caches, value_caches, slot_mapping, k_scales, v_scales)
+    elif kv_cache_dtype in _FP8_MODES:
+        kv_ops.reshape_and_cache_layers(keys, values, key_caches, value_caches, slot_mapping, k_scales, v_scales,
+                                        saturate=_FP8_MODES[kv_cache_dtype])
     else:
         raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
 
@@ -81,8 +92,9 @@ def layered_append(keys: Sequence[torch.Tensor], values: Sequence[torch.Tensor],
     value_caches = [c[1] for c in kv_caches]
     if kv_cache_dtype == "auto":
         return kv_ops.LayeredAppend(keys, values, key_caches, value_caches)
-    if kv_cache_dtype in ("fp8", "fp8_e4m3"):
-        return kv_ops.LayeredAppend(keys, values, key_caches, value_caches, k_scales, v_scales)
+    if kv_cache_dtype in _FP8_MODES:
+        return kv_ops.LayeredAppend(keys, values, key_caches, value_caches, k_scales, v_scales,
+                                    saturate=_FP8_MODES[kv_cache_dtype])
     raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
 
 
@@ -93,8 +105,9 @@ def paged_layered_append(keys: Sequence[torch.Tensor], values: Sequence[torch.Te
     ``[NB, H, D // x, bs, x]``, ``value_caches[l]`` ``[NB, H, D, bs]``; ``plan(slot_mapping)`` is one launch."""
     if kv_cache_dtype == "auto":
         return kv_ops.PagedLayeredAppend(keys, values, key_caches, value_caches)
-    if kv_cache_dtype in ("fp8", "fp8_e4m3"):
-        return kv_ops.PagedLayeredAppend(keys, values, key_caches, value_caches, k_scales, v_scales)
+    if kv_cache_dtype in _FP8_MODES:
+        return kv_ops.PagedLayeredAppend(keys, values, key_caches, value_caches, k_scales, v_scales,
+                                         saturate=_FP8_MODES[kv_cache_dtype])
     raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
 
 

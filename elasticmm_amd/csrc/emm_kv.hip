@@ -717,11 +717,19 @@ __global__ __launch_bounds__(WAVES * 64) void emm_append_kernel(
 #pragma unroll
   for (int r = 0; r < R; ++r) slot[r] = t0 + r < num_tokens ? slot_mapping[t0 + r] : -1;
   uint32_t off = lane * VB;
+  const uint32_t o = off < row_bytes ? off : 0; // lanes past the row re-read its start; only stores are predicated
   V a[R], b[R];
+  // Issue order (measured on a 28-layer chain of per-layer launches, 8448 tokens each; faster by 10 % than
+  // issuing all loads first): rows of tokens 1.. go out at once and are in flight while the slots
+  // arrive; token 0's rows are requested after the slot wait, and only if its slot is valid; then
+  // stores in token order. The wave's reads and writes then overlap those of its neighbours instead
+  // of the whole launch reading first and writing afterwards.
+  // A whole-step launch (TABLES) is long enough to reach that overlap by itself and measured 3 %
+  // faster with all rows requested before the slot wait.
+  constexpr int kFirstEarly = TABLES ? 0 : 1;
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
+  for (int r = kFirstEarly; r < R; ++r) {
     const uint32_t t = t0 + r < num_tokens ? t0 + r : num_tokens - 1; // tail: re-read the last row, dropped below
-    const uint32_t o = off < row_bytes ? off : 0;
     a[r] = ld_stream<V, POLICY>(key + (uint64_t)t * key_stride + o);
     b[r] = ld_stream<V, POLICY>(value + (uint64_t)t * value_stride + o);
   }
@@ -729,6 +737,12 @@ __global__ __launch_bounds__(WAVES * 64) void emm_append_kernel(
   for (int r = 0; r < R; ++r) {
     asm volatile("" : "+s"(slot[r]) : : "memory");
     if ((uint64_t)slot[r] >= (uint64_t)num_slots) slot[r] = -1; // padding (< 0) and out-of-range slots: skipped
+  }
+  if constexpr (kFirstEarly == 1) {
+    if (slot[0] >= 0) {
+      a[0] = ld_stream<V, POLICY>(key + (uint64_t)t0 * key_stride + o);
+      b[0] = ld_stream<V, POLICY>(value + (uint64_t)t0 * value_stride + o);
+    }
   }
   if (off < row_bytes) {
 #pragma unroll
@@ -882,14 +896,18 @@ int append_copy(const void *const *k, const void *const *v, void *const *kc, voi
   int vec = al;
   while (vec > 1 && (row_bytes % vec || ks % vec || vs % vec)) vec >>= 1;
   if (vec == 16) {
-    // one wave per two tokens in workgroups of one wave: the fastest start and drain of a per-layer
-    // launch; the other shapes exist for benchmark builds
-    switch ((move_variant() >> 12) & 0xf) {
+    // workgroups of one wave start and drain fastest. A per-layer launch is best with four token rows
+    // per wave (39.9 M tokens/s on the 28-layer chain of 8448-token launches; two rows 38.6, one 37.6),
+    // a whole-step launch with one (6.23 TB/s; the others 6.11-6.14); the other shapes are selectable
+    // in benchmark builds
+    int shape = (move_variant() >> 12) & 0xf;
+    if (shape == 0) shape = tables ? 4 : 3;
+    switch (shape) {
     case 1: launch_append<u32x4, 1, 4, 1>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
     case 2: launch_append<u32x4, 2, 4, 1>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
-    case 3: launch_append<u32x4, 4, 1, 1>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
     case 4: launch_append<u32x4, 1, 1, 1>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
-    default: launch_append<u32x4, 2, 1, 1>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
+    case 5: launch_append<u32x4, 2, 1, 1>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
+    default: launch_append<u32x4, 4, 1, 1>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
     }
   } else {
     switch (vec) {

@@ -19,7 +19,8 @@ extern "C" {
 /* Launch variants of the hooks library's own kernels: 0 = the product's defaults.
  * bits 8-11: 1 = non-temporal stores in the 16-byte block moves (default: sc0 sc1);
  * bits 12-15: shape of the 16-byte copy append (token rows per wave, waves per workgroup):
- *   0 = (2, 1) default, 1 = (1, 4), 2 = (2, 4), 3 = (4, 1), 4 = (1, 1);
+ *   0 = default ((4, 1) for a per-layer launch, (1, 1) for a whole-step launch), 1 = (1, 4), 2 = (2, 4),
+ *   3 = (4, 1), 4 = (1, 1), 5 = (2, 1);
  * bits 16-19: log2 of the blocks per plane visit of pack / unpack (15 = plain order);
  * bit 24: fp8 append with the IEEE division instead of the reciprocal form.
  * Process-wide, not thread-safe. Returns the previous value. */

@@ -12,7 +12,8 @@ import numpy as np
 import torch
 
 from . import _lib
-from ._lib import EMM_DTYPE_BF16, EMM_DTYPE_F16, EMM_MAX_LAYERS, EMM_MAX_SEGMENTS, check, ptr_table
+from ._lib import (EMM_DTYPE_BF16, EMM_DTYPE_F16, EMM_FP8_SATURATE, EMM_MAX_LAYERS, EMM_MAX_SEGMENTS, check,
+                   ptr_table)
 
 IndexLike = Union[Sequence[int], np.ndarray, torch.Tensor]
 
@@ -203,11 +204,13 @@ def copy_blocks(pool: PoolView, block_mapping: Union[torch.Tensor, Sequence[Sequ
                                   m.data_ptr(), m.shape[0], stream), "emm_copy_blocks")
 
 
-def _half_code(dt: torch.dtype, what: str) -> int:
+def _half_code(dt: torch.dtype, what: str, saturate: bool = False) -> int:
+    """src_dtype code of the C ABI; ``saturate`` selects the clamping fp8 mode (EMM_FP8_SATURATE)."""
+    flag = EMM_FP8_SATURATE if saturate else 0
     if dt == torch.bfloat16:
-        return EMM_DTYPE_BF16
+        return EMM_DTYPE_BF16 | flag
     if dt == torch.float16:
-        return EMM_DTYPE_F16
+        return EMM_DTYPE_F16 | flag
     raise TypeError(f"{what}: 16-bit side must be bfloat16 or float16, got {dt}")
 
 
@@ -279,11 +282,13 @@ def _cache_slots(cache: torch.Tensor, row_elems: int, what: str) -> int:
 
 def reshape_and_cache(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
                       slot_mapping: torch.Tensor, k_scale: Optional[torch.Tensor] = None,
-                      v_scale: Optional[torch.Tensor] = None) -> None:
+                      v_scale: Optional[torch.Tensor] = None, saturate: bool = False) -> None:
     """Append one layer: ``cache.view(slots, row)[slot_mapping[t]] = cvt(x[t])`` for slots >= 0.
 
     Same-width caches are copied bit for bit; a 1-byte cache with a 16-bit source
-    is quantised to fp8-e4m3fn with ``k_scale`` / ``v_scale`` (one float each)."""
+    is quantised to fp8-e4m3fn with ``k_scale`` / ``v_scale`` (one float each):
+    ``(x.float() / scale).to(float8_e4m3fn)``, or with ``saturate`` the quotient clamped to
+    [-448, 448] first (overflow gives +-448 instead of NaN; never the default)."""
     lib = _lib.load()
     if not (key.is_cuda and value.is_cuda and key_cache.is_cuda and value_cache.is_cuda and slot_mapping.is_cuda):
         raise RuntimeError("reshape_and_cache: every tensor must be on the GPU; the KV kernels run on the GPU only")
@@ -310,7 +315,7 @@ def reshape_and_cache(key: torch.Tensor, value: torch.Tensor, key_cache: torch.T
     elif ceb == 1 and eb == 2:
         if k_scale is None or v_scale is None:
             raise ValueError("fp8 cache needs k_scale and v_scale")
-        code = _half_code(key.dtype, "reshape_and_cache")
+        code = _half_code(key.dtype, "reshape_and_cache", saturate)
         k_s = _scales_tensor(k_scale, 1, key.device)
         v_s = _scales_tensor(v_scale, 1, key.device)
         check(lib.emm_reshape_and_cache_fp8(key.data_ptr(), value.data_ptr(), key_cache.data_ptr(),
@@ -408,7 +413,8 @@ def _check_slot_mapping(slot_mapping: torch.Tensor, T: int) -> torch.Tensor:
 
 def reshape_and_cache_paged(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor,
                             value_cache: torch.Tensor, slot_mapping: torch.Tensor,
-                            k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None) -> None:
+                            k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None,
+                            saturate: bool = False) -> None:
     """Append one layer into the paged-attention layout:
     ``key_cache[b, h, d // x, o, d % x] = key[t, h, d]``, ``value_cache[b, h, d, o] = value[t, h, d]``
     with ``b, o = divmod(slot_mapping[t], block_size)``; slots < 0 are skipped.
@@ -426,7 +432,7 @@ def reshape_and_cache_paged(key: torch.Tensor, value: torch.Tensor, key_cache: t
             raise ValueError("fp8 cache needs k_scale and v_scale")
         keep = (_scales_tensor(k_scale, 1, key.device), _scales_tensor(v_scale, 1, key.device))
         k_ptr, v_ptr = keep[0].data_ptr(), keep[1].data_ptr()
-    code = _half_code(key.dtype, "reshape_and_cache_paged") if ceb == 1 else 0
+    code = _half_code(key.dtype, "reshape_and_cache_paged", saturate) if ceb == 1 else 0
     check(lib.emm_reshape_and_cache_paged(key.data_ptr(), value.data_ptr(), key_cache.data_ptr(),
                                           value_cache.data_ptr(), slot_mapping.data_ptr(), T, H, D, bs, NB, ks, vs,
                                           code, ceb, k_ptr, v_ptr, _stream_ptr(key.device)),
@@ -440,7 +446,7 @@ class PagedLayeredAppend:
 
     def __init__(self, keys: Sequence[torch.Tensor], values: Sequence[torch.Tensor],
                  key_caches: Sequence[torch.Tensor], value_caches: Sequence[torch.Tensor],
-                 k_scales=None, v_scales=None):
+                 k_scales=None, v_scales=None, saturate: bool = False):
         self.lib = _lib.load()
         L = len(keys)
         if not (len(values) == len(key_caches) == len(value_caches) == L):
@@ -460,7 +466,7 @@ class PagedLayeredAppend:
         if self.fp8:
             if k_scales is None or v_scales is None:
                 raise ValueError("fp8 cache needs k_scales and v_scales")
-            self.code = _half_code(keys[0].dtype, "PagedLayeredAppend")
+            self.code = _half_code(keys[0].dtype, "PagedLayeredAppend", saturate)
             self.k_s = _scales_tensor(k_scales, L, self.device)
             self.v_s = _scales_tensor(v_scales, L, self.device)
         self.groups = []
@@ -495,7 +501,7 @@ class LayeredAppend:
 
     def __init__(self, keys: Sequence[torch.Tensor], values: Sequence[torch.Tensor],
                  key_caches: Sequence[torch.Tensor], value_caches: Sequence[torch.Tensor],
-                 k_scales=None, v_scales=None):
+                 k_scales=None, v_scales=None, saturate: bool = False):
         self.lib = _lib.load()
         L = len(keys)
         if not (len(values) == len(key_caches) == len(value_caches) == L):
@@ -527,7 +533,7 @@ class LayeredAppend:
         if self.fp8:
             if k_scales is None or v_scales is None:
                 raise ValueError("fp8 cache needs k_scales and v_scales")
-            self.code = _half_code(keys[0].dtype, "LayeredAppend")
+            self.code = _half_code(keys[0].dtype, "LayeredAppend", saturate)
             self.k_s = _scales_tensor(k_scales, L, self.device)
             self.v_s = _scales_tensor(v_scales, L, self.device)
         self.groups = []
@@ -564,9 +570,9 @@ class LayeredAppend:
 
 def reshape_and_cache_layers(keys: Sequence[torch.Tensor], values: Sequence[torch.Tensor],
                              key_caches: Sequence[torch.Tensor], value_caches: Sequence[torch.Tensor],
-                             slot_mapping: torch.Tensor, k_scales=None, v_scales=None) -> None:
+                             slot_mapping: torch.Tensor, k_scales=None, v_scales=None, saturate: bool = False) -> None:
     """Append all layers of one step in a single launch (per group of EMM_MAX_LAYERS)."""
-    LayeredAppend(keys, values, key_caches, value_caches, k_scales, v_scales)(slot_mapping)
+    LayeredAppend(keys, values, key_caches, value_caches, k_scales, v_scales, saturate)(slot_mapping)
 
 
 def _launch_concat(lib, ptrs, sizes, out: torch.Tensor, stream) -> None:

@@ -185,6 +185,20 @@ void orc_quant_fp8(const uint16_t *x, int64_t n, float scale, int src_dtype, uin
   }
 }
 
+/* saturating variant: the quotient is clamped to [-448, 448] before the cast (NaN stays NaN), so
+ * overflow and +-inf give sign|0x7E and only NaN gives sign|0x7F:
+ * torch.clamp(x.float() / scale, -448, 448).to(torch.float8_e4m3fn), the convention of vLLM's fp8
+ * KV cache (the cache dtype the reference leaves open at elasticmm/engine/v0/worker.py:194). */
+void orc_quant_fp8_sat(const uint16_t *x, int64_t n, float scale, int src_dtype, uint8_t *q) {
+  for (int64_t i = 0; i < n; ++i) {
+    volatile float d = half_to_f32(x[i], src_dtype) / scale; /* one fp32 division */
+    float c = d;
+    if (c > 448.0f) c = 448.0f;   /* comparisons with NaN are false: NaN passes through */
+    if (c < -448.0f) c = -448.0f;
+    q[i] = orc_f32_to_e4m3fn(c);
+  }
+}
+
 /* dequantise n fp8 bytes: out = 16bit_rne(float(q) * scale) */
 void orc_dequant_fp8(const uint8_t *q, int64_t n, float scale, int out_dtype, uint16_t *out) {
   for (int64_t i = 0; i < n; ++i) {

@@ -35,6 +35,10 @@ tests/test_oracle.py:
       and on the explicit known answers 448, 464, 465, 480, -1000, 2^-9, 2^-10,
       2^-10*1.0001, 17, 18, 19, inf (bytes 126,126,127,127,255,1,0,1,88,89,90,127);
       SHA-256 of each sweep committed under tests/golden/.
+  fp8 quantise, saturating mode: c_quant_fp8_sat == torch.clamp(x.float() / s, -448, 448)
+      .to(torch.float8_e4m3fn) on all 65 536 bf16 and f16 inputs x 6 scales; known answers
+      (448, 464, 465, 1e6, inf -> 0x7E; NaN -> 0x7F; the negatives with the sign bit); equal to the
+      non-saturating cast wherever that one is not 0x7F / 0xFF.
   fp8 dequantise: exhaustive over 256 bytes x scales against torch
       ``(q.float() * s).to(bfloat16)``; NaN bytes are compared as "is NaN"
       because torch's CPU bf16 cast yields 0xFFFF (vectorised) or 0x7FC0
@@ -282,6 +286,22 @@ def c_quant_fp8(x: torch.Tensor, scale: float) -> np.ndarray:
     out = np.empty(bits.size, dtype=np.uint8)
     lib().orc_quant_fp8(_ptr(bits), ctypes.c_int64(bits.size), ctypes.c_float(scale), _dtype_code(x.dtype), _ptr(out))
     return out.reshape(tuple(x.shape))
+
+
+def c_quant_fp8_sat(x: torch.Tensor, scale: float) -> np.ndarray:
+    """Saturating variant: e4m3fn(clamp(float(x) / scale, -448, 448)); returns uint8 of x.shape."""
+    bits = x.contiguous().view(torch.int16).reshape(-1).numpy().view(np.uint16)
+    out = np.empty(bits.size, dtype=np.uint8)
+    lib().orc_quant_fp8_sat(_ptr(bits), ctypes.c_int64(bits.size), ctypes.c_float(scale), _dtype_code(x.dtype),
+                            _ptr(out))
+    return out.reshape(tuple(x.shape))
+
+
+def ref_quant_fp8_sat(x: torch.Tensor, scale: float) -> torch.Tensor:
+    """The saturating cast as a torch expression (uint8 bit patterns): the quotient clamped to the
+    finite range of e4m3fn before the library cast. NaN passes through clamp unchanged."""
+    q = x.float() / torch.tensor(scale, dtype=torch.float32)
+    return torch.clamp(q, -448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)
 
 
 def c_dequant_fp8(q: np.ndarray, scale: float, out_dtype: torch.dtype = torch.bfloat16) -> np.ndarray:

@@ -31,6 +31,30 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f"{name} declared in emm_kv.h but not exported"
 
 
+def test_hooks_exist_only_in_the_hooks_build():
+    """The product library carries no benchmark switch or probe: those live in libemm_kv_hooks.so, which
+    exports the whole product ABI next to them (so a benchmark can route its calls through it)."""
+    from elasticmm_amd.build import hooks_library_path
+
+    hooks_header = open(os.path.join(ROOT, "elasticmm_amd", "csrc", "emm_kv_hooks.h")).read()
+    hooks_header = re.sub(r"/\*.*?\*/", "", hooks_header, flags=re.S)
+    hook_syms = sorted(set(re.findall(r"\b(emm_hook_[a-z0-9_]+)\s*\(", hooks_header)))
+    assert hook_syms == sorted(_lib.HOOK_SIGNATURES) and len(hook_syms) >= 3
+    product = ctypes.CDLL(library_path())
+    for name in hook_syms + ["emm_set_move_variant"]:
+        assert not hasattr(product, name), f"{name} must not be exported by the product library"
+    assert os.path.exists(hooks_library_path()), "libemm_kv_hooks.so has not been built"
+    hooks = ctypes.CDLL(hooks_library_path())
+    for name in hook_syms + declared_symbols():
+        assert hasattr(hooks, name), f"{name} missing from the hooks build"
+    # nothing in the package reaches for the hooks build on its own
+    pkg = os.path.join(ROOT, "elasticmm_amd")
+    for fn in os.listdir(pkg):
+        if fn.endswith(".py") and fn not in ("_lib.py", "build.py"):
+            text = open(os.path.join(pkg, fn)).read()
+            assert "hooks" not in text, f"{fn} refers to the hooks build"
+
+
 def test_binding_table_matches_header():
     assert sorted(_lib.SIGNATURES) == declared_symbols()
     text = open(HEADER).read()

@@ -745,6 +745,52 @@ def test_worker_coordinated_pull_and_collective():
         dst.write_kv_blocks([1, 2], torch.zeros(shape, dtype=torch.bfloat16, device=DEV))
 
 
+def test_failed_receive_leaves_no_stale_layers_on_the_link():
+    """A receive that gives up (deadline, wrong block count) drops the rest of that transfer from the link:
+    the next transfer between the same ranks moves its own bytes, not the stale layers."""
+    src, dst = make_pair()
+    si, di = [5, 9, 0, 31], [1, 2, 3, 30]
+    # timeout before the first layer: the three queued layer messages must go away
+    res = dst.p2p_coordinated_transfer_kv(src, 0, si, di, timeout=-1.0)
+    assert "error" in res and src.link.pending(0, 1) == 0
+    # wrong block count on the receiving side: error dict, link drained
+    assert src.p2p_send_kv(1, si)["blocks"] == 4 and src.link.pending(0, 1) == 3
+    bad = dst.p2p_recv_kv(0, di[:3])
+    assert bad["bytes"] == 0 and "error" in bad and src.link.pending(0, 1) == 0
+    # two sends queued, the first received with the wrong count: only the first is dropped
+    si2, di2 = [7, 8, 30, 2], [0, 15, 16, 17]
+    src.p2p_send_kv(1, si)
+    src.p2p_send_kv(1, si2)
+    assert "error" in dst.p2p_recv_kv(0, di[:2]) and src.link.pending(0, 1) == 3
+    good = dst.p2p_recv_kv(0, di2)
+    assert good["blocks"] == 4 and "error" not in good
+    check_moved(src, dst, si2, di2)
+    # pull: a request larger than the protocol's 1024 slots raises before anything is queued
+    with pytest.raises(ValueError):
+        dst.p2p_pull_kv(0, list(range(1025)), list(range(1025)))
+    assert src.link.pending(1, 0, 999) == 0
+
+
+def test_transfer_manager_moves_vision_embeddings():
+    from elasticmm_amd.kv_transfer import KVTransferManager, TransferMethod
+
+    src, dst = make_pair()
+    src.init_vecache()
+    dst.init_vecache()
+    ve = torch.randn((300, 3584), generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+    src.write_vision_blocks("img0", ve.to(DEV))
+    m = KVTransferManager(TransferMethod.NCCL)
+    m.register_workers("encoding", [src, dst], [0, 1])
+    assert m.transfer_vision_embeddings_sync("img0", 0, [0, 1], 1, [4, 5]) is True
+    assert same_bits(dst.extract_vision_blocks("img0"), ve)
+    assert m.transfer_vision_embeddings_sync("absent", 0, [], 1, []) is False   # KeyError on the source -> False
+    import asyncio
+    assert asyncio.run(m.transfer_vision_embeddings("img0", 0, [0], 1, [1])) is True
+    assert m.get_stats()["transfer_count"] == 2
+    m.close()
+
+
+
 # ------------------------------------------------------------------ full-size properties
 def test_cfg2_full_size_migration_properties():
     """Qwen2-7B KV shape at full size: 28 x [2,60000,16,4,128] bf16 twice (2 x 51.3 GiB).
@@ -1240,6 +1286,83 @@ def test_fp8_quantise_many_scales_against_the_division():
                 assert bad.size == 0, f"{dtype} scale {sv!r}: {bad.size} mismatches, first input bits " \
                                       f"{bad[:6].tolist()} got {got[bad[:6]].tolist()} want {want[bad[:6]].tolist()}"
                 assert (raw(pools[l][1]) == want).all()
+
+
+def test_fp8_saturating_mode_exhaustive_on_gpu():
+    """kv_cache_dtype "fp8_e4m3_sat": every bf16 and f16 input at the golden scales, extreme scales that
+    take the division path, and a negative scale, through the flash append (vector and element paths), the
+    whole-step launch and the paged layout, against the oracle's clamp-then-cast. NaN inputs stay NaN,
+    overflow and infinities give +-448."""
+    import struct
+
+    def f32(bits):
+        return struct.unpack("<f", struct.pack("<I", bits))[0]
+
+    kat = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "fp8_kat.json")))
+    scales = list(kat["scales"]) + [2.0 ** -31, 2.0 ** 31, -0.05, f32(0x3DFFFFFF), 448.0]
+    slots = torch.arange(64, device=DEV)
+    for dtype in (torch.bfloat16, torch.float16):
+        allx = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype)
+        key = allx.view(64, 8, 128).to(DEV)
+        for sv in scales:
+            s32 = float(np.float32(sv))
+            want = orc.c_quant_fp8_sat(allx, s32).reshape(-1)
+            sc = torch.tensor([s32], dtype=torch.float32, device=DEV)
+            kc = torch.zeros((4, 16, 8, 128), dtype=torch.uint8, device=DEV)
+            vc = torch.zeros_like(kc)
+            cache_ops.reshape_and_cache_flash(key, key, kc, vc, slots, "fp8_e4m3_sat", sc, sc)
+            got = raw(kc)
+            bad = np.nonzero(got != want)[0]
+            assert bad.size == 0, f"{dtype} scale {s32!r}: {bad.size} mismatches, first input bits {bad[:6].tolist()} " \
+                                  f"got {got[bad[:6]].tolist()} want {want[bad[:6]].tolist()}"
+            assert (raw(vc) == want).all()
+        # the other entry points at one scale: whole-step launch, element-wise path (rows of 7 elements),
+        # paged layout
+        s32 = float(np.float32(0.037))
+        want = orc.c_quant_fp8_sat(allx, s32).reshape(-1)
+        sc = torch.tensor([s32], dtype=torch.float32, device=DEV)
+        pools = [torch.zeros((2, 4, 16, 8, 128), dtype=torch.uint8, device=DEV) for _ in range(2)]
+        cache_ops.reshape_and_cache_flash_layers([key, key], [key, key], pools, slots, "fp8_sat", [s32, s32], [s32, s32])
+        assert (raw(pools[1][0]) == want).all() and (raw(pools[0][1]) == want).all()
+        odd = allx[:7 * 9360].view(9360, 1, 7).to(DEV)
+        kc7 = torch.zeros((585, 16, 1, 7), dtype=torch.uint8, device=DEV)
+        vc7 = torch.zeros_like(kc7)
+        cache_ops.reshape_and_cache_flash(odd, odd, kc7, vc7, torch.arange(9360, device=DEV), "fp8_e4m3_sat", sc, sc)
+        assert (raw(kc7) == want[:7 * 9360]).all()
+        kcp = torch.zeros((4, 8, 128 // 16, 16, 16), dtype=torch.uint8, device=DEV)
+        vcp = torch.zeros((4, 8, 128, 16), dtype=torch.uint8, device=DEV)
+        cache_ops.reshape_and_cache(key, key, kcp, vcp, slots, "fp8_e4m3_sat", sc, sc)
+        # value_cache[b, h, d, o] = q(value[t, h, d]) with t = b * 16 + o
+        assert (raw(vcp.permute(0, 3, 1, 2).contiguous()) == want).all()
+        assert (raw(kcp.permute(0, 3, 1, 2, 4).contiguous()) == want).all()
+
+
+def test_fp8_fast_quotient_equals_the_division_for_every_significand_pair():
+    """The append divides through a reciprocal and one correction step. That the result is the correctly rounded
+    quotient is established by exhaustion: the three operations commute with powers of two while everything stays
+    in the normal range, so only the significands matter — all 2^10 x significands (the 11 significant bits of an
+    f16; bf16 values are a subset), both signs, against all 2^23 scale significands, 1.7e10 pairs per exponent
+    pair. Several exponent pairs are swept: quotients in the middle of the fp8 range, at its overflow edge and in
+    its subnormal range, and scales at both ends of the interval the fast form is used in. Every fp32 quotient
+    must equal the division's, and the bytes after conversion too, in both overflow modes."""
+    hooks = _lib.load_hooks()
+    pairs = [(0, 0), (3, -5), (-2, -4), (4, -5), (-12, -5), (-3, -30), (5, 30), (2, -7)]
+    for x_exp, s_exp in pairs:
+        counters = torch.zeros(5, dtype=torch.int64, device=DEV)
+        rc = hooks.emm_hook_fp8_quotient_sweep(x_exp, s_exp, 0, 1 << 23, counters.data_ptr(),
+                                               torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, hooks.emm_last_error()
+        c = counters.cpu().tolist()
+        say(f"quotient sweep x_exp={x_exp} s_exp={s_exp}: {c[3]} pairs, raw mismatches {c[0]}, byte mismatches {c[1]} / {c[2]}")
+        assert c[3] == 2048 * (1 << 23)
+        assert c[0] == 0 and c[1] == 0 and c[2] == 0, f"x_exp={x_exp} s_exp={s_exp}: first differing pair {c[4]:#x}"
+    # outside the interval the library takes the division itself: the sweep then compares it with itself and
+    # still has to report a clean run (keeps the hook honest about which path it exercised)
+    counters = torch.zeros(5, dtype=torch.int64, device=DEV)
+    assert hooks.emm_hook_fp8_quotient_sweep(0, 40, 0, 1 << 12, counters.data_ptr(),
+                                             torch.cuda.current_stream().cuda_stream) == 0
+    assert counters.cpu().tolist()[:4] == [0, 0, 0, 2048 * (1 << 12)]
+
 
 
 # ------------------------------------------------------------------ transfer manager on real workers

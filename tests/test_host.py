@@ -310,6 +310,96 @@ def test_migrate_requests_allocates_moves_frees_and_rolls_back():
     assert src_bm.get_block_table("c") != [] and src_bm.get_block_table("e") != []
 
 
+def test_batched_migration_rollback_leaves_nothing_queued():
+    """With batching, requests that were already queued when a later allocation fails must leave the queue
+    before their destination blocks are freed: a later flush may not touch the destination."""
+    src_bm, dst_bm = BlockManager(16), BlockManager(4)
+    src_bm.allocate_blocks("a", 2)
+    src_bm.allocate_blocks("b", 1)
+    src_bm.allocate_blocks("c", 3)          # does not fit once a and b hold 3 of the 4 destination blocks
+    tm = KVTransferManager(TransferMethod.NCCL, enable_batching=True, batch_size=10, batch_timeout=1e9)
+    w0, w1 = _FakeWorker(0), _FakeWorker(1)
+    tm.register_worker(0, w0, "prefill")
+    tm.register_worker(1, w1, "decoding")
+    assert not tm.migrate_requests_sync(["a", "b", "c"], 0, src_bm, 1, dst_bm)
+    assert tm._transfer_queue.get((0, 1), []) == []
+    assert tm.flush_all() is True
+    assert w0.calls == [] and w1.calls == []                  # nothing was sent, nothing was written
+    assert dst_bm.get_num_avail_gpu_blocks() == 4             # destination blocks all free again
+    assert src_bm.get_block_table("a") == [0, 1] and src_bm.get_block_table("c") == [3, 4, 5]
+    # an unrelated request queued before the failing migration stays queued and is flushed normally
+    assert tm.transfer_kv_cache_sync("other", 0, 1, [9], [3]) is True
+    assert not tm.migrate_requests_sync(["a", "b", "c"], 0, src_bm, 1, dst_bm)
+    assert [t[0] for t in tm._transfer_queue[(0, 1)]] == ["other"]
+    assert tm.flush_all() is True and w0.calls == [("send", 1, [9])] and w1.calls == [("recv", 0, [3])]
+
+
+def test_transfer_coroutines_do_not_block_the_event_loop():
+    """The blocking part of a transfer (launches + the workers' device synchronisation) runs on the manager's
+    own thread: other coroutines of the loop keep running while it is in progress."""
+    import asyncio
+    import threading
+    import time as _time
+
+    loop_thread = threading.get_ident()
+    seen = {}
+
+    class _SlowWorker(_FakeWorker):
+        def extract_kv_blocks(self, blocks):
+            seen["thread"] = threading.get_ident()
+            _time.sleep(0.25)                    # stands for a long device synchronisation
+            return super().extract_kv_blocks(blocks)
+
+    tm = KVTransferManager(TransferMethod.P2P_COPY)
+    tm.register_worker(0, _SlowWorker(0), "prefill")
+    tm.register_worker(1, _FakeWorker(1), "decoding")
+    ticks = []
+
+    async def ticker():
+        for _ in range(20):
+            ticks.append(_time.perf_counter())
+            await asyncio.sleep(0.01)
+
+    async def main():
+        t = asyncio.ensure_future(ticker())
+        t0 = _time.perf_counter()
+        ok = await tm.transfer_kv_cache("r", 0, 1, [1, 2], [3, 4])
+        t1 = _time.perf_counter()
+        await t
+        return ok, t0, t1
+
+    ok, t0, t1 = asyncio.run(main())
+    assert ok is True and seen["thread"] != loop_thread
+    during = [x for x in ticks if t0 < x < t1]
+    assert len(during) >= 10, f"the loop ran only {len(during)} other steps during a 0.25 s transfer"
+    tm.close()
+
+
+def test_vision_transfer_through_the_manager_with_fake_workers():
+    class _VeWorker(_FakeWorker):
+        def __init__(self, rank):
+            super().__init__(rank)
+            self.ve = {}
+
+        def extract_vision_blocks(self, rid):
+            if rid not in self.ve:
+                raise KeyError(f"Request {rid} not found in vision cache")
+            return self.ve[rid]
+
+        def write_vision_blocks(self, rid, data):
+            self.ve[rid] = data
+
+    seen = []
+    tm = KVTransferManager(TransferMethod.NCCL, metrics_callback=lambda **kw: seen.append(kw))
+    a, b = _VeWorker(0), _VeWorker(1)
+    a.ve["img"] = "embedding"
+    tm.register_workers("encoding", [a, b], [0, 1])
+    assert tm.transfer_vision_embeddings_sync("img", 0, [1], 1, [2]) is True and b.ve["img"] == "embedding"
+    assert tm.transfer_vision_embeddings_sync("none", 0, [], 1, []) is False
+    assert tm.transfer_vision_embeddings_sync("img", 0, [1], 7, [2]) is False      # unknown rank
+    assert tm.get_stats()["transfer_count"] == 1 and seen == []                     # counted, not a kv metric
+
+
 def test_compute_slot_mapping_matches_the_definition():
     from elasticmm_amd import cache_ops
 

@@ -377,6 +377,39 @@ def test_fp8_quant_exhaustive_vs_torch_cast(golden_dir, dtype, name):
         assert hashlib.sha256(got.tobytes()).hexdigest() == kat["sweep_sha256"][f"{name}@{s}"]
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fp8_saturating_quant_exhaustive_vs_torch_clamp_cast(golden_dir, dtype):
+    """The saturating mode is pinned to the library routines that define it — torch.clamp then
+    torch's cast — on every 16-bit input, and to the non-saturating cast (pinned above) wherever
+    that one does not overflow. A wrong clamp bound, a clamp after the cast, or NaN folded into
+    the bound each fail one of the three checks."""
+    kat = json.load(open(os.path.join(golden_dir, "fp8_kat.json")))
+    allx = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype)
+    nan_in = torch.isnan(allx.float()).numpy()
+    for s in kat["scales"]:
+        got = orc.c_quant_fp8_sat(allx, s)
+        want = orc.ref_quant_fp8_sat(allx, s).numpy()
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, f"scale {s}: first mismatch at bits {bad[:5]}: {got[bad[:5]]} vs {want[bad[:5]]}"
+        plain = orc.c_quant_fp8(allx, s)
+        finite = (plain & 0x7F) != 0x7F
+        assert (got[finite] == plain[finite]).all()            # no overflow: the two modes agree
+        over = ~finite & ~nan_in
+        assert ((got[over] & 0x7F) == 0x7E).all()              # overflow and +-inf: 448 with the sign
+        assert (got[over] & 0x80 == plain[over] & 0x80).all()
+        assert ((got[nan_in] & 0x7F) == 0x7F).all()            # NaN stays NaN
+
+
+def test_fp8_saturating_known_answers():
+    x = torch.tensor([448.0, 464.0, 465.0, 1.0e6, float("inf"), -465.0, -float("inf"), float("nan"), 17.0, 2.0 ** -10],
+                     dtype=torch.float32).to(torch.bfloat16)
+    got = orc.c_quant_fp8_sat(x, 1.0).tolist()
+    assert got[:7] == [0x7E, 0x7E, 0x7E, 0x7E, 0x7E, 0xFE, 0xFE]
+    assert got[7] & 0x7F == 0x7F and got[8:] == [88, 0]
+    # a scale turns the bound into 448 * scale in input units
+    assert orc.c_quant_fp8_sat(torch.tensor([44.0, 44.8, 50.0], dtype=torch.bfloat16), 0.1).tolist()[1:] == [0x7E, 0x7E]
+
+
 def test_fp8_monotone_and_nearest():
     """Brute force from the definition: the chosen code is a nearest representable
     value (ties to the even code), for a dense sample of magnitudes below 464."""
