@@ -1,22 +1,37 @@
 #!/usr/bin/env python3
 """Benchmark of the KV data-movement path on one MI355X.
 
-Workload (default, ``qwen2_7b_migrate``): the Qwen2-7B KV shape — 28 layers of
+Headline workload (``qwen2_7b_migrate``): the Qwen2-7B KV shape — 28 layers of
 ``[2, 60000, 16, 4, 128]`` bf16 (51.3 GiB per pool) — and a batch of 32 migrating
 requests with prompt lengths U{512..4096} plus a 1024-token image prefix
 (96..320 blocks each). One *step* moves every request of the batch: pack from the
 source pool under its block table into a contiguous transfer buffer
 (``KVWorker.extract_kv_blocks``, one call per request as the reference does), then
 unpack every buffer into a second, independently allocated pool under a different
-table (``KVWorker.write_kv_blocks``, one call per request). Everything is resident in HBM before the timed
-region (pools, block tables); values are synthetic N(0, 0.5).
+table (``KVWorker.write_kv_blocks``, one call per request). Everything is resident in
+HBM before the timed region (pools, block tables); values are synthetic N(0, 0.5).
 
-Prints ONE JSON line. ``value`` is whole-job GB/s = algorithmic bytes (read +
-write of pack and of unpack = 4 x payload) / wall time of the timed steps.
-``roofline`` prices the block-move kernel (pack and unpack are two instances of
-the same kernel) against the 8 TB/s HBM peak from HIP-event times of its launches
-inside the timed region. ``cpu_baseline`` times the reference's torch expressions
-(oracle ``ref_*``) on the host cores for a bounded sample of the same batch.
+Prints ONE JSON line. ``value`` is whole-job GB/s = algorithmic bytes (read + write of
+pack and of unpack = 4 x payload) / wall time of the timed steps. ``roofline`` prices the
+block-move kernel (pack and unpack are two instances of the same kernel) against the
+8 TB/s HBM peak from HIP-event times of its launches inside the timed region.
+``cpu_baseline`` times the reference's torch expressions (oracle ``ref_*``) on the host
+cores for bounded samples of the same workloads.
+
+``extra`` holds the other shapes of the path, each with its own algorithmic bytes, rate,
+fraction of the 8 TB/s peak, kernel name and average launch time:
+  allocation_modes   the headline again with each pool in one allocation and with one
+                     allocation per layer (what a pool adopted from vLLM looks like)
+  list_indices       the headline with block tables passed as Python lists (the reference's
+                     call shape: one pinned staging + H2D copy per call)
+  batched / fused    one launch for the whole batch; fused pool-to-pool migrate; copy_blocks
+  ceilings           what this memory system does for the same access patterns without the
+                     other half of the copy (sequential / gathered reads, sequential /
+                     scattered writes, plain copy), from the hooks build of the library
+  append             reshape_and_cache for one step (config 3): per-layer calls eager / from a
+                     HIP graph, one launch for all layers, and the launch-bound yardsticks
+  append_paged_layout, cfg1_latency, fp8_70b_shape (config 4), rebalance_200GB (config 5,
+  with the vision gather on the same and on a second stream), swap_pcie
 """
 import argparse
 import json
@@ -30,6 +45,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+ALL_SECTIONS = ["batched", "ceilings", "append", "paged", "lists", "modes", "cfg1", "fp8", "rebalance", "swap"]
 
 
 def parse():
@@ -40,18 +56,54 @@ def parse():
     ap.add_argument("--blocks", type=int, default=60000, help="pool size in blocks (the Qwen2-7B migration workload uses 60000)")
     ap.add_argument("--requests", type=int, default=32)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements (append, batched, copy)")
-    ap.add_argument("--variant", type=int, default=0, help="block-move launch variant (tuning)")
+    ap.add_argument("--no-extra", action="store_true", help="headline only (same as --sections none)")
+    ap.add_argument("--sections", default="all",
+                    help="comma-separated secondary measurements to run: " + ",".join(ALL_SECTIONS) + " (all | none)")
+    ap.add_argument("--variant", type=int, default=0,
+                    help="launch variant of the hooks build (tuning; routes every call through libemm_kv_hooks.so)")
     ap.add_argument("--spread", type=int, default=4,
-                    help="stripes per pool: each pool's layers are allocated in this many pieces spread over the "
-                         "free device memory (0 or 1: one allocation per pool)")
-    ap.add_argument("--extended", action="store_true",
-                    help="after the headline, free its pools and measure the fp8 70B-class shape and the ~200 GB "
-                         "rebalancing shape at full size (adds about a minute)")
+                    help="stripes per pool of the headline: each pool's layers are allocated in this many pieces spread "
+                         "over the free device memory (0 or 1: one allocation per pool)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB copy with the same tile engine (a kernel of known traffic, "
                          "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     return ap.parse_args()
+
+
+# ---------------------------------------------------------------------------------------------- helpers
+def rec(nbytes, ms, launches=1, kernel=None, **more):
+    """One measurement: algorithmic bytes, milliseconds, rate, fraction of the HBM peak."""
+    gbps = nbytes / (ms * 1e-3) / 1e9
+    out = {"GBps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4), "ms": round(ms, 4),
+           "algorithmic_bytes": int(nbytes), "launches": launches,
+           "avg_launch_us": round(ms * 1e3 / launches, 2)}
+    if kernel:
+        out["kernel"] = kernel
+    out.update(more)
+    return out
+
+
+def timed(fn, iters, warmup=2):
+    """Median and min milliseconds of fn() over iters runs, HIP events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(iters):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        e1.synchronize()
+        ts.append(e0.elapsed_time(e1))
+    ts.sort()
+    return ts[len(ts) // 2], ts[0]
+
+
+def _wall(fn):
+    t0 = time.perf_counter()
+    fn()
+    return time.perf_counter() - t0
 
 
 def make_requests(num_requests, num_blocks, seed):
@@ -71,7 +123,76 @@ def make_requests(num_requests, num_blocks, seed):
     return tables, total
 
 
-def cpu_baseline(tables, L, bs, H, D, dtype, budget_s=15.0):
+def measure_migrate(src_w, dst_w, tabs, steps, warmup, payload):
+    """`steps` timed steps of: pack every request on the source side, then unpack every request on the
+    destination side. All packs run before the unpacks: 6 GB of transfer buffers lie between a buffer's
+    pack and its unpack, so the unpack reads come from HBM (not from the 256 MB Infinity Cache) as they
+    would on a receiving GPU. HIP events bracket each phase (3 per step, on the launch stream), not each
+    launch: an event record between every two kernels costs several microseconds of idle GPU."""
+    def step(events=None):
+        if events is not None:
+            e0, e1, e2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+            e0.record()
+        bufs = [src_w.extract_kv_blocks(si) for si, _ in tabs]
+        if events is not None:
+            e1.record()
+        for k, (_, di) in enumerate(tabs):
+            dst_w.write_kv_blocks(di, bufs[k])
+        if events is not None:
+            e2.record()
+            events.append((e0, e1, e2))
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    events = []
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step(events)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    pack_ms = sum(e0.elapsed_time(e1) for e0, e1, _ in events)
+    unpack_ms = sum(e1.elapsed_time(e2) for _, e1, e2 in events)
+    launches = 2 * len(tabs) * steps
+    kern_bytes = 4 * payload * steps
+    return {
+        "value": 4 * payload * steps / wall / 1e9,
+        "ms_per_step": wall / steps * 1e3,
+        "kernel_GBps": kern_bytes / ((pack_ms + unpack_ms) * 1e-3) / 1e9,
+        "pack_GBps": kern_bytes / 2 / (pack_ms * 1e-3) / 1e9,
+        "unpack_GBps": kern_bytes / 2 / (unpack_ms * 1e-3) / 1e9,
+        "launches": launches,
+        "avg_launch_us": (pack_ms + unpack_ms) * 1e3 / launches,
+        "avg_bytes_per_launch": kern_bytes / launches,
+    }
+
+
+def make_workers(NB, L, bs, H, D, dtype, dev, spread, monolithic=True, fill=True):
+    from elasticmm_amd.worker import KVWorker
+
+    src_w, dst_w = KVWorker(0, "cuda:0", bs), KVWorker(1, "cuda:0", bs)
+    for w in (src_w, dst_w):
+        w.init_kvcache(NB, num_layers=L, num_kv_heads=H, head_size=D, dtype=dtype, monolithic=monolithic,
+                       spread_stripes=spread)
+    if fill:
+        g = torch.Generator(device=dev).manual_seed(2)
+        for t in src_w.kv_cache:
+            t.normal_(0.0, 0.5, generator=g)
+    for t in dst_w.kv_cache:
+        t.zero_()
+    torch.cuda.synchronize()
+    return src_w, dst_w
+
+
+def release(*workers):
+    for w in workers:
+        w.kv_cache = None
+        w._pool = None
+    torch.cuda.empty_cache()
+
+
+# ---------------------------------------------------------------------------------------------- CPU baselines
+def cpu_baseline(tables, L, bs, H, D, dtype, budget_s=8.0):
     """The reference's torch path on the host cores: the same batch (same block counts per
     request) on pools reduced to just hold it — bytes moved depend on the blocks per request,
     not on the pool size. Passes repeat until about `budget_s` seconds of CPU work are done."""
@@ -113,6 +234,61 @@ def cpu_baseline(tables, L, bs, H, D, dtype, budget_s=15.0):
     }
 
 
+def cpu_baseline_append(budget_s=5.0, L=28, bs=16, H=4, D=128, T=8448):
+    """Config 3 on the host: the closed form of reshape_and_cache_flash (index_copy_ of the valid rows) per
+    layer, same T, same 5 % padded slots, pool reduced to 2048 blocks (bytes moved depend on T, not on the pool)."""
+    from oracle import kv_oracle as orc
+
+    NBc = 2048
+    g = torch.Generator().manual_seed(3)
+    slots = torch.randperm(NBc * bs, generator=g)[:T].clone()
+    slots[torch.rand(T, generator=g) < 0.05] = -1
+    valid = int((slots >= 0).sum())
+    key = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+    value = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+    caches = [torch.zeros((2, NBc, bs, H, D), dtype=torch.bfloat16) for _ in range(L)]
+    step_bytes = L * (valid * 2 * H * D * 4 + 8 * T)
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 200):
+        t0 = time.perf_counter()
+        for l in range(L):
+            orc.ref_reshape_and_cache_flash(key, value, caches[l][0], caches[l][1], slots)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": round(valid / med), "unit": "tokens/s", "GBps": round(step_bytes / med / 1e9, 2),
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"one step of {T} tokens ({valid} valid) x {L} layers, per-layer index_copy_ of the valid rows on "
+                      f"CPU tensors, pool reduced to {NBc} blocks; median of {len(times)} steps ({med * 1e3:.1f} ms each)"}
+
+
+def cpu_baseline_cfg1(budget_s=2.0):
+    """Config 1 exactly as specified, on the host."""
+    from oracle import kv_oracle as orc
+
+    L, NB, bs, H, D = 4, 1024, 16, 8, 128
+    g = torch.Generator().manual_seed(0)
+    src = [torch.randn((2, NB, bs, H, D), generator=g).to(torch.float16) for _ in range(L)]
+    dst = [torch.zeros((2, NB, bs, H, D), dtype=torch.float16) for _ in range(L)]
+    si = torch.randperm(NB, generator=g)[:32].tolist()
+    di = torch.randperm(NB, generator=torch.Generator().manual_seed(1))[:32].tolist()
+    nbytes = 4 * 32 * L * 2 * bs * H * D * 2
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 5 or (time.perf_counter() - t_start < budget_s and len(times) < 2000):
+        t0 = time.perf_counter()
+        orc.ref_write_kv_blocks(dst, di, orc.ref_extract_kv_blocks(src, si))
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": round(nbytes / med / 1e9, 3), "unit": "GB/s", "us_per_pack_plus_unpack": round(med * 1e6, 1),
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"config 1 (4 layers x [2,1024,16,8,128] fp16, one request of 32 blocks), extract + write on "
+                      f"CPU tensors; median of {len(times)} passes"}
+
+
+# ---------------------------------------------------------------------------------------------- main
 def main():
     args = parse()
     if args.gpus != 1:
@@ -122,93 +298,56 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the KV kernels have no CPU fallback", file=sys.stderr)
         sys.exit(2)
+    if args.no_extra or args.sections == "none":
+        sections = set()
+    elif args.sections == "all":
+        sections = set(ALL_SECTIONS)
+    else:
+        sections = set(args.sections.split(","))
+        unknown = sections - set(ALL_SECTIONS)
+        if unknown:
+            raise SystemExit(f"unknown sections: {sorted(unknown)}")
 
     from elasticmm_amd import _lib, kv_ops
-    from elasticmm_amd.kv_ops import PoolView
-    from elasticmm_amd.worker import KVWorker
 
     if args.variant:
         # launch variants exist only in the hooks build of the library: route this process through it
         _lib.use_hooks_build().emm_hook_set_move_variant(args.variant)
-    lib = _lib.load()
+    _lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     L, bs, H, D, dtype = 28, 16, 4, 128, torch.bfloat16
     NB = args.blocks
     chunk = bs * H * D * 2
     tables, total_blocks = make_requests(args.requests, NB, seed=2)
-
-    src_w, dst_w = KVWorker(0, "cuda:0", bs), KVWorker(1, "cuda:0", bs)
-    src_w.init_kvcache(NB, num_layers=L, num_kv_heads=H, head_size=D, dtype=dtype, monolithic=True,
-                       spread_stripes=args.spread)
-    dst_w.init_kvcache(NB, num_layers=L, num_kv_heads=H, head_size=D, dtype=dtype, monolithic=True,
-                       spread_stripes=args.spread)
-    g = torch.Generator(device=dev).manual_seed(2)
-    for t in src_w.kv_cache:
-        t.normal_(0.0, 0.5, generator=g)
-    for t in dst_w.kv_cache:
-        t.zero_()
-    dev_tables = [(s.to(dev), d.to(dev)) for s, d in tables]
-    torch.cuda.synchronize()
-
     payload = total_blocks * L * 2 * chunk       # bytes held by the batch's blocks
     bytes_per_step = 4 * payload                 # pack: read + write, unpack: read + write
 
-    def step(events=None):
-        # pack every request on the source side, then unpack every request on the destination
-        # side: 6 GB of transfer buffers lie between a buffer's pack and its unpack, so the
-        # unpack reads come from HBM (not from the 256 MB Infinity Cache) as they would on a
-        # receiving GPU.
-        # HIP events bracket each phase (3 per step, on the launch stream), not each launch: an
-        # event record between every two kernels costs several microseconds of idle GPU.
-        if events is not None:
-            e0, e1, e2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
-            e0.record()
-        bufs = [src_w.extract_kv_blocks(si) for si, _ in dev_tables]
-        if events is not None:
-            e1.record()
-        for k, (_, di) in enumerate(dev_tables):
-            dst_w.write_kv_blocks(di, bufs[k])
-        if events is not None:
-            e2.record()
-            events.append((e0, e1, e2))
-
-    for _ in range(args.warmup):
-        step()
+    src_w, dst_w = make_workers(NB, L, bs, H, D, dtype, dev, args.spread)
+    dev_tables = [(s.to(dev), d.to(dev)) for s, d in tables]
     torch.cuda.synchronize()
-    events = []
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step(events)
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    wall = t1 - t0
-    ms_per_step = wall / args.steps * 1e3
-    value = bytes_per_step * args.steps / wall / 1e9
 
-    # kernel time of the block-move kernel (pack and unpack instances) from the phase events:
-    # each phase is 32 back-to-back launches of that kernel and nothing else
-    pack_ms = sum(e0.elapsed_time(e1) for e0, e1, _ in events)
-    unpack_ms = sum(e1.elapsed_time(e2) for _, e1, e2 in events)
-    launches = 2 * len(dev_tables) * len(events)
-    kern_bytes = 2 * 2 * payload * len(events)  # per step: pack 2 x payload + unpack 2 x payload
-    achieved = kern_bytes / ((pack_ms + unpack_ms) * 1e-3) / 1e9
+    m = measure_migrate(src_w, dst_w, dev_tables, args.steps, args.warmup, payload)
+    # HBM bytes per launch from rocprofv3: FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 (factors from a plain 1 GiB
+    # copy in the same profile run) came to TRAFFIC_RATIO x the algorithmic bytes for this kernel on this
+    # workload (profiles/block_move_qwen2_7b_migrate_pmc.txt). A counter cannot be read inside this process;
+    # the figure below is that measured ratio applied to this run's bytes per launch.
+    TRAFFIC_RATIO = 1.0004
     roofline = {
         "bound": "hbm",
         "kernel": "emm_block_move_kernel (pack + unpack instances)",
-        "achieved": round(achieved, 1),
+        "achieved": round(m["kernel_GBps"], 1),
         "peak": HBM_PEAK_GBPS,
         "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBPS, 4),
-        # HBM bytes per launch: rocprofv3 FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 (factors from a plain
-        # 1 GiB copy in the same profile run) came to 1.0004 x the algorithmic bytes for this kernel on this
-        # workload (profiles/block_move_qwen2_7b_migrate_pmc.txt); the figure is that ratio, not a live counter
-        "traffic": int(kern_bytes / launches * 1.0004),
-        "launches": launches,
-        "avg_launch_us": round((pack_ms + unpack_ms) * 1e3 / launches, 2),
-        "avg_bytes_per_launch": int(kern_bytes / launches),
-        "pack_GBps": round(kern_bytes / 2 / (pack_ms * 1e-3) / 1e9, 1),
-        "unpack_GBps": round(kern_bytes / 2 / (unpack_ms * 1e-3) / 1e9, 1),
+        "frac": round(m["kernel_GBps"] / HBM_PEAK_GBPS, 4),
+        "traffic": int(m["avg_bytes_per_launch"] * TRAFFIC_RATIO),
+        "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by a plain copy of known size: "
+                          "%.4f x algorithmic (profiles/block_move_qwen2_7b_migrate_pmc.txt)" % TRAFFIC_RATIO,
+        "launches": m["launches"],
+        "avg_launch_us": round(m["avg_launch_us"], 2),
+        "avg_bytes_per_launch": int(m["avg_bytes_per_launch"]),
+        "pack_GBps": round(m["pack_GBps"], 1),
+        "unpack_GBps": round(m["unpack_GBps"], 1),
     }
 
     if args.calibrate_copy:
@@ -223,30 +362,65 @@ def main():
     assert torch.equal(dst_w.kv_cache[L - 1][:, di], src_w.kv_cache[L - 1][:, si]), "migration check failed"
 
     extra = {}
-    if not args.no_extra:
-        extra = secondary(src_w, dst_w, dev_tables, payload, L, bs, H, D, NB, dev)
+    if "lists" in sections:
+        list_tables = [(s.tolist(), d.tolist()) for s, d in tables]
+        ml = measure_migrate(src_w, dst_w, list_tables, max(3, args.steps // 4), 1, payload)
+        extra["list_indices"] = {
+            "what": "the headline with block tables passed as Python lists (the reference's call shape): every call "
+                    "checks the ids on the host, stages them in pinned memory and copies them to the device",
+            "value_GBps": round(ml["value"], 1), "frac": round(ml["value"] / HBM_PEAK_GBPS, 4),
+            "ms_per_step": round(ml["ms_per_step"], 4), "pack_GBps": round(ml["pack_GBps"], 1),
+            "unpack_GBps": round(ml["unpack_GBps"], 1)}
+    if "batched" in sections:
+        extra.update(batched(src_w, dst_w, dev_tables, payload, L, chunk, NB, dev))
+    if "ceilings" in sections:
+        extra["ceilings"] = ceilings(src_w, dst_w, dev_tables, payload, dev)
+    if "append" in sections:
+        extra["append"] = append_bench(src_w.kv_cache, NB, bs, H, D, None, None, dev)
+    if "paged" in sections:
+        extra["append_paged_layout"] = paged_append_bench(src_w.kv_cache, NB, bs, H, D, dev)
+    release(src_w, dst_w)
+    dev_tables = None
 
-    if args.extended:
-        src_w.kv_cache = dst_w.kv_cache = None
-        src_w._pool = dst_w._pool = None
-        dev_tables = None
-        torch.cuda.empty_cache()
-        extra["extended"] = extended(dev, args.spread)
+    if "modes" in sections:
+        modes = {}
+        for name, spread, mono in (("one_allocation_per_pool", 0, True), ("one_allocation_per_layer", 0, False)):
+            sw, dw = make_workers(NB, L, bs, H, D, dtype, dev, spread, monolithic=mono)
+            tabs = [(s.to(dev), d.to(dev)) for s, d in tables]
+            mm = measure_migrate(sw, dw, tabs, max(3, args.steps // 4), 2, payload)
+            modes[name] = {"value_GBps": round(mm["value"], 1), "frac": round(mm["value"] / HBM_PEAK_GBPS, 4),
+                           "pack_GBps": round(mm["pack_GBps"], 1), "unpack_GBps": round(mm["unpack_GBps"], 1),
+                           "avg_launch_us": round(mm["avg_launch_us"], 2)}
+            release(sw, dw)
+            del tabs
+        modes["what"] = ("the headline workload on pools allocated differently: 'one_allocation_per_pool' is "
+                         "init_kvcache's default (spread_stripes=0), 'one_allocation_per_layer' is what a pool adopted "
+                         "from vLLM's CacheEngine through bind_kv_cache looks like (28 separate torch.empty); the "
+                         "headline itself uses %d stripes per pool" % args.spread)
+        extra["allocation_modes"] = modes
+    if "cfg1" in sections:
+        extra["cfg1_latency"] = cfg1_latency(dev)
+    if "fp8" in sections:
+        extra["fp8_70b_shape"] = fp8_shape(dev, args.spread)
+    if "rebalance" in sections:
+        extra["rebalance_200GB"] = rebalance(dev)
+    if "swap" in sections:
+        extra["swap_pcie"] = swap_bench(dev)
 
     result = {
         "metric": "KV pack+unpack GB/s",
-        "value": round(value, 1),
+        "value": round(m["value"], 1),
         "unit": "GB/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4),
+        "ms_per_step": round(m["ms_per_step"], 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "u8",
         "data": "synthetic",
-        "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "pct_hbm_peak": round(100.0 * m["value"] / HBM_PEAK_GBPS, 2),
         "config": {
             "workload": "qwen2_7b_migrate: 28 layers x [2,%d,16,4,128] bf16 x 2 pools, %d requests (%d blocks, "
                         "%.2f GB payload), 32 per-request packs, then 32 per-request unpacks under different block tables"
@@ -254,70 +428,51 @@ def main():
             "num_layers": L, "num_blocks": NB, "block_size": bs, "kv_heads": H, "head_dim": D,
             "requests": len(tables), "blocks_moved": total_blocks, "algorithmic_bytes_per_step": bytes_per_step,
             "pool_allocation": ("each pool allocated on its own, layers in %d stripes spread over the free device "
-                                "memory" % args.spread) if args.spread > 1 else "each pool one allocation",
+                                "memory (extra.allocation_modes has the other layouts)" % args.spread)
+            if args.spread > 1 else "each pool one allocation",
         },
         "roofline": roofline,
         "extra": extra,
     }
     if not args.no_cpu_baseline:
-        # free the device pools first: the host leg needs nothing from them
         result["cpu_baseline"] = cpu_baseline(tables, L, bs, H, D, dtype)
+        result["cpu_baseline"]["append"] = cpu_baseline_append()
+        result["cpu_baseline"]["cfg1"] = cpu_baseline_cfg1()
     print(json.dumps(result), flush=True)
 
 
-def _wall(fn):
-    t0 = time.perf_counter()
-    fn()
-    return time.perf_counter() - t0
-
-
-def timed(fn, iters, warmup=2):
-    """Median and min milliseconds of fn() over iters runs, HIP events on the current stream."""
-    for _ in range(warmup):
-        fn()
-    torch.cuda.synchronize()
-    ts = []
-    for _ in range(iters):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        fn()
-        e1.record()
-        e1.synchronize()
-        ts.append(e0.elapsed_time(e1))
-    ts.sort()
-    return ts[len(ts) // 2], ts[0]
-
-
-def secondary(src_w, dst_w, dev_tables, payload, L, bs, H, D, NB, dev):
-    """Other shapes of the same path, reported next to the headline (not bench lines of their own)."""
-    from elasticmm_amd import cache_ops, kv_ops
+# ---------------------------------------------------------------------------------------------- secondary shapes
+def batched(src_w, dst_w, dev_tables, payload, L, chunk, NB, dev):
+    """One launch for the whole batch, the fused pool-to-pool migrate, copy_blocks, plain-copy yardsticks."""
+    from elasticmm_amd import kv_ops
 
     out = {}
-    chunk = bs * H * D * 2
     sp, dp = src_w.pool, dst_w.pool
-    # one launch for the whole batch (concatenated tables)
     all_si = torch.cat([s for s, _ in dev_tables])
     all_di = torch.cat([d for _, d in dev_tables])
     buf = torch.empty(sp.packed_shape(all_si.numel()), dtype=sp.dtype, device=dev)
-    med, mn = timed(lambda: kv_ops.kv_pack(sp, all_si, out=buf), 10)
-    out["batched_pack_GBps"] = round(2 * payload / (med * 1e-3) / 1e9, 1)
-    med, mn = timed(lambda: kv_ops.kv_unpack(dp, all_di, buf), 10)
-    out["batched_unpack_GBps"] = round(2 * payload / (med * 1e-3) / 1e9, 1)
-    med, mn = timed(lambda: kv_ops.kv_migrate(sp, all_si, dp, all_di), 10)
-    out["fused_migrate_GBps"] = round(2 * payload / (med * 1e-3) / 1e9, 1)
+    med, _ = timed(lambda: kv_ops.kv_pack(sp, all_si, out=buf), 10)
+    out["batched_pack"] = rec(2 * payload, med, 1, "emm_block_move_kernel<pack, plain order>")
+    med, _ = timed(lambda: kv_ops.kv_unpack(dp, all_di, buf), 10)
+    out["batched_unpack"] = rec(2 * payload, med, 1, "emm_block_move_kernel<unpack, grouped order>")
+    med, _ = timed(lambda: kv_ops.kv_migrate(sp, all_si, dp, all_di), 10)
+    out["fused_migrate"] = rec(2 * payload, med, 1, "emm_block_move_kernel<pool to pool, runs order>",
+                               note="replaces a pack and an unpack: half their traffic")
+
     def interleaved():
         for si, di in dev_tables:
             dst_w.write_kv_blocks(di, src_w.extract_kv_blocks(si))
 
-    med, mn = timed(interleaved, 5)
-    out["per_request_pack_then_unpack_interleaved_GBps"] = round(4 * payload / (med * 1e-3) / 1e9, 1)
-    # yardsticks: plain copies of the same byte count
+    med, _ = timed(interleaved, 5)
+    out["per_request_pack_then_unpack_interleaved"] = rec(
+        4 * payload, med, 2 * len(dev_tables), note="each buffer unpacked right after its pack: partly read back from "
+                                                    "the 256 MB last-level cache, not the headline")
     flat = buf.view(-1)
     other = torch.empty_like(flat)
-    med, mn = timed(lambda: kv_ops.stream_copy(flat, other), 10)
-    out["plain_copy_same_engine_GBps"] = round(2 * payload / (med * 1e-3) / 1e9, 1)
-    med, mn = timed(lambda: other.copy_(flat), 10)
-    out["torch_copy_GBps"] = round(2 * payload / (med * 1e-3) / 1e9, 1)
+    med, _ = timed(lambda: kv_ops.stream_copy(flat, other), 10)
+    out["plain_copy_same_engine"] = rec(2 * payload, med, 1, "emm_stream_copy_kernel")
+    med, _ = timed(lambda: other.copy_(flat), 10)
+    out["torch_copy"] = rec(2 * payload, med, 1, "torch.Tensor.copy_")
     del other, buf
     # copy_blocks: half of the batch's blocks to free blocks of the same pool
     P = all_si.numel() // 2
@@ -326,10 +481,50 @@ def secondary(src_w, dst_w, dev_tables, payload, L, bs, H, D, NB, dev):
     free = (~used).nonzero().squeeze(1)
     if free.numel() >= P:
         mapping = torch.stack([all_si[:P], free[:P]], 1).contiguous()
-        med, mn = timed(lambda: kv_ops.copy_blocks(sp, mapping), 10)
-        out["copy_blocks_GBps"] = round(2 * P * L * 2 * chunk / (med * 1e-3) / 1e9, 1)
-    out["append"] = append_bench(src_w.kv_cache, NB, bs, H, D, torch.bfloat16, None, None, dev)
-    out["append_paged_layout"] = paged_append_bench(src_w.kv_cache, NB, bs, H, D, dev)
+        med, _ = timed(lambda: kv_ops.copy_blocks(sp, mapping), 10)
+        out["copy_blocks"] = rec(2 * P * L * 2 * chunk, med, 1, "emm_block_move_kernel<pool to pool, pairs>")
+    return out
+
+
+def ceilings(src_w, dst_w, dev_tables, payload, dev):
+    """Measured ceilings of this memory system for the access patterns of pack and unpack, each half on its own
+    (kernels of the hooks build with the grid of pack / unpack: one 4 KiB tile per 256-thread workgroup):
+    sequential read, sequential write, gathered read of the batch's 16 KiB chunks from the source pool,
+    scattered write of them into the destination pool. Rates are bytes touched / time (one direction)."""
+    from elasticmm_amd import _lib
+
+    hooks = _lib.load_hooks()
+    sp, dp = src_w.pool, dst_w.pool
+    all_si = torch.cat([s for s, _ in dev_tables]).contiguous()
+    all_di = torch.cat([d for _, d in dev_tables]).contiguous()
+    n = all_si.numel()
+    lin = torch.empty(payload, dtype=torch.uint8, device=dev).random_(0, 255)
+    sink = torch.zeros(1024, dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    stab, dtab = _lib.ptr_table(sp.ptrs), _lib.ptr_table(dp.ptrs)
+
+    def probe(kind, table, idx):
+        rc = hooks.emm_hook_probe(kind, table, sp.num_layers, sp.num_kv, sp.num_blocks, sp.chunk_bytes,
+                                  idx.data_ptr() if idx is not None else None, n, lin.data_ptr(), sink.data_ptr(), stream)
+        if rc != 0:
+            raise RuntimeError(hooks.emm_last_error().decode())
+
+    out = {}
+    for name, kind, table, idx in (("sequential_read", _lib.EMM_PROBE_SEQ_READ, None, None),
+                                   ("sequential_write", _lib.EMM_PROBE_SEQ_WRITE, None, None),
+                                   ("gather_read_16KiB_chunks", _lib.EMM_PROBE_GATHER_READ, stab, all_si),
+                                   ("scatter_write_16KiB_chunks", _lib.EMM_PROBE_SCATTER_WRITE, dtab, all_di)):
+        med, _ = timed(lambda: probe(kind, table, idx), 10)
+        out[name] = rec(payload, med, 1, "emm_probe_kernel")
+    r, w = out["sequential_read"]["GBps"], out["sequential_write"]["GBps"]
+    g, s = out["gather_read_16KiB_chunks"]["GBps"], out["scatter_write_16KiB_chunks"]["GBps"]
+    out["harmonic_seq_read_seq_write"] = round(2 / (1 / r + 1 / w), 1)
+    out["harmonic_gather_read_seq_write"] = round(2 / (1 / g + 1 / w), 1)
+    out["harmonic_seq_read_scatter_write"] = round(2 / (1 / r + 1 / s), 1)
+    out["note"] = ("a copy alternates reads and writes on the same channels and stays below the harmonic mean of its two "
+                   "halves (compare plain_copy_same_engine with harmonic_seq_read_seq_write); the scatter probe overwrote "
+                   "the destination blocks of the batch")
+    del lin
     return out
 
 
@@ -359,13 +554,12 @@ def paged_append_bench(kv, NB, bs, H, D, dev, T=8448, decode=256):
         for l in range(L):
             cache_ops.reshape_and_cache(keys[l], values[l], kcs[l], vcs[l], slots, "auto")
 
-    def entry(ms):
-        return {"tokens_per_s": round(T / (ms * 1e-3)), "ms_per_step": round(ms, 4),
-                "GBps": round(step_bytes / (ms * 1e-3) / 1e9, 1)}
+    def entry(ms, launches):
+        return rec(step_bytes, ms, launches, "emm_append_paged_kernel", tokens_per_s=round(T / (ms * 1e-3)))
 
-    res = {"T": T, "decode_tokens": decode, "layers": L, "algorithmic_bytes_per_step": step_bytes}
+    res = {"T": T, "decode_tokens": decode, "layers": L}
     med, _ = timed(per_layer, 20)
-    res["per_layer_calls_eager"] = entry(med)
+    res["per_layer_calls_eager"] = entry(med, L)
     graph = torch.cuda.CUDAGraph()
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -375,27 +569,31 @@ def paged_append_bench(kv, NB, bs, H, D, dev, T=8448, decode=256):
     with torch.cuda.graph(graph):
         per_layer()
     med, _ = timed(graph.replay, 20)
-    res["per_layer_calls_hip_graph"] = entry(med)
+    res["per_layer_calls_hip_graph"] = entry(med, L)
     plan = cache_ops.paged_layered_append(keys, values, kcs, vcs)
     med, _ = timed(lambda: plan(slots), 20)
-    res["one_launch_all_layers"] = entry(med)
+    res["one_launch_all_layers"] = entry(med, 1)
     # a decode-only step: every token alone in its block (each 2-byte V element and each 16-byte K piece
     # lands in a cache line of its own, so the memory system rewrites the token's whole block region)
     Td = 256
     dplan = cache_ops.paged_layered_append([k[:Td] for k in keys], [v[:Td] for v in values], kcs, vcs)
     dslots = dec[:Td].contiguous() if decode >= Td else slots[:Td].contiguous()
     med, _ = timed(lambda: dplan(dslots), 20)
-    res["decode_only_256_tokens_one_launch"] = {"tokens_per_s": round(Td / (med * 1e-3)), "ms_per_step": round(med, 4),
-                                                "GBps": round(L * Td * 2 * H * D * 4 / (med * 1e-3) / 1e9, 1)}
+    res["decode_only_256_tokens_one_launch"] = rec(L * Td * 2 * H * D * 4, med, 1, "emm_append_paged_kernel",
+                                                   tokens_per_s=round(Td / (med * 1e-3)))
     return res
 
 
-def append_bench(kv, NB, bs, H, D, cache_dtype_name, k_scales, v_scales, dev, T=8448):
+def append_bench(kv, NB, bs, H, D, k_scales, v_scales, dev, T=8448):
     """reshape_and_cache for one step: 256 decode tokens + one 8192-token prefill chunk, slots random
     over the pool, 5 % padded (-1). Three ways of issuing it: the vLLM-shaped call once per layer
     (eager Python), the same L launches replayed from a HIP graph, and one launch for all layers from
-    a prepared plan. tokens/s = valid tokens / time of all layers."""
-    from elasticmm_amd import cache_ops
+    a prepared plan (possible only where every layer's K/V already exists: re-ingest, prefix load — not
+    a model forward, which produces layer l+1's K/V after layer l's append). tokens/s = valid tokens /
+    time of all layers. `launch_bound_yardsticks` replays, from the same kind of graph, L plain copies
+    of one layer's bytes with the library's copy kernel: what a chain of L dependent launches of
+    that size costs on this machine with no indirection at all."""
+    from elasticmm_amd import cache_ops, kv_ops
 
     L = len(kv)
     fp8 = kv[0].element_size() == 1
@@ -410,42 +608,106 @@ def append_bench(kv, NB, bs, H, D, cache_dtype_name, k_scales, v_scales, dev, T=
     step_bytes = L * (valid * 2 * row * (2 + kv[0].element_size()) + 8 * T)
     ks = [None] * L if not fp8 else [k_scales[l:l + 1] for l in range(L)]
     vs = [None] * L if not fp8 else [v_scales[l:l + 1] for l in range(L)]
+    kernel = "emm_append_fp8_kernel" if fp8 else "emm_append_kernel"
 
     def per_layer():
         for l in range(L):
             cache_ops.reshape_and_cache_flash(keys[l], values[l], kv[l][0], kv[l][1], slots, mode, ks[l], vs[l])
 
-    def entry(ms):
-        return {"tokens_per_s": round(valid / (ms * 1e-3)), "ms_per_step": round(ms, 4),
-                "GBps": round(step_bytes / (ms * 1e-3) / 1e9, 1)}
+    def entry(ms, launches):
+        return rec(step_bytes, ms, launches, kernel, tokens_per_s=round(valid / (ms * 1e-3)))
 
-    res = {"T": T, "valid": valid, "layers": L, "algorithmic_bytes_per_step": step_bytes}
+    def graphed(fn):
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()
+        torch.cuda.current_stream().wait_stream(side)
+        with torch.cuda.graph(graph):
+            fn()
+        return graph
+
+    res = {"T": T, "valid": valid, "layers": L}
     med, _ = timed(per_layer, 20)
-    res["per_layer_calls_eager"] = entry(med)
-    graph = torch.cuda.CUDAGraph()
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        per_layer()
-    torch.cuda.current_stream().wait_stream(side)
-    with torch.cuda.graph(graph):
-        per_layer()
-    med, _ = timed(graph.replay, 20)
-    res["per_layer_calls_hip_graph"] = entry(med)
+    res["per_layer_calls_eager"] = entry(med, L)
+    med, _ = timed(graphed(per_layer).replay, 20)
+    res["per_layer_calls_hip_graph"] = entry(med, L)
     plan = cache_ops.layered_append(keys, values, kv, mode, k_scales, v_scales)
     med, _ = timed(lambda: plan(slots), 20)
-    res["one_launch_all_layers"] = entry(med)
+    res["one_launch_all_layers"] = entry(med, 1)
+    # yardstick: L dependent launches of a plain copy of the same bytes per layer
+    layer_bytes = step_bytes // L
+    half = layer_bytes // 2 // 4096 * 4096
+    srcs = [torch.empty(half, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(L)]
+    dsts = [torch.empty(half, dtype=torch.uint8, device=dev) for _ in range(L)]
+
+    def copies():
+        for l in range(L):
+            kv_ops.stream_copy(srcs[l], dsts[l])
+
+    med, _ = timed(graphed(copies).replay, 20)
+    res["launch_bound_yardsticks"] = {
+        "plain_copy_of_one_layers_bytes_per_launch_hip_graph": rec(2 * half * L, med, L, "emm_stream_copy_kernel"),
+        "note": "a chain of L dependent launches moving one layer's bytes each, no slot indirection: the per-layer "
+                "append cannot be faster than this on this machine"}
     return res
 
 
-def extended(dev, spread=4):
-    """The two other target shapes at full size (run with --extended; needs the whole GPU):
-    the fp8-e4m3 70B-class per-GPU shape and the elastic rebalancing of a ~200 GB pool."""
+def cfg1_latency(dev):
+    """Config 1: 4 layers x [2,1024,16,8,128] fp16, one request of 32 blocks (8 MiB buffer). Latency of one
+    extract_kv_blocks + one write_kv_blocks; 32 disjoint block tables are cycled so that consecutive calls
+    touch different blocks (512 MiB of pools in total, twice the last-level cache)."""
+    from elasticmm_amd.worker import KVWorker
+
+    L, NB, bs, H, D = 4, 1024, 16, 8, 128
+    sw, dw = KVWorker(0, "cuda:0", bs), KVWorker(1, "cuda:0", bs)
+    for w in (sw, dw):
+        w.init_kvcache(NB, num_layers=L, num_kv_heads=H, head_size=D, dtype=torch.float16)
+    for t in sw.kv_cache:
+        t.normal_()
+    g = torch.Generator().manual_seed(0)
+    sp, dp = torch.randperm(NB, generator=g), torch.randperm(NB, generator=torch.Generator().manual_seed(1))
+    tabs = [(sp[i * 32:(i + 1) * 32].to(dev), dp[i * 32:(i + 1) * 32].to(dev)) for i in range(32)]
+    lists = [(s.tolist(), d.tolist()) for s, d in tabs]
+    nbytes = 4 * 32 * L * 2 * bs * H * D * 2
+    state = {"i": 0}
+
+    def one(tables):
+        s, d = tables[state["i"] % 32]
+        state["i"] += 1
+        dw.write_kv_blocks(d, sw.extract_kv_blocks(s))
+
+    def many(tables, k=32):
+        for _ in range(k):
+            one(tables)
+
+    med, _ = timed(lambda: many(tabs), 10)
+    out = {"device_tables": rec(nbytes * 32, med, 64, "emm_block_move_kernel", us_per_pack_plus_unpack=round(med * 1e3 / 32, 2))}
+    med, _ = timed(lambda: many(lists), 10)
+    out["list_indices"] = rec(nbytes * 32, med, 64, "emm_block_move_kernel", us_per_pack_plus_unpack=round(med * 1e3 / 32, 2))
+    # one isolated call, device idle before and after (host launch + kernel + completion)
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(20):
+        t0 = time.perf_counter()
+        one(tabs)
+        torch.cuda.synchronize()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    out["isolated_call_wall_us"] = round(ts[len(ts) // 2] * 1e6, 1)
+    out["bytes_per_pack_plus_unpack"] = nbytes
+    release(sw, dw)
+    return out
+
+
+def fp8_shape(dev, spread=4):
+    """Config 4: 80 layers x [2, NB, 16, 8, 128] e4m3, 64 requests of U{1024..8192} tokens: pack / unpack of fp8
+    bytes, the quantising append (bf16 -> fp8), the dequantising unpack (fp8 -> bf16 pool)."""
     from elasticmm_amd import kv_ops
     from elasticmm_amd.kv_ops import PoolView
+    from elasticmm_amd.worker import allocate_layers_spread
 
-    out = {}
-    # ---- fp8: 80 layers x [2, NB, 16, 8, 128] e4m3, 64 requests of U{1024..8192} tokens
     L, bs, H, D, NB = 80, 16, 8, 128, 20000
     chunk = bs * H * D
     g = torch.Generator().manual_seed(4)
@@ -456,7 +718,6 @@ def extended(dev, spread=4):
     perm_d = torch.randperm(NB, generator=g)[:total].to(dev)
     k_scales = (torch.rand(L, generator=g) * 0.09 + 0.01).to(dev)
     v_scales = (torch.rand(L, generator=g) * 0.09 + 0.01).to(dev)
-    from elasticmm_amd.worker import allocate_layers_spread
 
     def make_pool(dtype):
         shape = (2, NB, bs, H, D)
@@ -482,11 +743,11 @@ def extended(dev, spread=4):
         payload += n * L * 2 * chunk
         off += n
         del buf
-    out["fp8_70b_shape"] = {"layers": L, "pool_blocks": NB, "requests": 64, "blocks": total,
-                            "payload_GB": round(payload / 1e9, 2),
-                            "pack_GBps": round(2 * payload / (ts_pack * 1e-3) / 1e9, 1),
-                            "unpack_GBps": round(2 * payload / (ts_unpack * 1e-3) / 1e9, 1)}
-    out["fp8_70b_shape"]["append"] = append_bench(src, NB, bs, H, D, "fp8", k_scales, v_scales, dev)
+    out = {"layers": L, "pool_blocks": NB, "requests": 64, "blocks": total, "payload_GB": round(payload / 1e9, 2),
+           "pack": rec(2 * payload, ts_pack, 64, "emm_block_move_kernel<pack>"),
+           "unpack": rec(2 * payload, ts_unpack, 64, "emm_block_move_kernel<unpack>"),
+           "pack_plus_unpack": rec(4 * payload, ts_pack + ts_unpack, 128, "emm_block_move_kernel")}
+    out["append"] = append_bench(src, NB, bs, H, D, k_scales, v_scales, dev)
     del dst, dp
     torch.cuda.empty_cache()
     # dequantising unpack into a bf16 pool (first 16 requests)
@@ -503,12 +764,17 @@ def extended(dev, spread=4):
         pay += n * L * 2 * chunk
         off += n
         del buf
-    out["fp8_70b_shape"]["dequant_unpack_GBps"] = round(3 * pay / (t_dq * 1e-3) / 1e9, 1)
+    out["dequant_unpack"] = rec(3 * pay, t_dq, 16, "emm_unpack_dequant_fp8_kernel",
+                                note="1 fp8 byte read + 2 bf16 bytes written per element")
     del src, sp, dq, dqp
     torch.cuda.empty_cache()
+    return out
 
-    # ---- GPU <-> CPU swap (pinned host pool, kernels read / write it over PCIe): Qwen2-7B layout
+
+def swap_bench(dev):
+    """GPU <-> CPU swap (pinned host pool, kernels read / write it over PCIe): Qwen2-7B layout."""
     from elasticmm_amd.worker import KVWorker
+
     w = KVWorker(0, "cuda:0", 16)
     w.init_kvcache(4096, 2048, num_layers=28, num_kv_heads=4, head_size=128, dtype=torch.bfloat16)
     for t in w.kv_cache:
@@ -538,14 +804,22 @@ def extended(dev, spread=4):
 
     t_d2h = min(_wall(d2h) for _ in range(4))
     t_h2d = min(_wall(h2d) for _ in range(4))
-    out["swap_pcie"] = {"blocks": nsw, "GB": round(sw_bytes / 1e9, 3),
-                        "swap_out_GBps": round(sw_bytes / t_out / 1e9, 1), "swap_in_GBps": round(sw_bytes / t_in / 1e9, 1),
-                        "contiguous_memcpy_d2h_GBps": round(sw_bytes / t_d2h / 1e9, 1),
-                        "contiguous_memcpy_h2d_GBps": round(sw_bytes / t_h2d / 1e9, 1)}
+    out = {"blocks": nsw, "GB": round(sw_bytes / 1e9, 3), "bound": "PCIe, not HBM",
+           "swap_out_GBps": round(sw_bytes / t_out / 1e9, 1), "swap_in_GBps": round(sw_bytes / t_in / 1e9, 1),
+           "contiguous_memcpy_d2h_GBps": round(sw_bytes / t_d2h / 1e9, 1),
+           "contiguous_memcpy_h2d_GBps": round(sw_bytes / t_h2d / 1e9, 1)}
     del w, stage_g, stage_c
     torch.cuda.empty_cache()
+    return out
 
-    # ---- rebalancing: ~200 GB bf16 pool in the Qwen2-7B layout, move 50 % of the live half
+
+def rebalance(dev):
+    """Config 5: ~200 GB bf16 pool in the Qwen2-7B layout, copy_blocks moves 50 % of the live half to disjoint free
+    blocks; the vision-embedding gather (128 images, 64..2304 patches x 3584 bf16) alone, interleaved with
+    copy_blocks on the same stream, and on a second stream next to it."""
+    from elasticmm_amd import kv_ops
+    from elasticmm_amd.kv_ops import PoolView
+
     L, bs, H, D = 28, 16, 4, 128
     chunk = bs * H * D * 2
     NB = 218000
@@ -559,39 +833,57 @@ def extended(dev, spread=4):
     free = perm[NB // 2:]
     P = live.numel() // 2
     mapping = torch.stack([live[:P], free[:P]], 1).contiguous().to(dev)
-    med, mn = timed(lambda: kv_ops.copy_blocks(pv, mapping), 5, warmup=1)
+    copy_bytes = 2 * P * L * 2 * chunk
+    med, _ = timed(lambda: kv_ops.copy_blocks(pv, mapping), 5, warmup=1)
     ok = bool(torch.equal(pool[3][:, mapping[:1000, 1]], pool[3][:, mapping[:1000, 0]]))
-    out["rebalance_200GB"] = {"pool_GB": round(pool.numel() * 2 / 1e9, 1), "pairs": P,
-                              "algorithmic_GB": round(2 * P * L * 2 * chunk / 1e9, 1), "ms": round(med, 3),
-                              "copy_blocks_GBps": round(2 * P * L * 2 * chunk / (med * 1e-3) / 1e9, 1),
-                              "spot_check": ok}
-    # vision-embedding gather interleaved on the same stream
+    out = {"pool_GB": round(pool.numel() * 2 / 1e9, 1), "pairs": P, "spot_check": ok,
+           "copy_blocks": rec(copy_bytes, med, 1, "emm_block_move_kernel<pool to pool, pairs>")}
     imgs = torch.randint(64, 2305, (128,), generator=g).tolist()
     embeds = [torch.randn((p_, 3584), device=dev).to(torch.bfloat16) for p_ in imgs]
     vis_bytes = 2 * sum(imgs) * 3584 * 2
     outbuf = torch.empty((sum(imgs), 3584), dtype=torch.bfloat16, device=dev)
+    vc = {"images": 128, "rows": sum(imgs)}
     med, _ = timed(lambda: kv_ops.concat_rows(embeds, out=outbuf), 10)
-    out["rebalance_200GB"]["vision_concat"] = {"images": 128, "rows": sum(imgs), "ms": round(med, 4),
-                                               "GBps": round(vis_bytes / (med * 1e-3) / 1e9, 1)}
+    vc["tensor_list"] = rec(vis_bytes, med, 1, "emm_concat_rows_kernel")
     # the same gather from segments prepared when the embeddings entered the cache (what
     # KVWorker.gather_vision_embeddings does): the host reads two fields per image instead of the tensors
     prepared = [kv_ops.RowSource(e) for e in embeds]
     med, _ = timed(lambda: kv_ops.concat_row_sources(prepared, out=outbuf), 10)
-    out["rebalance_200GB"]["vision_concat"]["prepared_segments_ms"] = round(med, 4)
-    out["rebalance_200GB"]["vision_concat"]["prepared_segments_GBps"] = round(vis_bytes / (med * 1e-3) / 1e9, 1)
+    vc["prepared_segments"] = rec(vis_bytes, med, 1, "emm_concat_rows_kernel")
     med_t, _ = timed(lambda: torch.cat(embeds, 0, out=outbuf), 10)
-    out["rebalance_200GB"]["vision_concat"]["torch_cat_GBps"] = round(vis_bytes / (med_t * 1e-3) / 1e9, 1)
-    quarter = mapping[:P // 8]
+    vc["torch_cat"] = rec(vis_bytes, med_t, 1, "torch.cat")
+    out["vision_concat"] = vc
+    parts = 8
+    row_off = [0]
+    for k in range(parts):
+        row_off.append(row_off[-1] + sum(imgs[k * 16:(k + 1) * 16]))
+    tot = 2 * (P // parts) * parts * L * 2 * chunk + vis_bytes
 
     def interleaved():
-        for k in range(8):
-            kv_ops.copy_blocks(pv, mapping[k * (P // 8):(k + 1) * (P // 8)])
-            kv_ops.concat_rows(embeds[k * 16:(k + 1) * 16], out=outbuf[:sum(imgs[k * 16:(k + 1) * 16])])
+        for k in range(parts):
+            kv_ops.copy_blocks(pv, mapping[k * (P // parts):(k + 1) * (P // parts)])
+            kv_ops.concat_row_sources(prepared[k * 16:(k + 1) * 16], out=outbuf[row_off[k]:row_off[k + 1]])
 
     med, _ = timed(interleaved, 3, warmup=1)
-    tot = 2 * (P // 8) * 8 * L * 2 * chunk + vis_bytes
-    out["rebalance_200GB"]["interleaved_copy_and_concat_GBps"] = round(tot / (med * 1e-3) / 1e9, 1)
-    del quarter
+    out["interleaved_same_stream"] = rec(tot, med, 2 * parts, note="8 x (copy_blocks of an eighth of the pairs, then "
+                                                                   "the gather of 16 images), alternating on one stream")
+    side = torch.cuda.Stream()  # default priority
+
+    def two_streams():
+        cur = torch.cuda.current_stream()
+        side.wait_stream(cur)
+        with torch.cuda.stream(side):
+            for k in range(parts):
+                kv_ops.concat_row_sources(prepared[k * 16:(k + 1) * 16], out=outbuf[row_off[k]:row_off[k + 1]])
+        for k in range(parts):
+            kv_ops.copy_blocks(pv, mapping[k * (P // parts):(k + 1) * (P // parts)])
+        cur.wait_stream(side)
+
+    med, _ = timed(two_streams, 3, warmup=1)
+    out["interleaved_two_streams"] = rec(tot, med, 2 * parts, note="the same launches with the gathers on a second "
+                                                                   "stream of the same priority, joined at the end")
+    del pool, pv, embeds, prepared, outbuf
+    torch.cuda.empty_cache()
     return out
 
 

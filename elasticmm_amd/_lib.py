@@ -14,6 +14,7 @@ from .build import hooks_library_path, library_path
 EMM_KV_ABI_VERSION = 2
 EMM_MAX_LAYERS = 96
 EMM_MAX_SEGMENTS = 128
+EMM_MAX_INLINE_IDS = 512
 EMM_DTYPE_BF16 = 0
 EMM_DTYPE_F16 = 1
 EMM_FP8_SATURATE = 0x100
@@ -28,6 +29,8 @@ SIGNATURES = {
     "emm_abi_version": (c_int, []),
     "emm_kv_pack": (c_int, [_PP, c_int, c_int, c_int64, c_int64, _P, c_int64, _P, _P]),
     "emm_kv_unpack": (c_int, [_PP, c_int, c_int, c_int64, c_int64, _P, c_int64, _P, _P]),
+    "emm_kv_pack_host_ids": (c_int, [_PP, c_int, c_int, c_int64, c_int64, _P, c_int64, _P, _P]),
+    "emm_kv_unpack_host_ids": (c_int, [_PP, c_int, c_int, c_int64, c_int64, _P, c_int64, _P, _P]),
     "emm_copy_blocks": (c_int, [_PP, c_int, c_int, c_int64, c_int64, _P, c_int64, _P]),
     "emm_kv_migrate": (c_int, [_PP, c_int64, _PP, c_int64, c_int, c_int, c_int64, _P, _P, c_int64, _P]),
     "emm_kv_unpack_dequant_fp8": (c_int, [_PP, c_int, c_int64, c_int64, _P, c_int64, _P, _P, _P, c_int, _P]),
@@ -51,7 +54,7 @@ SIGNATURES = {
 # libemm_kv_hooks.so only (csrc/emm_kv_hooks.h): benchmark / test hooks, absent from the product library
 HOOK_SIGNATURES = {
     "emm_hook_set_move_variant": (c_int, [c_int]),
-    "emm_hook_probe": (c_int, [_PP, c_int, c_int, c_int64, c_int64, _P, c_int64, _P, _P, _P]),
+    "emm_hook_probe": (c_int, [c_int, _PP, c_int, c_int, c_int64, c_int64, _P, c_int64, _P, _P, _P]),
     "emm_hook_fp8_quotient_sweep": (c_int, [c_int, c_int, ctypes.c_uint32, ctypes.c_uint32, _P, _P]),
 }
 EMM_PROBE_SEQ_READ, EMM_PROBE_SEQ_WRITE, EMM_PROBE_GATHER_READ, EMM_PROBE_SCATTER_WRITE = 0, 1, 2, 3

@@ -196,6 +196,14 @@ struct PlaneTables {
   PlaneTable t[N]; // pack: source; unpack: destination; pool-to-pool: source, destination
 };
 
+// Block ids carried in the argument block itself (host-side tables of up to EMM_MAX_INLINE_IDS
+// entries): no device-side table, no host-to-device copy, and the id fetch is a scalar load from the
+// argument block, which every workgroup of the launch shares. 0xFFFFFFFF marks an id to skip.
+struct InlineIds {
+  uint32_t id[EMM_MAX_INLINE_IDS];
+};
+struct NoIds {};
+
 constexpr int kPack = 0, kUnpack = 1, kPoolToPool = 2;
 // Launch orders (grid x is always the tile inside a chunk):
 //  plain    y = block, z = plane: walks the transfer buffer linearly.
@@ -213,11 +221,13 @@ constexpr int kOrderPlain = 0, kOrderGrouped = 1, kOrderRuns = 2;
 // idx_a / idx_b: source / destination ids (PAIRS: idx_a holds (src, dst) pairs, idx_b unused).
 // `n` = blocks of this launch (ids and linear buffer already offset to its first block),
 // `order_arg` = log2 of the group size (grouped) or the per-plane rotation of the runs (runs).
-template <typename V, int U, int KIND, int ORDER, bool FULL, bool PAIRS, int POLICY>
+// INLINE: the ids come from `ids` in the argument block (pack / unpack, plain order) instead.
+template <typename V, int U, int KIND, int ORDER, bool FULL, bool PAIRS, int POLICY, bool INLINE = false>
 __global__ __launch_bounds__(kThreads) void emm_block_move_kernel(
     const int64_t *__restrict__ idx_a, const int64_t *__restrict__ idx_b, char *lin,
     int64_t lin_plane_stride, int64_t chunk, uint32_t src_nb, uint32_t dst_nb, uint32_t n,
-    uint32_t order_arg, const PlaneTables<KIND == kPoolToPool ? 2 : 1> tables) {
+    uint32_t order_arg, const PlaneTables<KIND == kPoolToPool ? 2 : 1> tables,
+    const std::conditional_t<INLINE, InlineIds, NoIds> ids) {
   constexpr int64_t TILE = (int64_t)U * kThreads * sizeof(V);
   constexpr bool SRC_POOL = KIND != kUnpack, DST_POOL = KIND != kPack;
   uint32_t pl, j;
@@ -238,7 +248,11 @@ __global__ __launch_bounds__(kThreads) void emm_block_move_kernel(
   }
   // round trip 1: ids and plane bases, all issued before the one wait below
   int64_t sb = 0, db = 0;
-  if constexpr (PAIRS) {
+  if constexpr (INLINE) {
+    static_assert(!INLINE || (KIND != kPoolToPool && ORDER == kOrderPlain && !PAIRS), "inline ids: pack / unpack only");
+    if constexpr (SRC_POOL) sb = ids.id[j];
+    if constexpr (DST_POOL) db = ids.id[j];
+  } else if constexpr (PAIRS) {
     sb = idx_a[2 * (uint64_t)j];
     db = idx_a[2 * (uint64_t)j + 1];
   } else {
@@ -304,10 +318,21 @@ void launch_move_full(const MoveArgs &a, uint32_t n, uint32_t order_arg, dim3 gr
                       const PlaneTables<KIND == kPoolToPool ? 2 : 1> &t, hipStream_t s) {
   if (full)
     emm_block_move_kernel<V, U, KIND, ORDER, true, PAIRS, POLICY><<<grid, kThreads, 0, s>>>(
-        a.idx_a, a.idx_b, a.lin, a.lin_plane_stride, a.chunk, a.src_nb, a.dst_nb, n, order_arg, t);
+        a.idx_a, a.idx_b, a.lin, a.lin_plane_stride, a.chunk, a.src_nb, a.dst_nb, n, order_arg, t, NoIds{});
   else
     emm_block_move_kernel<V, U, KIND, ORDER, false, PAIRS, POLICY><<<grid, kThreads, 0, s>>>(
-        a.idx_a, a.idx_b, a.lin, a.lin_plane_stride, a.chunk, a.src_nb, a.dst_nb, n, order_arg, t);
+        a.idx_a, a.idx_b, a.lin, a.lin_plane_stride, a.chunk, a.src_nb, a.dst_nb, n, order_arg, t, NoIds{});
+}
+
+template <typename V, int U, int KIND, int POLICY>
+void launch_move_inline(const MoveArgs &a, uint32_t n, dim3 grid, bool full, const PlaneTables<1> &t,
+                        const InlineIds &ids, hipStream_t s) {
+  if (full)
+    emm_block_move_kernel<V, U, KIND, kOrderPlain, true, false, POLICY, true><<<grid, kThreads, 0, s>>>(
+        nullptr, nullptr, a.lin, a.lin_plane_stride, a.chunk, a.src_nb, a.dst_nb, n, 0, t, ids);
+  else
+    emm_block_move_kernel<V, U, KIND, kOrderPlain, false, false, POLICY, true><<<grid, kThreads, 0, s>>>(
+        nullptr, nullptr, a.lin, a.lin_plane_stride, a.chunk, a.src_nb, a.dst_nb, n, 0, t, ids);
 }
 
 template <int KIND, int ORDER, bool PAIRS>
@@ -351,9 +376,15 @@ template <int KIND>
 int move_planes(const void *const *src_layers, int64_t src_nb, void *const *dst_layers,
                 int64_t dst_nb, int num_layers, int num_kv, int64_t chunk,
                 const int64_t *idx_a, const int64_t *idx_b, bool pairs, int64_t n,
-                const void *linear, hipStream_t s, const char *what) {
+                const void *linear, hipStream_t s, const char *what, const int64_t *host_ids = nullptr) {
   constexpr bool SP = KIND != kUnpack, DP = KIND != kPack;
   if (n == 0 || num_layers == 0 || num_kv == 0 || chunk == 0) return EMM_OK;
+  InlineIds inline_ids;
+  if (host_ids) { // ids travel in the argument block; what the device path would skip becomes the skip mark
+    const int64_t nb = SP ? src_nb : dst_nb;
+    for (int64_t j = 0; j < n; ++j)
+      inline_ids.id[j] = (host_ids[j] >= 0 && host_ids[j] < nb) ? (uint32_t)host_ids[j] : 0xffffffffu;
+  }
   int al = 16;
   if (KIND != kPoolToPool) al = common_align(al, linear);
   for (int l = 0; l < num_layers; ++l) {
@@ -391,6 +422,18 @@ int move_planes(const void *const *src_layers, int64_t src_nb, void *const *dst_
       a.chunk = chunk;
       a.src_nb = (uint32_t)src_nb;
       a.dst_nb = (uint32_t)dst_nb;
+      if constexpr (KIND != kPoolToPool) {
+        if (host_ids) { // n <= EMM_MAX_INLINE_IDS: one launch, plain order
+          const dim3 grid((uint32_t)tpc, (uint32_t)ny, (uint32_t)cnt);
+          if (vec == 16) launch_move_inline<u32x4, 1, KIND, 1>(a, (uint32_t)ny, grid, full, t, inline_ids, s);
+          else if (vec == 4) launch_move_inline<uint32_t, 4, KIND, 0>(a, (uint32_t)ny, grid, false, t, inline_ids, s);
+          else if (vec == 2) launch_move_inline<uint16_t, 4, KIND, 0>(a, (uint32_t)ny, grid, false, t, inline_ids, s);
+          else launch_move_inline<uint8_t, 4, KIND, 0>(a, (uint32_t)ny, grid, false, t, inline_ids, s);
+          const int rc = check_launch(what);
+          if (rc != EMM_OK) return rc;
+          continue;
+        }
+      }
       if constexpr (KIND == kPoolToPool) {
         const uint32_t runs = (uint32_t)((ny + kRun - 1) / kRun);
         const dim3 grid((uint32_t)tpc, (uint32_t)(cnt * kRun), runs);
@@ -619,56 +662,49 @@ __device__ __forceinline__ u32x4 dequant8(u32x2 in, float scale) {
 // ----------------------------------------------------------------------------
 // dequant-unpack: fp8 transfer buffer -> 16-bit pool
 // ----------------------------------------------------------------------------
-struct DequantParams {
-  char *dst_layers[EMM_MAX_LAYERS];
-  const char *packed;
-  const int64_t *dst_idx;
-  const float *k_scales;
-  const float *v_scales;
-  int64_t dst_num_blocks;
-  int64_t chunk_elems; // fp8 bytes per chunk == elements
-  int64_t n;     // blocks per plane of the transfer buffer
-  int64_t j0;    // first block of this launch
-  int64_t j_end; // one past its last block
-  int32_t group_log2;
+struct LayerTable {
+  char *base[EMM_MAX_LAYERS];
 };
 
 // One workgroup converts one tile of 4 KiB of fp8 bytes into 8 KiB. A wave owns 1 KiB of
 // input: lane i loads bytes [8i, 8i+8) and [512+8i, 512+8i+8) and stores the two 16-byte
 // results at twice those offsets, so that every load instruction covers 512 contiguous bytes
-// and every store instruction 1 KiB of whole cache lines.
-// grid: x = tiles per chunk, y = blocks (at most kMaxGridY per launch), z = 2 * layers.
-template <int OUT_DTYPE>
-__global__ __launch_bounds__(kThreads) void emm_unpack_dequant_fp8_kernel(const DequantParams p) {
-  constexpr int64_t TILE = (int64_t)kThreads * 16;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  uint32_t pl;
-  int64_t j;
-  if (p.group_log2 > 0) { // long tables: groups of blocks per plane visit, as in the plain unpack
-    pl = blockIdx.y >> p.group_log2;
-    j = p.j0 + ((int64_t)blockIdx.z << p.group_log2) + (blockIdx.y & ((1u << p.group_log2) - 1));
-    if (j >= p.j_end) return;
+// and every store instruction 1 KiB of whole cache lines. Scalar arguments are explicit and
+// ordered by first use (preloaded into scalar registers); the source does not depend on the
+// block id, so it is loaded first and id, layer base and scale are waited for once.
+// grid: x = tiles per chunk, y = blocks, z = 2 * layers (plain order), or the grouped order
+// of the long unpack (GROUPED: y = plane * 2^g + position, z = group).
+template <int OUT_DTYPE, bool GROUPED>
+__global__ __launch_bounds__(kThreads) void emm_unpack_dequant_fp8_kernel(
+    const char *__restrict__ packed, const int64_t *__restrict__ dst_idx, const float *__restrict__ k_scales,
+    const float *__restrict__ v_scales, int64_t plane_stride /* n * chunk */, uint32_t chunk, uint32_t dst_nb,
+    uint32_t n, uint32_t group_log2, const LayerTable layers) {
+  constexpr uint32_t TILE = kThreads * 16;
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint32_t pl, j;
+  if constexpr (GROUPED) {
+    pl = blockIdx.y >> group_log2;
+    j = (blockIdx.z << group_log2) + (blockIdx.y & ((1u << group_log2) - 1u));
+    if (j >= n) return;
   } else {
     pl = blockIdx.z;
-    j = p.j0 + blockIdx.y;
+    j = blockIdx.y;
   }
   const uint32_t l = pl >> 1, kv = pl & 1;
-  const int64_t chunk = p.chunk_elems;
-  const int64_t off0 = (int64_t)blockIdx.x * TILE + wave * 1024 + lane * 8;
-  const int64_t off1 = off0 + 512;
+  const uint32_t off0 = blockIdx.x * TILE + wave * 1024 + lane * 8;
+  const uint32_t off1 = off0 + 512;
   const bool live0 = off0 < chunk, live1 = off1 < chunk; // chunk is a multiple of 16
-  char *dst_layer = p.dst_layers[l];
-  const float scale = kv == 0 ? p.k_scales[l] : p.v_scales[l];
-  // the source does not depend on the block id: load first, then wait for the id
-  const char *src = p.packed + ((int64_t)pl * p.n + j) * chunk;
+  const char *src = packed + (int64_t)pl * plane_stride + (uint64_t)j * chunk;
   const u32x2 a = ld<u32x2, true>(src + (live0 ? off0 : 0));
   const u32x2 c = ld<u32x2, true>(src + (live1 ? off1 : 0));
-  int64_t b = p.dst_idx[j];
-  asm volatile("" : "+s"(b) : : "memory");
-  if ((uint64_t)b >= (uint64_t)p.dst_num_blocks) return;
-  char *dst = dst_layer + ((int64_t)kv * p.dst_num_blocks + b) * chunk * 2;
-  if (live0) st_stream<u32x4, 1>(dst + off0 * 2, dequant8<OUT_DTYPE>(a, scale));
-  if (live1) st_stream<u32x4, 1>(dst + off1 * 2, dequant8<OUT_DTYPE>(c, scale));
+  int64_t b = dst_idx[j];
+  char *dst_layer = layers.base[l];
+  float scale = kv == 0 ? k_scales[l] : v_scales[l];
+  asm volatile("" : "+s"(b), "+s"(dst_layer), "+s"(scale) : : "memory");
+  if ((uint64_t)b >= (uint64_t)dst_nb) return;
+  char *dst = dst_layer + ((uint64_t)kv * dst_nb + (uint64_t)b) * chunk * 2;
+  if (live0) st_stream<u32x4, 1>(dst + (uint64_t)off0 * 2, dequant8<OUT_DTYPE>(a, scale));
+  if (live1) st_stream<u32x4, 1>(dst + (uint64_t)off1 * 2, dequant8<OUT_DTYPE>(c, scale));
 }
 
 // ----------------------------------------------------------------------------
@@ -1439,6 +1475,32 @@ int emm_kv_unpack(void *const *layer_ptrs, int num_layers, int num_kv,
                               nullptr, block_idx, false, n, packed, as_stream(stream), "emm_kv_unpack");
 }
 
+int emm_kv_pack_host_ids(const void *const *layer_ptrs, int num_layers, int num_kv,
+                         int64_t num_blocks, int64_t chunk_bytes, const int64_t *host_block_idx,
+                         int64_t n, void *packed, emm_stream_t stream) {
+  const char *what = "emm_kv_pack_host_ids";
+  int rc = check_pool_args(what, layer_ptrs, num_layers, num_kv, num_blocks, chunk_bytes, n);
+  if (rc != EMM_OK) return rc;
+  if (n > EMM_MAX_INLINE_IDS) return fail(EMM_EINVAL, "%s: n=%lld exceeds EMM_MAX_INLINE_IDS=%d", what, (long long)n, EMM_MAX_INLINE_IDS);
+  if (n == 0 || num_layers == 0 || num_kv == 0 || chunk_bytes == 0) return EMM_OK;
+  if (!host_block_idx || !packed) return fail(EMM_EINVAL, "%s: null host_block_idx / packed", what);
+  return move_planes<kPack>(layer_ptrs, num_blocks, nullptr, 0, num_layers, num_kv, chunk_bytes,
+                            nullptr, nullptr, false, n, packed, as_stream(stream), what, host_block_idx);
+}
+
+int emm_kv_unpack_host_ids(void *const *layer_ptrs, int num_layers, int num_kv,
+                           int64_t num_blocks, int64_t chunk_bytes, const int64_t *host_block_idx,
+                           int64_t n, const void *packed, emm_stream_t stream) {
+  const char *what = "emm_kv_unpack_host_ids";
+  int rc = check_pool_args(what, (const void *const *)layer_ptrs, num_layers, num_kv, num_blocks, chunk_bytes, n);
+  if (rc != EMM_OK) return rc;
+  if (n > EMM_MAX_INLINE_IDS) return fail(EMM_EINVAL, "%s: n=%lld exceeds EMM_MAX_INLINE_IDS=%d", what, (long long)n, EMM_MAX_INLINE_IDS);
+  if (n == 0 || num_layers == 0 || num_kv == 0 || chunk_bytes == 0) return EMM_OK;
+  if (!host_block_idx || !packed) return fail(EMM_EINVAL, "%s: null host_block_idx / packed", what);
+  return move_planes<kUnpack>(nullptr, 0, layer_ptrs, num_blocks, num_layers, num_kv, chunk_bytes,
+                              nullptr, nullptr, false, n, packed, as_stream(stream), what, host_block_idx);
+}
+
 int emm_copy_blocks(void *const *layer_ptrs, int num_layers, int num_kv,
                     int64_t num_blocks, int64_t chunk_bytes,
                     const int64_t *block_mapping, int64_t num_pairs, emm_stream_t stream) {
@@ -1508,37 +1570,31 @@ int emm_kv_unpack_dequant_fp8(void *const *layer_ptrs, int num_layers, int64_t n
   if (chunk_elems % 16 != 0 || !aligned(packed_fp8, 16))
     return fail(EMM_EINVAL, "%s: chunk_elems (%lld) and packed_fp8 must be multiples of 16",
                 what, (long long)chunk_elems);
-  DequantParams p;
-  memset(&p, 0, sizeof(p));
+  if (chunk_elems > 0x3fffffffLL || num_blocks > 0x7fffffffLL)
+    return fail(EMM_EINVAL, "%s: chunk_elems / num_blocks too large", what);
+  LayerTable t;
   for (int l = 0; l < num_layers; ++l) {
     if (!aligned(layer_ptrs[l], 16))
       return fail(EMM_EINVAL, "%s: layer_ptrs[%d] not 16-byte aligned", what, l);
-    p.dst_layers[l] = (char *)layer_ptrs[l];
+    t.base[l] = (char *)layer_ptrs[l];
   }
-  p.packed = (const char *)packed_fp8;
-  p.dst_idx = block_idx;
-  p.k_scales = k_scales;
-  p.v_scales = v_scales;
-  p.dst_num_blocks = num_blocks;
-  p.chunk_elems = chunk_elems;
-  p.n = n;
   const int64_t tile = (int64_t)kThreads * 16;
   const int64_t tpc = (chunk_elems + tile - 1) / tile;
-  if (tpc > 0x7fffffffLL) return fail(EMM_EINVAL, "%s: grid too large", what);
+  hipStream_t s = as_stream(stream);
   for (int64_t j0 = 0; j0 < n; j0 += kMaxGridY) {
     const int64_t ny = (n - j0 < kMaxGridY) ? (n - j0) : kMaxGridY;
-    p.j0 = j0;
-    p.j_end = j0 + ny;
-    p.group_log2 = 0;
-    dim3 grid((uint32_t)tpc, (uint32_t)ny, (uint32_t)(2 * num_layers));
-    if (ny >= 1024 && ((2 * num_layers) << 7) <= kMaxGridY) {
-      p.group_log2 = 7;
-      grid = dim3((uint32_t)tpc, (uint32_t)((2 * num_layers) << 7), (uint32_t)((ny + 127) >> 7));
-    }
-    if (out_dtype == EMM_DTYPE_BF16)
-      emm_unpack_dequant_fp8_kernel<EMM_DTYPE_BF16><<<grid, kThreads, 0, as_stream(stream)>>>(p);
-    else
-      emm_unpack_dequant_fp8_kernel<EMM_DTYPE_F16><<<grid, kThreads, 0, as_stream(stream)>>>(p);
+    const char *packed = (const char *)packed_fp8 + j0 * chunk_elems;
+    const int64_t *idx = block_idx + j0;
+    const int64_t stride = n * chunk_elems;
+    const bool grouped = ny >= 1024 && ((2 * num_layers) << 7) <= kMaxGridY;
+    const dim3 grid = grouped ? dim3((uint32_t)tpc, (uint32_t)((2 * num_layers) << 7), (uint32_t)((ny + 127) >> 7))
+                              : dim3((uint32_t)tpc, (uint32_t)ny, (uint32_t)(2 * num_layers));
+#define EMM_DQ_LAUNCH(DT, G) \
+  emm_unpack_dequant_fp8_kernel<DT, G><<<grid, kThreads, 0, s>>>(packed, idx, k_scales, v_scales, stride, \
+      (uint32_t)chunk_elems, (uint32_t)num_blocks, (uint32_t)ny, 7u, t)
+    if (out_dtype == EMM_DTYPE_BF16) { if (grouped) EMM_DQ_LAUNCH(EMM_DTYPE_BF16, true); else EMM_DQ_LAUNCH(EMM_DTYPE_BF16, false); }
+    else { if (grouped) EMM_DQ_LAUNCH(EMM_DTYPE_F16, true); else EMM_DQ_LAUNCH(EMM_DTYPE_F16, false); }
+#undef EMM_DQ_LAUNCH
     const int rc2 = check_launch(what);
     if (rc2 != EMM_OK) return rc2;
   }

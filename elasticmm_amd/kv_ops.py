@@ -12,7 +12,8 @@ import numpy as np
 import torch
 
 from . import _lib
-from ._lib import (EMM_DTYPE_BF16, EMM_DTYPE_F16, EMM_FP8_SATURATE, EMM_MAX_LAYERS, EMM_MAX_SEGMENTS, check,
+from ._lib import (EMM_DTYPE_BF16, EMM_DTYPE_F16, EMM_FP8_SATURATE, EMM_MAX_INLINE_IDS, EMM_MAX_LAYERS,
+                   EMM_MAX_SEGMENTS, check,
                    ptr_table)
 
 IndexLike = Union[Sequence[int], np.ndarray, torch.Tensor]
@@ -33,26 +34,21 @@ def _require_gpu(t: torch.Tensor, what: str) -> None:
         raise RuntimeError(f"{what}: tensor is on {t.device}; the KV kernels run on the GPU only")
 
 
-def block_index_tensor(block_indices: IndexLike, num_blocks: int, device: torch.device) -> torch.Tensor:
-    """int64 device tensor of block ids.
-
-    A Python list / numpy array is checked on the host with the semantics torch
-    gives ``tensor[:, idx]`` (worker.py:597, :604): ids in [-num_blocks,
-    num_blocks), negatives counted from the end, anything else IndexError. It is
-    then staged through pinned memory and copied asynchronously. A device tensor
-    is used as is (int64, contiguous); the kernels skip negative or too-large
-    entries instead of faulting.
-    """
+def host_block_ids(block_indices: IndexLike, num_blocks: int) -> Optional[np.ndarray]:
+    """Block ids held on the host (Python list, numpy array, CPU tensor) as a contiguous int64 array,
+    checked with the semantics torch gives ``tensor[:, idx]`` (worker.py:597, :604): ids in
+    [-num_blocks, num_blocks), negatives counted from the end, anything else IndexError.
+    None for a device tensor."""
     if isinstance(block_indices, torch.Tensor):
         t = block_indices
         if t.dtype != torch.long:
             raise TypeError(f"block index tensor must be int64, got {t.dtype}")
         if t.is_cuda:
-            return t.contiguous()
+            return None
         arr = t.numpy()
     else:
         arr = np.asarray(block_indices, dtype=np.int64)
-    arr = arr.reshape(-1)
+    arr = np.ascontiguousarray(arr.reshape(-1))
     if arr.size:
         lo, hi = int(arr.min()), int(arr.max())
         if lo < -num_blocks or hi >= num_blocks:
@@ -60,7 +56,20 @@ def block_index_tensor(block_indices: IndexLike, num_blocks: int, device: torch.
             raise IndexError(f"index {bad} is out of bounds for dimension 1 with size {num_blocks}")
         if lo < 0:
             arr = np.where(arr < 0, arr + num_blocks, arr)
-    host = torch.from_numpy(np.ascontiguousarray(arr))
+    return arr
+
+
+def block_index_tensor(block_indices: IndexLike, num_blocks: int, device: torch.device) -> torch.Tensor:
+    """int64 device tensor of block ids.
+
+    Host ids are checked (``host_block_ids``), staged through pinned memory and copied
+    asynchronously. A device tensor is used as is (int64, contiguous); the kernels skip
+    negative or too-large entries instead of faulting.
+    """
+    arr = host_block_ids(block_indices, num_blocks)
+    if arr is None:
+        return block_indices.contiguous()
+    host = torch.from_numpy(arr)
     if device.type == "cuda":
         return host.pin_memory().to(device, non_blocking=True)
     return host
@@ -130,8 +139,13 @@ class PoolView:
 def kv_pack(pool: PoolView, block_indices: IndexLike, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Gather ``n`` blocks of every layer into ``[L, num_kv, n, *block_shape]``."""
     lib = _lib.load()
-    idx = block_index_tensor(block_indices, pool.num_blocks, pool.device)
-    n = idx.numel()
+    # a table of up to EMM_MAX_INLINE_IDS ids held on the host (the reference's List[int]) travels in the
+    # kernel argument block: no staging, no host-to-device copy
+    host = host_block_ids(block_indices, pool.num_blocks)
+    inline = host is not None and host.size <= EMM_MAX_INLINE_IDS and not pool.on_host
+    idx = None if inline else block_index_tensor(host if host is not None else block_indices, pool.num_blocks,
+                                                 pool.device)
+    n = host.size if inline else idx.numel()
     shape = pool.packed_shape(n)
     if out is None:
         out = torch.empty(shape, dtype=pool.dtype, device=pool.device)
@@ -142,8 +156,13 @@ def kv_pack(pool: PoolView, block_indices: IndexLike, out: Optional[torch.Tensor
     stream = _stream_ptr(pool.device)
     plane = pool.num_kv * n * pool.chunk_bytes
     for l0, table in pool.layer_groups():
-        check(lib.emm_kv_pack(table, len(table), pool.num_kv, pool.num_blocks, pool.chunk_bytes,
-                              idx.data_ptr(), n, out.data_ptr() + l0 * plane, stream), "emm_kv_pack")
+        if inline:
+            check(lib.emm_kv_pack_host_ids(table, len(table), pool.num_kv, pool.num_blocks, pool.chunk_bytes,
+                                           host.ctypes.data, n, out.data_ptr() + l0 * plane, stream),
+                  "emm_kv_pack_host_ids")
+        else:
+            check(lib.emm_kv_pack(table, len(table), pool.num_kv, pool.num_blocks, pool.chunk_bytes,
+                                  idx.data_ptr(), n, out.data_ptr() + l0 * plane, stream), "emm_kv_pack")
     return out
 
 
@@ -151,8 +170,11 @@ def kv_unpack(pool: PoolView, block_indices: IndexLike, packed: torch.Tensor) ->
     """Scatter ``packed`` ``[L, num_kv, n, ...]`` into the pool under ``block_indices``."""
     lib = _lib.load()
     _require_gpu(packed, "kv_unpack")
-    idx = block_index_tensor(block_indices, pool.num_blocks, pool.device)
-    n = idx.numel()
+    host = host_block_ids(block_indices, pool.num_blocks)
+    inline = host is not None and host.size <= EMM_MAX_INLINE_IDS and not pool.on_host
+    idx = None if inline else block_index_tensor(host if host is not None else block_indices, pool.num_blocks,
+                                                 pool.device)
+    n = host.size if inline else idx.numel()
     want = pool.num_layers * pool.num_kv * n * pool.chunk_bytes
     if packed.device != pool.device:
         raise ValueError("kv_unpack: packed buffer is on another device")
@@ -164,8 +186,13 @@ def kv_unpack(pool: PoolView, block_indices: IndexLike, packed: torch.Tensor) ->
     stream = _stream_ptr(pool.device)
     plane = pool.num_kv * n * pool.chunk_bytes
     for l0, table in pool.layer_groups():
-        check(lib.emm_kv_unpack(table, len(table), pool.num_kv, pool.num_blocks, pool.chunk_bytes,
-                                idx.data_ptr(), n, packed.data_ptr() + l0 * plane, stream), "emm_kv_unpack")
+        if inline:
+            check(lib.emm_kv_unpack_host_ids(table, len(table), pool.num_kv, pool.num_blocks, pool.chunk_bytes,
+                                             host.ctypes.data, n, packed.data_ptr() + l0 * plane, stream),
+                  "emm_kv_unpack_host_ids")
+        else:
+            check(lib.emm_kv_unpack(table, len(table), pool.num_kv, pool.num_blocks, pool.chunk_bytes,
+                                    idx.data_ptr(), n, packed.data_ptr() + l0 * plane, stream), "emm_kv_unpack")
 
 
 def kv_migrate(src: PoolView, src_indices: IndexLike, dst: PoolView, dst_indices: IndexLike) -> None:
