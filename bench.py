@@ -647,10 +647,21 @@ def append_bench(kv, NB, bs, H, D, k_scales, v_scales, dev, T=8448):
             kv_ops.stream_copy(srcs[l], dsts[l])
 
     med, _ = timed(graphed(copies).replay, 20)
+    from elasticmm_amd import _lib
+    hooks = _lib.load_hooks()
+
+    def empties():
+        stream = torch.cuda.current_stream().cuda_stream
+        for _ in range(L):
+            hooks.emm_hook_empty_launch(stream)
+
+    med_e, _ = timed(graphed(empties).replay, 20)
     res["launch_bound_yardsticks"] = {
         "plain_copy_of_one_layers_bytes_per_launch_hip_graph": rec(2 * half * L, med, L, "emm_stream_copy_kernel"),
-        "note": "a chain of L dependent launches moving one layer's bytes each, no slot indirection: the per-layer "
-                "append cannot be faster than this on this machine"}
+        "empty_kernel_per_launch_hip_graph_us": round(med_e * 1e3 / L, 2),
+        "note": "chains of L dependent launches replayed from a HIP graph: a plain copy of one layer's bytes per launch "
+                "(no slot indirection) and a kernel that does nothing; the per-layer append cannot be faster than the "
+                "first, and no chain of launches than the second plus the bytes at copy speed"}
     return res
 
 

@@ -55,6 +55,7 @@ SIGNATURES = {
 HOOK_SIGNATURES = {
     "emm_hook_set_move_variant": (c_int, [c_int]),
     "emm_hook_probe": (c_int, [c_int, _PP, c_int, c_int, c_int64, c_int64, _P, c_int64, _P, _P, _P]),
+    "emm_hook_empty_launch": (c_int, [_P]),
     "emm_hook_fp8_quotient_sweep": (c_int, [c_int, c_int, ctypes.c_uint32, ctypes.c_uint32, _P, _P]),
 }
 EMM_PROBE_SEQ_READ, EMM_PROBE_SEQ_WRITE, EMM_PROBE_GATHER_READ, EMM_PROBE_SCATTER_WRITE = 0, 1, 2, 3

@@ -1771,6 +1771,9 @@ __global__ __launch_bounds__(kThreads) void emm_probe_kernel(const int64_t *__re
   }
 }
 
+// A kernel that does nothing: a chain of these measures what a dependent launch costs by itself.
+__global__ void emm_empty_kernel() {}
+
 // The fast quotient against the division for one exponent pair and a range of scale significands:
 // thread = one scale significand, loop over all 2^10 x significands (the 11 significant bits of an
 // f16; bf16 values are the subset with 3 more trailing zeros) and both signs.
@@ -1857,6 +1860,11 @@ int emm_hook_probe(int kind, void *const *layer_ptrs, int num_layers, int num_kv
   default: emm_probe_kernel<EMM_PROBE_SCATTER_WRITE><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
   }
   return check_launch(what);
+}
+
+int emm_hook_empty_launch(emm_stream_t stream) {
+  emm_empty_kernel<<<1, 64, 0, as_stream(stream)>>>();
+  return check_launch("emm_hook_empty_launch");
 }
 
 int emm_hook_fp8_quotient_sweep(int x_exp, int s_exp, uint32_t s_begin, uint32_t s_end, uint64_t *counters,

@@ -37,6 +37,10 @@ int emm_hook_probe(int kind, void *const *layer_ptrs, int num_layers, int num_kv
                    int64_t chunk_bytes, const int64_t *block_idx, int64_t n, void *linear, uint32_t *sink,
                    emm_stream_t stream);
 
+/* Launch a kernel that does nothing (one wave): a chain of these in a HIP graph measures the cost of a
+ * dependent launch by itself, the floor under every per-layer launch. */
+int emm_hook_empty_launch(emm_stream_t stream);
+
 /* Exhaustive check of the fp8 append's reciprocal-form quotient: for x = +-1.m * 2^x_exp over all
  * 2^10 ten-bit m and scale = 1.f * 2^s_exp for f in [s_begin, s_end) (23-bit significand fields),
  * compare with the IEEE division. counters (DEVICE, 5 x uint64, zeroed by the caller):
