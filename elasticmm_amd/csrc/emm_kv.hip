@@ -1132,88 +1132,80 @@ int append_strided(const void *const *k, const void *const *v, void *const *kc, 
 // every K group and one element to every V run, so tokens that fill a block in order produce
 // contiguous output; a single token produces 16-byte (K) and element-sized (V) stores at a stride
 // of block_size * 16 bytes resp. block_size elements.
-struct PagedParams {
-  const char *key[EMM_MAX_LAYERS];
-  const char *value[EMM_MAX_LAYERS];
-  char *key_cache[EMM_MAX_LAYERS];
-  char *value_cache[EMM_MAX_LAYERS];
-  const int64_t *slot_mapping;
-  const float *k_scales; // fp8 cache only: one float per layer
-  const float *v_scales;
-  int64_t num_tokens;
-  int64_t row_elems; // num_heads * head_size
-  int64_t key_stride; // elements
-  int64_t value_stride;
-  int64_t num_blocks;
-  int32_t block_size;
-  int32_t vec_src; // 1: sources allow 16-byte loads
-};
-
 constexpr int kPagedTokens = 16; // tokens per tile: the tile owns the runs that start in it
-constexpr int kPagedRows = 32;   // LDS rows: an owned run may reach 15 tokens past the tile
-constexpr int kPagedSeg = 256;   // row elements per tile
+constexpr int kPagedRows = 32;   // token positions a tile looks at: an owned run may reach 15 tokens past the tile
+constexpr int kPagedSeg = 256;   // row elements per workgroup
 
-// One workgroup transposes the rows of up to 31 tokens x up to 256 row elements of K or V.
+// One workgroup handles the rows of up to 31 tokens x up to 256 row elements of K or V.
 //
 // Runs. Consecutive tokens with consecutive slots inside one 16-slot-aligned window of a block
 // form a run (at most 16 tokens). A run belongs to the tile its first token lies in, so a tile
 // of 16 tokens owns runs that may extend up to 15 tokens into the next tile, and leaves the
 // head of a run that started in the previous tile to that tile: prompts written in order give
-// whole 16-token runs no matter where they start in the token list. Wave 0 finds the runs from
-// the 32 slots after the tile start with two ballots and writes a compact list of the owned
-// tokens (block, offset, token) to LDS.
-// Phase 1: coalesced 16-byte loads of the owned source rows (quantised to e4m3fn here when the
-// cache is fp8) into LDS, rows padded by 16 bytes so that a column walk touches every bank once.
-// Phase 2, K: lane q handles (group q / 16, owned token q % 16): one 16-byte LDS read, one
-// 16-byte store; 16 neighbouring lanes cover one group, so a run of n tokens gives n * 16
-// contiguous bytes per group and a whole block 16 KiB.
-// Phase 2, V: for a whole run of 16 tokens (at most one per tile) lane q gathers one 16-byte
-// piece of the run's [element][16 tokens] region from a column of the tile (8 or 16
-// element-sized LDS reads); the other owned tokens are stored one element per lane, token by
-// token (every such store is a partial write of a 32-byte sector, which is what the layout costs
-// for tokens that do not fill a block; the lane order makes no measurable difference).
+// whole 16-token runs no matter where they start in the token list. Wave 0 finds the runs in
+// registers from the 32 slots after the tile start (lane = token position, three ballots) and
+// leaves the result in LDS: where the whole run (16 tokens that fill a 16-slot window; at most
+// one per tile) starts and lands, and a compact list of the other owned tokens. One wave only:
+// the instructions of this step are a visible part of a launch that lasts a few microseconds.
+//
+// Rows. Item q of a round of 16 tokens is (row q / 32, 16-byte source piece q % 32), two per
+// thread, both requested before either is used.
+//  * The whole run goes to LDS (quantised to e4m3fn on the way when the cache is fp8; rows padded
+//    by 16 bytes so that a column walk touches every bank once) and, after a barrier, to the cache.
+//    K: lane q moves (group q / 16, token q % 16), one 16-byte LDS read and one 16-byte store; 16
+//    neighbouring lanes cover one group, a wave instruction 1 KiB of contiguous cache. V: lane q
+//    gathers one 16-byte piece of the run's [element][16 tokens] region from a column of the tile
+//    (8 or 16 element-sized LDS reads).
+//  * Every other owned token (decode tokens, heads and tails of prompts) is stored straight from
+//    the registers, K as 16-byte (fp8 cache: 8-byte) pieces, V element by element. Each such store
+//    is a partial write of a 32-byte sector — what the layout costs for tokens that do not fill a
+//    block — but no barrier and no LDS latency is spent on them.
+// The scalar arguments are explicit and ordered by first use: the 14 dwords up to value_stride
+// arrive preloaded in scalar registers.
 // grid: x = token tiles, y = 2 * row segments (bit 0: K | V), z = layers.
-template <int CE, int SRC_DTYPE, bool SAT>
-__global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(const PagedParams p) {
+template <int CE, int SRC_DTYPE, bool SAT, bool TABLES>
+__global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
+    const int64_t *__restrict__ slot_mapping, const char *key, const char *value, char *key_cache,
+    char *value_cache, uint32_t num_tokens, uint32_t row_elems, uint32_t key_stride, uint32_t value_stride,
+    uint32_t block_size, uint32_t vec_src, int64_t num_blocks, const float *k_scales, const float *v_scales,
+    const std::conditional_t<TABLES, AppendTables, NoTables> tables) {
   constexpr int X = 16 / CE;               // elements per 16-byte piece of the cache
   constexpr int ROW = kPagedSeg * CE + 16; // LDS row stride in bytes
-  __shared__ __attribute__((aligned(16))) char tile[kPagedRows * ROW];
-  __shared__ int64_t s_blk[kPagedRows];
+  constexpr int kPieces = kPagedSeg / 8;   // 16-byte source pieces per full row
+  constexpr int N = kPagedTokens * kPieces / kThreads; // items per thread in a round of 16 tokens
+  __shared__ __attribute__((aligned(16))) char tile[kPagedTokens * ROW];  // the whole run
+  __shared__ __attribute__((aligned(16))) char stage[kPagedTokens * ROW]; // V rows of the other tokens, wave-private
+  __shared__ int64_t s_blk[kPagedRows];                                  // the other owned tokens
   __shared__ int32_t s_off[kPagedRows];
-  __shared__ int32_t s_tok[kPagedRows];
-  __shared__ int32_t s_count; // owned tokens
-  __shared__ int32_t s_whole; // position of the whole run in the owned list, or -1
+  __shared__ int32_t s_pos[kPagedRows];
+  __shared__ int64_t s_wblk; // block and first offset of the whole run
+  __shared__ int32_t s_woff;
+  __shared__ int32_t s_w0;    // token position of the whole run's first token, or -1
+  __shared__ int32_t s_count; // other owned tokens
   const int tid = threadIdx.x;
   const uint32_t kv = blockIdx.y & 1u, seg = blockIdx.y >> 1;
-  const int64_t t0 = (int64_t)blockIdx.x * kPagedTokens;
-  const int64_t e0 = (int64_t)seg * kPagedSeg;
-  const int64_t left = p.row_elems - e0;
-  const int seg_elems = left < kPagedSeg ? (int)left : kPagedSeg; // multiple of X
-  const uint32_t l = blockIdx.z;
-  const char *src = kv == 0 ? p.key[l] : p.value[l];
-  char *cache = kv == 0 ? p.key_cache[l] : p.value_cache[l];
-  const int64_t stride = kv == 0 ? p.key_stride : p.value_stride;
-  const int bs = p.block_size;
+  const uint32_t t0 = blockIdx.x * kPagedTokens;
+  const int bs = (int)block_size;
 
-  float scale = 1.0f;
-  if constexpr (CE == 1) scale = kv == 0 ? p.k_scales[l] : p.v_scales[l];
-  const Divisor div = make_divisor(scale, true);
-
-  // ---- phase 0 (wave 0): runs and the list of owned tokens ----
+  // ---- wave 0: slots, runs, owned tokens ----
   if (tid < 64) {
     const int i = tid;
-    const int64_t t = t0 + i;
     int64_t s = -1, prev = -1;
-    if (i < kPagedRows && t < p.num_tokens) {
-      s = p.slot_mapping[t];
-      if (t > 0) prev = p.slot_mapping[t - 1];
+    if (i < kPagedRows && t0 + i < num_tokens) {
+      s = slot_mapping[t0 + i];
+      if (t0 + i > 0) prev = slot_mapping[t0 + i - 1];
     }
-    const bool valid = s >= 0 && s < p.num_blocks * bs;
+    const bool valid = s >= 0 && s < num_blocks * bs;
     int64_t blk = 0;
     int32_t off = 0;
     if (valid) {
-      blk = s / bs;
-      off = (int32_t)(s - blk * bs);
+      if ((bs & (bs - 1)) == 0) { // wave-uniform
+        blk = s >> __builtin_ctz(bs);
+        off = (int32_t)s & (bs - 1);
+      } else {
+        blk = s / bs;
+        off = (int32_t)(s - blk * bs);
+      }
     }
     const bool cont = valid && s == prev + 1 && (off & 15) != 0; // continues the previous token's run
     const uint64_t starts = __ballot(!cont); // bit j: token j starts a run or is skipped (lanes >= 32: set)
@@ -1221,120 +1213,219 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(const PagedP
     const int head = below ? 63 - __builtin_clzll(below) : -1; // first token of this token's run
     const bool owned = valid && head >= 0 && head < kPagedTokens;
     const uint64_t owned_mask = __ballot(owned);
-    const int k = __builtin_popcountll(owned_mask & ((1ull << i) - 1ull));
-    if (owned) {
-      s_blk[k] = blk;
-      s_off[k] = off;
-      s_tok[k] = i;
-    }
-    // a run of 16 tokens starts at a multiple of 16 slots; its V region is 16-byte aligned if
-    // the block's is
+    // a run of 16 tokens starts at a multiple of 16 slots; its V region is 16-byte aligned if the block's is
     const bool whole = owned && !cont && i < kPagedTokens && ((bs * CE) & 15) == 0 &&
                        __builtin_ctzll(starts >> (i + 1)) + 1 == 16;
     const uint64_t whole_mask = __ballot(whole);
-    if (i == 0) {
-      s_count = __builtin_popcountll(owned_mask);
-      s_whole = whole_mask ? __builtin_popcountll(owned_mask & ((1ull << __builtin_ctzll(whole_mask)) - 1ull)) : -1;
+    const int w0 = whole_mask ? (int)__builtin_ctzll(whole_mask) : -1;
+    const uint64_t other_mask = owned_mask & ~(w0 >= 0 ? 0xffffull << w0 : 0ull);
+    if ((other_mask >> i) & 1ull) {
+      const int r = __builtin_popcountll(other_mask & ((1ull << i) - 1ull));
+      s_blk[r] = blk;
+      s_off[r] = off;
+      s_pos[r] = i;
+    }
+    if (i == (w0 >= 0 ? w0 : 0)) {
+      s_wblk = blk;
+      s_woff = off;
+      s_w0 = w0;
+      s_count = __builtin_popcountll(other_mask);
     }
   }
-  __syncthreads();
-  const int count = s_count;
-  if (count == 0) return;
-
-  // ---- phase 1: owned source rows into LDS ----
-  if (p.vec_src) {
-    const int pieces = seg_elems >> 3; // 16-byte source pieces per row
-    for (int q = tid; q < count * pieces; q += kThreads) {
-      const int r = q / pieces, c = q - r * pieces;
-      const u32x4 v = ld<u32x4, true>(src + ((t0 + s_tok[r]) * stride + e0 + c * 8) * 2);
-      if constexpr (CE == 2)
-        *reinterpret_cast<u32x4 *>(tile + r * ROW + c * 16) = v;
-      else
-        *reinterpret_cast<u32x2 *>(tile + r * ROW + c * 8) = quant8<SRC_DTYPE, SAT>(v, div);
-    }
-  } else {
-    for (int q = tid; q < count * seg_elems; q += kThreads) {
-      const int r = q / seg_elems, c = q - r * seg_elems;
-      const uint16_t h = ld<uint16_t, false>(src + ((t0 + s_tok[r]) * stride + e0 + c) * 2);
-      if constexpr (CE == 2)
-        *reinterpret_cast<uint16_t *>(tile + r * ROW + c * 2) = h;
-      else
-        *reinterpret_cast<uint8_t *>(tile + r * ROW + c) = quant1<SRC_DTYPE, SAT>(h, scale);
-    }
+  if constexpr (TABLES) {
+    const uint32_t l = blockIdx.z;
+    key = tables.key[l];
+    value = tables.value[l];
+    key_cache = tables.key_cache[l];
+    value_cache = tables.value_cache[l];
   }
+  const uint32_t e0 = seg * kPagedSeg;
+  const uint32_t left = row_elems - e0;
+  const int seg_elems = left < kPagedSeg ? (int)left : kPagedSeg; // multiple of X
+  const int pieces = seg_elems >> 3;
+  const char *src = kv == 0 ? key : value;
+  char *cache = kv == 0 ? key_cache : value_cache;
+  const uint32_t stride = kv == 0 ? key_stride : value_stride;
+  const int64_t groups_per_block = row_elems / X;
+  float scale = 1.0f;
+  if constexpr (CE == 1) scale = kv == 0 ? k_scales[blockIdx.z] : v_scales[blockIdx.z];
+  const Divisor div = make_divisor(scale, true);
   __syncthreads();
+  const int w0 = s_w0, count = s_count;
+  if (w0 < 0 && count == 0) return;
+  const int c = tid % kPieces < pieces ? tid % kPieces : 0; // lanes past the row re-read its start; nothing of theirs is stored
+  const bool live = tid % kPieces < pieces;
+  const int row0 = tid / kPieces; // rows of the thread's items in a round: row0 + 8 * it
 
-  if (kv == 0) {
-    // ---- K: 16-byte pieces, token fastest ----
-    const int groups = seg_elems / X;
-    const int64_t g0 = e0 / X, groups_per_block = p.row_elems / X;
-    for (int base = 0; base < count; base += 16) {
-      for (int q = tid; q < groups * 16; q += kThreads) {
-        const int g = q >> 4, r = base + (q & 15);
-        if (r >= count) continue;
-        const u32x4 v = *reinterpret_cast<const u32x4 *>(tile + r * ROW + g * 16);
-        char *dst = cache + ((s_blk[r] * groups_per_block + g0 + g) * bs + s_off[r]) * 16;
-        st_stream<u32x4, 1>(dst, v);
+  // One element of a source row that does not allow 16-byte loads, converted for the cache.
+  auto slow_elem = [&](int pos, int e) -> uint32_t {
+    const uint16_t h = ld<uint16_t, false>(src + ((uint64_t)(t0 + pos) * stride + e0 + e) * 2);
+    if constexpr (CE == 1) return quant1<SRC_DTYPE, SAT>(h, scale);
+    return h;
+  };
+
+  // ---- the whole run -> LDS ----
+  if (w0 >= 0) {
+    if (vec_src) {
+      // one row after the other (the second request goes out when the first row has arrived): a launch for one
+      // layer has every workgroup in the same phase, and spreading the requests measured faster than bunching them
+#pragma unroll
+      for (int it = 0; it < N; ++it) {
+        u32x4 v = ld<u32x4, true>(src + ((uint64_t)(t0 + w0 + row0 + 8 * it) * stride + e0 + c * 8) * 2);
+        asm volatile("" : "+v"(v));
+        if (live) {
+          char *dst = tile + (row0 + 8 * it) * ROW;
+          if constexpr (CE == 2)
+            *reinterpret_cast<u32x4 *>(dst + (tid % kPieces) * 16) = v;
+          else
+            *reinterpret_cast<u32x2 *>(dst + (tid % kPieces) * 8) = quant8<SRC_DTYPE, SAT>(v, div);
+        }
       }
+    } else {
+      for (int r = 0; r < kPagedTokens; ++r)
+        for (int e = tid; e < seg_elems; e += kThreads) {
+          const uint32_t a = slow_elem(w0 + r, e);
+          if constexpr (CE == 2)
+            *reinterpret_cast<uint16_t *>(tile + r * ROW + e * 2) = (uint16_t)a;
+          else
+            *reinterpret_cast<uint8_t *>(tile + r * ROW + e) = (uint8_t)a;
+        }
+    }
+  }
+
+  // ---- the other owned tokens: straight from the registers, 16 tokens per round ----
+  for (int base = 0; base < count; base += kPagedTokens) {
+    if (vec_src) {
+      u32x4 v[N];
+      int64_t dblk[N];
+      int doff[N];
+#pragma unroll
+      for (int it = 0; it < N; ++it) {
+        const int r = base + row0 + 8 * it;
+        const int rc = r < count ? r : count - 1; // rows past the list re-read its last row
+        dblk[it] = s_blk[rc];
+        doff[it] = s_off[rc];
+        v[it] = ld<u32x4, true>(src + ((uint64_t)(t0 + s_pos[rc]) * stride + e0 + c * 8) * 2);
+      }
+      // Wait for all rows here: a wait placed after the first item's stores would also wait for those
+      // stores (loads and stores share one in-order counter).
+#pragma unroll
+      for (int it = 0; it < N; ++it) asm volatile("" : "+v"(v[it]));
+#pragma unroll
+      for (int it = 0; it < N; ++it) {
+        if (base + row0 + 8 * it >= count || !live) continue;
+        const uint32_t e = e0 + (tid % kPieces) * 8; // first element of the piece
+        u32x2 q8{0, 0};
+        if constexpr (CE == 1) q8 = quant8<SRC_DTYPE, SAT>(v[it], div);
+        if (kv == 0) {
+          char *dst = cache + ((dblk[it] * groups_per_block + e / X) * bs + doff[it]) * 16;
+          if constexpr (CE == 2)
+            st_stream<u32x4, 1>(dst, v[it]);
+          else
+            st<u32x2, false>(dst + (e % X), q8);
+        } else {
+          // V: through the wave's own rows of the staging tile, so that a store instruction covers 64
+          // consecutive elements of one token (64 sectors in 16 consecutive lines) instead of every eighth
+          char *dst = stage + (row0 + 8 * it) * ROW;
+          if constexpr (CE == 2)
+            *reinterpret_cast<u32x4 *>(dst + (tid % kPieces) * 16) = v[it];
+          else
+            *reinterpret_cast<u32x2 *>(dst + (tid % kPieces) * 8) = q8;
+        }
+      }
+      if (kv == 1) {
+        // rows row0 + 8 * it of lanes 0-31 and 32-63: the wave wrote them itself, LDS keeps a wave's order
+        __builtin_amdgcn_wave_barrier();
+        const int lane = tid & 63, first = (tid >> 6) * (64 / kPieces);
+#pragma unroll
+        for (int rr = 0; rr < N * (64 / kPieces); ++rr) {
+          const int rl = first + (rr % (64 / kPieces)) + 8 * (rr / (64 / kPieces));
+          if (base + rl >= count) continue;
+          const int64_t rblk = s_blk[base + rl];
+          const int roff = s_off[base + rl];
+          char *dst = cache + ((rblk * row_elems + e0) * bs + roff) * CE;
+#pragma unroll
+          for (int m = 0; m < kPagedSeg / 64; ++m) {
+            const int e = m * 64 + lane;
+            if (e >= seg_elems) continue;
+            if constexpr (CE == 2)
+              st<uint16_t, false>(dst + (int64_t)e * bs * 2, *reinterpret_cast<const uint16_t *>(stage + rl * ROW + e * 2));
+            else
+              st<uint8_t, false>(dst + (int64_t)e * bs, *reinterpret_cast<const uint8_t *>(stage + rl * ROW + e));
+          }
+        }
+        __builtin_amdgcn_wave_barrier(); // the next round overwrites the rows
+      }
+    } else {
+      const int end = base + kPagedTokens < count ? base + kPagedTokens : count;
+      for (int r = base; r < end; ++r) {
+        const int pos = s_pos[r];
+        const int64_t dblk = s_blk[r];
+        const int doff = s_off[r];
+        for (int e = tid; e < seg_elems; e += kThreads) {
+          const uint32_t a = slow_elem(pos, e);
+          const uint32_t ee = e0 + e;
+          char *dst = kv == 0 ? cache + ((dblk * groups_per_block + ee / X) * bs + doff) * 16 + (ee % X) * CE
+                              : cache + ((dblk * row_elems + ee) * bs + doff) * CE;
+          if constexpr (CE == 2)
+            st<uint16_t, false>(dst, (uint16_t)a);
+          else
+            st<uint8_t, false>(dst, (uint8_t)a);
+        }
+      }
+    }
+  }
+  if (w0 < 0) return; // no whole run in this tile (the same in every wave)
+
+  __syncthreads();
+  const int64_t wblk = s_wblk;
+  const int woff = s_woff;
+  if (kv == 0) {
+    // ---- K, whole run: 16-byte pieces, token fastest ----
+    const int groups = seg_elems / X;
+    const int64_t g0 = e0 / X;
+    for (int q = tid; q < groups * 16; q += kThreads) {
+      const int g = q >> 4, r = q & 15;
+      const u32x4 v = *reinterpret_cast<const u32x4 *>(tile + r * ROW + g * 16);
+      st_stream<u32x4, 1>(cache + ((wblk * groups_per_block + g0 + g) * bs + woff + r) * 16, v);
     }
     return;
   }
-  const int whole = s_whole;
-  if (whole >= 0) {
-    // ---- V, whole run: 16-byte pieces of the run's [element][16 tokens] region ----
-    const int64_t blk = s_blk[whole];
-    const int off0 = s_off[whole];
-    const char *rows = tile + whole * ROW;
-    if constexpr (CE == 2) {
-      // Lanes 0-31 of a wave gather tokens 0-7 of 32 consecutive elements, lanes 32-63 tokens 8-15 of
-      // the same elements: the two half-waves read different tile rows at the same column (the same
-      // LDS banks) in different passes, and one store instruction still covers the 32 elements'
-      // 1 KiB of output completely.
-      const int lane = tid & 63, half = lane >> 5;
-      for (int q0 = (tid >> 6) * 32; q0 < seg_elems; q0 += (kThreads >> 6) * 32) {
-        const int e = q0 + (lane & 31);
-        if (e >= seg_elems) continue;
-        const char *col = rows + half * 8 * ROW + e * 2;
-        uint32_t w[4];
+  // ---- V, whole run: 16-byte pieces of the run's [element][16 tokens] region ----
+  if constexpr (CE == 2) {
+    // Lanes 0-31 of a wave gather tokens 0-7 of 32 consecutive elements, lanes 32-63 tokens 8-15 of
+    // the same elements: the two half-waves read different tile rows at the same column (the same
+    // LDS banks) in different passes, and one store instruction still covers the 32 elements'
+    // 1 KiB of output completely.
+    const int lane = tid & 63, half = lane >> 5;
+    for (int q0 = (tid >> 6) * 32; q0 < seg_elems; q0 += (kThreads >> 6) * 32) {
+      const int e = q0 + (lane & 31);
+      if (e >= seg_elems) continue;
+      const char *col = tile + half * 8 * ROW + e * 2;
+      uint32_t w[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const uint32_t lo = *reinterpret_cast<const uint16_t *>(col + (2 * i) * ROW);
-          const uint32_t hi = *reinterpret_cast<const uint16_t *>(col + (2 * i + 1) * ROW);
-          w[i] = lo | (hi << 16);
-        }
-        char *dst = cache + ((blk * p.row_elems + e0 + e) * bs + off0) * 2 + half * 16;
-        st_stream<u32x4, 1>(dst, u32x4{w[0], w[1], w[2], w[3]});
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = *reinterpret_cast<const uint16_t *>(col + (2 * j) * ROW);
+        const uint32_t hi = *reinterpret_cast<const uint16_t *>(col + (2 * j + 1) * ROW);
+        w[j] = lo | (hi << 16);
       }
-    } else {
-      for (int e = tid; e < seg_elems; e += kThreads) {
-        const char *col = rows + e;
-        uint32_t w[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          uint32_t x = 0;
-#pragma unroll
-          for (int k = 0; k < 4; ++k)
-            x |= (uint32_t) * reinterpret_cast<const uint8_t *>(col + (4 * i + k) * ROW) << (8 * k);
-          w[i] = x;
-        }
-        char *dst = cache + ((blk * p.row_elems + e0 + e) * bs + off0);
-        st_stream<u32x4, 1>(dst, u32x4{w[0], w[1], w[2], w[3]});
-      }
+      char *dst = cache + ((wblk * row_elems + e0 + e) * bs + woff) * 2 + half * 16;
+      st_stream<u32x4, 1>(dst, u32x4{w[0], w[1], w[2], w[3]});
     }
-  }
-  // ---- V, the other owned tokens: one element per lane, element fastest ----
-  // (a wave instruction covers 64 consecutive elements of one token: 64 sectors in 16 consecutive
-  // cache lines of the block's V region)
-  const int rest = whole >= 0 ? count - 16 : count;
-  for (int i = 0; i < rest; ++i) {
-    const int r = (whole >= 0 && i >= whole) ? i + 16 : i; // step over the whole run
-    char *base = cache + ((s_blk[r] * p.row_elems + e0) * bs + s_off[r]) * CE;
+  } else {
     for (int e = tid; e < seg_elems; e += kThreads) {
-      char *dst = base + (int64_t)e * bs * CE;
-      if constexpr (CE == 2)
-        st<uint16_t, false>(dst, *reinterpret_cast<const uint16_t *>(tile + r * ROW + e * 2));
-      else
-        st<uint8_t, false>(dst, *reinterpret_cast<const uint8_t *>(tile + r * ROW + e));
+      const char *col = tile + e;
+      uint32_t w[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        uint32_t x = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          x |= (uint32_t) * reinterpret_cast<const uint8_t *>(col + (4 * j + k) * ROW) << (8 * k);
+        w[j] = x;
+      }
+      char *dst = cache + ((wblk * row_elems + e0 + e) * bs + woff);
+      st_stream<u32x4, 1>(dst, u32x4{w[0], w[1], w[2], w[3]});
     }
   }
 }
@@ -1366,41 +1457,44 @@ int append_paged(const void *const *k, const void *const *v, void *const *kc, vo
   const int64_t tiles = (num_tokens + kPagedTokens - 1) / kPagedTokens;
   const int64_t segs = (row_elems + kPagedSeg - 1) / kPagedSeg;
   if (tiles > 0x7fffffffLL || segs * 2 > kMaxGridY) return fail(EMM_EINVAL, "%s: too many tokens / too long rows", what);
-  PagedParams p;
-  memset(&p, 0, sizeof(p));
-  p.vec_src = ks % 8 == 0 && vs % 8 == 0;
+  if (num_tokens > 0x7fffffffLL || row_elems > 0x7fffffffLL || ks > 0xffffffffLL || vs > 0xffffffffLL)
+    return fail(EMM_EINVAL, "%s: num_tokens / row / token stride too large", what);
+  const bool tables = num_layers > 1;
+  AppendTables t;
+  uint32_t vec_src = ks % 8 == 0 && vs % 8 == 0;
   for (int l = 0; l < num_layers; ++l) {
     if (!k[l] || !v[l] || !kc[l] || !vc[l]) return fail(EMM_EINVAL, "%s: null tensor pointer at layer %d", what, l);
     if (!aligned(k[l], 2) || !aligned(v[l], 2))
       return fail(EMM_EINVAL, "%s: 16-bit source not 2-byte aligned at layer %d", what, l);
     if (!aligned(kc[l], 16) || !aligned(vc[l], 16))
       return fail(EMM_EINVAL, "%s: cache not 16-byte aligned at layer %d", what, l);
-    if (!aligned(k[l], 16) || !aligned(v[l], 16)) p.vec_src = 0;
-    p.key[l] = (const char *)k[l];
-    p.value[l] = (const char *)v[l];
-    p.key_cache[l] = (char *)kc[l];
-    p.value_cache[l] = (char *)vc[l];
+    if (!aligned(k[l], 16) || !aligned(v[l], 16)) vec_src = 0;
+    if (tables) {
+      t.key[l] = (const char *)k[l];
+      t.value[l] = (const char *)v[l];
+      t.key_cache[l] = (char *)kc[l];
+      t.value_cache[l] = (char *)vc[l];
+    }
   }
-  p.slot_mapping = slot_mapping;
-  p.k_scales = k_scales;
-  p.v_scales = v_scales;
-  p.num_tokens = num_tokens;
-  p.row_elems = row_elems;
-  p.key_stride = ks;
-  p.value_stride = vs;
-  p.num_blocks = num_blocks;
-  p.block_size = block_size;
   const dim3 grid((uint32_t)tiles, (uint32_t)(segs * 2), (uint32_t)num_layers);
-  if (cache_elem_bytes == 2)
-    emm_append_paged_kernel<2, EMM_DTYPE_BF16, false><<<grid, kThreads, 0, s>>>(p);
-  else if (src_dtype == EMM_DTYPE_BF16 && !sat)
-    emm_append_paged_kernel<1, EMM_DTYPE_BF16, false><<<grid, kThreads, 0, s>>>(p);
-  else if (src_dtype == EMM_DTYPE_BF16)
-    emm_append_paged_kernel<1, EMM_DTYPE_BF16, true><<<grid, kThreads, 0, s>>>(p);
-  else if (!sat)
-    emm_append_paged_kernel<1, EMM_DTYPE_F16, false><<<grid, kThreads, 0, s>>>(p);
-  else
-    emm_append_paged_kernel<1, EMM_DTYPE_F16, true><<<grid, kThreads, 0, s>>>(p);
+#define EMM_PAGED_LAUNCH(CE_, DT_, SAT_) \
+  do { \
+    if (tables) \
+      emm_append_paged_kernel<CE_, DT_, SAT_, true><<<grid, kThreads, 0, s>>>( \
+          slot_mapping, nullptr, nullptr, nullptr, nullptr, (uint32_t)num_tokens, (uint32_t)row_elems, (uint32_t)ks, \
+          (uint32_t)vs, (uint32_t)block_size, vec_src, num_blocks, k_scales, v_scales, t); \
+    else \
+      emm_append_paged_kernel<CE_, DT_, SAT_, false><<<grid, kThreads, 0, s>>>( \
+          slot_mapping, (const char *)k[0], (const char *)v[0], (char *)kc[0], (char *)vc[0], (uint32_t)num_tokens, \
+          (uint32_t)row_elems, (uint32_t)ks, (uint32_t)vs, (uint32_t)block_size, vec_src, num_blocks, k_scales, \
+          v_scales, NoTables{}); \
+  } while (0)
+  if (cache_elem_bytes == 2) EMM_PAGED_LAUNCH(2, EMM_DTYPE_BF16, false);
+  else if (src_dtype == EMM_DTYPE_BF16 && !sat) EMM_PAGED_LAUNCH(1, EMM_DTYPE_BF16, false);
+  else if (src_dtype == EMM_DTYPE_BF16) EMM_PAGED_LAUNCH(1, EMM_DTYPE_BF16, true);
+  else if (!sat) EMM_PAGED_LAUNCH(1, EMM_DTYPE_F16, false);
+  else EMM_PAGED_LAUNCH(1, EMM_DTYPE_F16, true);
+#undef EMM_PAGED_LAUNCH
   return check_launch(what);
 }
 
