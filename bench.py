@@ -581,6 +581,21 @@ def paged_append_bench(kv, NB, bs, H, D, dev, T=8448, decode=256):
     med, _ = timed(lambda: dplan(dslots), 20)
     res["decode_only_256_tokens_one_launch"] = rec(L * Td * 2 * H * D * 4, med, 1, "emm_append_paged_kernel",
                                                    tokens_per_s=round(Td / (med * 1e-3)))
+
+    def decode_per_layer():
+        for l in range(L):
+            cache_ops.reshape_and_cache(keys[l][:Td], values[l][:Td], kcs[l], vcs[l], dslots, "auto")
+
+    dgraph = torch.cuda.CUDAGraph()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        decode_per_layer()
+    torch.cuda.current_stream().wait_stream(side)
+    with torch.cuda.graph(dgraph):
+        decode_per_layer()
+    med, _ = timed(dgraph.replay, 20)
+    res["decode_step_256_tokens_per_layer_hip_graph"] = rec(L * Td * 2 * H * D * 4, med, L, "emm_append_paged_kernel",
+                                                            tokens_per_s=round(Td / (med * 1e-3)))
     return res
 
 
@@ -636,6 +651,18 @@ def append_bench(kv, NB, bs, H, D, k_scales, v_scales, dev, T=8448):
     plan = cache_ops.layered_append(keys, values, kv, mode, k_scales, v_scales)
     med, _ = timed(lambda: plan(slots), 20)
     res["one_launch_all_layers"] = entry(med, 1)
+    # a decode step: 256 tokens, one per sequence, per-layer launches from a HIP graph (the most frequent step of a
+    # serving loop; 1 MB per launch, so the figure of merit is microseconds per launch against the empty launch)
+    Td = 256
+    dslots = slots[slots >= 0][:Td].contiguous()
+
+    def decode_per_layer():
+        for l in range(L):
+            cache_ops.reshape_and_cache_flash(keys[l][:Td], values[l][:Td], kv[l][0], kv[l][1], dslots, mode, ks[l], vs[l])
+
+    med, _ = timed(graphed(decode_per_layer).replay, 20)
+    res["decode_step_256_tokens_per_layer_hip_graph"] = rec(
+        L * (Td * 2 * row * (2 + kv[0].element_size()) + 8 * Td), med, L, kernel, tokens_per_s=round(Td / (med * 1e-3)))
     # yardstick: L dependent launches of a plain copy of the same bytes per layer
     layer_bytes = step_bytes // L
     half = layer_bytes // 2 // 4096 * 4096

@@ -762,7 +762,7 @@ __global__ __launch_bounds__(WAVES * 64) void emm_append_kernel(
   // of the whole launch reading first and writing afterwards.
   // A whole-step launch (TABLES) is long enough to reach that overlap by itself and measured 3 %
   // faster with all rows requested before the slot wait.
-  constexpr int kFirstEarly = TABLES ? 0 : 1;
+  constexpr int kFirstEarly = (TABLES || R == 1) ? 0 : 1;
 #pragma unroll
   for (int r = kFirstEarly; r < R; ++r) {
     const uint32_t t = t0 + r < num_tokens ? t0 + r : num_tokens - 1; // tail: re-read the last row, dropped below
@@ -937,7 +937,9 @@ int append_copy(const void *const *k, const void *const *v, void *const *kc, voi
     // a whole-step launch with one (6.23 TB/s; the others 6.11-6.14); the other shapes are selectable
     // in benchmark builds
     int shape = (move_variant() >> 12) & 0xf;
-    if (shape == 0) shape = tables ? 4 : 3;
+    // per-layer launches: as many waves as the tokens allow up to a few thousand (a decode step of 256 tokens:
+    // 2.2 us per launch with one row per wave, 2.9 with four; the floor of an empty launch is 2.0)
+    if (shape == 0) shape = tables ? 4 : num_tokens <= 1536 ? 4 : num_tokens <= 6144 ? 5 : 3;
     switch (shape) {
     case 1: launch_append<u32x4, 1, 4, 1>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
     case 2: launch_append<u32x4, 2, 4, 1>(tables, t, slot_mapping, num_tokens, row_bytes, ks, vs, num_slots, num_layers, s); break;
@@ -1132,7 +1134,7 @@ int append_strided(const void *const *k, const void *const *v, void *const *kc, 
 // every K group and one element to every V run, so tokens that fill a block in order produce
 // contiguous output; a single token produces 16-byte (K) and element-sized (V) stores at a stride
 // of block_size * 16 bytes resp. block_size elements.
-constexpr int kPagedTokens = 16; // tokens per tile: the tile owns the runs that start in it
+constexpr int kPagedRun = 16;    // tokens of a whole run = rows staged through LDS = rows of a round of direct stores
 constexpr int kPagedRows = 32;   // token positions a tile looks at: an owned run may reach 15 tokens past the tile
 constexpr int kPagedSeg = 256;   // row elements per workgroup
 
@@ -1162,8 +1164,12 @@ constexpr int kPagedSeg = 256;   // row elements per workgroup
 //    block — but no barrier and no LDS latency is spent on them.
 // The scalar arguments are explicit and ordered by first use: the 14 dwords up to value_stride
 // arrive preloaded in scalar registers.
+// TT = tokens per tile (the runs that start in a tile are its own): 16, or 4 for launches of few tokens — a
+// decode step's lone tokens then spread over four times as many compute units, whose rate of
+// element-sized stores is what such a launch waits for; finding the runs four times as often costs
+// long launches more than that gains.
 // grid: x = token tiles, y = 2 * row segments (bit 0: K | V), z = layers.
-template <int CE, int SRC_DTYPE, bool SAT, bool TABLES>
+template <int CE, int SRC_DTYPE, bool SAT, int TT, bool TABLES>
 __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
     const int64_t *__restrict__ slot_mapping, const char *key, const char *value, char *key_cache,
     char *value_cache, uint32_t num_tokens, uint32_t row_elems, uint32_t key_stride, uint32_t value_stride,
@@ -1172,9 +1178,9 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
   constexpr int X = 16 / CE;               // elements per 16-byte piece of the cache
   constexpr int ROW = kPagedSeg * CE + 16; // LDS row stride in bytes
   constexpr int kPieces = kPagedSeg / 8;   // 16-byte source pieces per full row
-  constexpr int N = kPagedTokens * kPieces / kThreads; // items per thread in a round of 16 tokens
-  __shared__ __attribute__((aligned(16))) char tile[kPagedTokens * ROW];  // the whole run
-  __shared__ __attribute__((aligned(16))) char stage[kPagedTokens * ROW]; // V rows of the other tokens, wave-private
+  constexpr int N = kPagedRun * kPieces / kThreads; // items per thread in a round of 16 tokens
+  __shared__ __attribute__((aligned(16))) char tile[kPagedRun * ROW];  // the whole run
+  __shared__ __attribute__((aligned(16))) char stage[kPagedRun * ROW]; // V rows of the other tokens, wave-private
   __shared__ int64_t s_blk[kPagedRows];                                  // the other owned tokens
   __shared__ int32_t s_off[kPagedRows];
   __shared__ int32_t s_pos[kPagedRows];
@@ -1184,7 +1190,7 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
   __shared__ int32_t s_count; // other owned tokens
   const int tid = threadIdx.x;
   const uint32_t kv = blockIdx.y & 1u, seg = blockIdx.y >> 1;
-  const uint32_t t0 = blockIdx.x * kPagedTokens;
+  const uint32_t t0 = blockIdx.x * TT;
   const int bs = (int)block_size;
 
   // ---- wave 0: slots, runs, owned tokens ----
@@ -1211,10 +1217,10 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
     const uint64_t starts = __ballot(!cont); // bit j: token j starts a run or is skipped (lanes >= 32: set)
     const uint64_t below = starts & ((2ull << i) - 1ull);
     const int head = below ? 63 - __builtin_clzll(below) : -1; // first token of this token's run
-    const bool owned = valid && head >= 0 && head < kPagedTokens;
+    const bool owned = valid && head >= 0 && head < TT;
     const uint64_t owned_mask = __ballot(owned);
     // a run of 16 tokens starts at a multiple of 16 slots; its V region is 16-byte aligned if the block's is
-    const bool whole = owned && !cont && i < kPagedTokens && ((bs * CE) & 15) == 0 &&
+    const bool whole = owned && !cont && i < TT && ((bs * CE) & 15) == 0 &&
                        __builtin_ctzll(starts >> (i + 1)) + 1 == 16;
     const uint64_t whole_mask = __ballot(whole);
     const int w0 = whole_mask ? (int)__builtin_ctzll(whole_mask) : -1;
@@ -1282,7 +1288,7 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
         }
       }
     } else {
-      for (int r = 0; r < kPagedTokens; ++r)
+      for (int r = 0; r < kPagedRun; ++r)
         for (int e = tid; e < seg_elems; e += kThreads) {
           const uint32_t a = slow_elem(w0 + r, e);
           if constexpr (CE == 2)
@@ -1294,7 +1300,7 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
   }
 
   // ---- the other owned tokens: straight from the registers, 16 tokens per round ----
-  for (int base = 0; base < count; base += kPagedTokens) {
+  for (int base = 0; base < count; base += kPagedRun) {
     if (vec_src) {
       u32x4 v[N];
       int64_t dblk[N];
@@ -1357,7 +1363,7 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
         __builtin_amdgcn_wave_barrier(); // the next round overwrites the rows
       }
     } else {
-      const int end = base + kPagedTokens < count ? base + kPagedTokens : count;
+      const int end = base + kPagedRun < count ? base + kPagedRun : count;
       for (int r = base; r < end; ++r) {
         const int pos = s_pos[r];
         const int64_t dblk = s_blk[r];
@@ -1454,7 +1460,12 @@ int append_paged(const void *const *k, const void *const *v, void *const *kc, vo
   if (!k || !v || !kc || !vc || !slot_mapping) return fail(EMM_EINVAL, "%s: null pointer", what);
   if (cache_elem_bytes == 1 && (!k_scales || !v_scales)) return fail(EMM_EINVAL, "%s: scale pointer is null", what);
   if (ks < row_elems || vs < row_elems) return fail(EMM_EINVAL, "%s: token stride smaller than the row", what);
-  const int64_t tiles = (num_tokens + kPagedTokens - 1) / kPagedTokens;
+  // tiles of 4 tokens for launches of at most 256 tokens (a decode step, 256 lone tokens: 4.6 us per launch against
+  // 5.9 with tiles of 16; a 512-token prompt: 5.4 against 4.5 — three of four small tiles find nothing to do)
+  int tile_tokens = num_tokens <= 256 ? 4 : 16;
+  if (((move_variant() >> 20) & 3) == 1) tile_tokens = 16;
+  if (((move_variant() >> 20) & 3) == 2) tile_tokens = 4;
+  const int64_t tiles = (num_tokens + tile_tokens - 1) / tile_tokens;
   const int64_t segs = (row_elems + kPagedSeg - 1) / kPagedSeg;
   if (tiles > 0x7fffffffLL || segs * 2 > kMaxGridY) return fail(EMM_EINVAL, "%s: too many tokens / too long rows", what);
   if (num_tokens > 0x7fffffffLL || row_elems > 0x7fffffffLL || ks > 0xffffffffLL || vs > 0xffffffffLL)
@@ -1477,17 +1488,22 @@ int append_paged(const void *const *k, const void *const *v, void *const *kc, vo
     }
   }
   const dim3 grid((uint32_t)tiles, (uint32_t)(segs * 2), (uint32_t)num_layers);
-#define EMM_PAGED_LAUNCH(CE_, DT_, SAT_) \
+#define EMM_PAGED_LAUNCH2(CE_, DT_, SAT_, TT_) \
   do { \
     if (tables) \
-      emm_append_paged_kernel<CE_, DT_, SAT_, true><<<grid, kThreads, 0, s>>>( \
+      emm_append_paged_kernel<CE_, DT_, SAT_, TT_, true><<<grid, kThreads, 0, s>>>( \
           slot_mapping, nullptr, nullptr, nullptr, nullptr, (uint32_t)num_tokens, (uint32_t)row_elems, (uint32_t)ks, \
           (uint32_t)vs, (uint32_t)block_size, vec_src, num_blocks, k_scales, v_scales, t); \
     else \
-      emm_append_paged_kernel<CE_, DT_, SAT_, false><<<grid, kThreads, 0, s>>>( \
+      emm_append_paged_kernel<CE_, DT_, SAT_, TT_, false><<<grid, kThreads, 0, s>>>( \
           slot_mapping, (const char *)k[0], (const char *)v[0], (char *)kc[0], (char *)vc[0], (uint32_t)num_tokens, \
           (uint32_t)row_elems, (uint32_t)ks, (uint32_t)vs, (uint32_t)block_size, vec_src, num_blocks, k_scales, \
           v_scales, NoTables{}); \
+  } while (0)
+#define EMM_PAGED_LAUNCH(CE_, DT_, SAT_) \
+  do { \
+    if (tile_tokens == 4) EMM_PAGED_LAUNCH2(CE_, DT_, SAT_, 4); \
+    else EMM_PAGED_LAUNCH2(CE_, DT_, SAT_, 16); \
   } while (0)
   if (cache_elem_bytes == 2) EMM_PAGED_LAUNCH(2, EMM_DTYPE_BF16, false);
   else if (src_dtype == EMM_DTYPE_BF16 && !sat) EMM_PAGED_LAUNCH(1, EMM_DTYPE_BF16, false);
@@ -1495,6 +1511,7 @@ int append_paged(const void *const *k, const void *const *v, void *const *kc, vo
   else if (!sat) EMM_PAGED_LAUNCH(1, EMM_DTYPE_F16, false);
   else EMM_PAGED_LAUNCH(1, EMM_DTYPE_F16, true);
 #undef EMM_PAGED_LAUNCH
+#undef EMM_PAGED_LAUNCH2
   return check_launch(what);
 }
 
@@ -1920,7 +1937,7 @@ extern "C" {
 
 int emm_hook_set_move_variant(int variant) {
   const int old = g_move_variant;
-  g_move_variant = variant & 0x10fff00;
+  g_move_variant = variant & 0x13fff00;
   return old;
 }
 

@@ -429,6 +429,10 @@ def paged_caches_cpu(NB, H, D, bs, dtype, fill_mod=61):
     (torch.float16, 96, 8, 3, 40, 333, 0, "120-element rows, block size 8"),
     (torch.bfloat16, 48, 32, 2, 64, 700, 0, "block size 32"),
     (torch.bfloat16, 33, 16, 5, 104, 1, 0, "a single token; 520-element rows (second segment of 8)"),
+    (torch.bfloat16, 64, 16, 4, 128, 256, 5, "256 tokens (tiles of 4 tokens): prompts off the tile grid"),
+    (torch.float16, 64, 16, 8, 128, 200, 0, "200 tokens (tiles of 4 tokens), two row segments"),
+    (torch.float16, 96, 8, 3, 40, 150, 3, "150 tokens (tiles of 4 tokens), block size 8"),
+    (torch.bfloat16, 48, 32, 2, 64, 250, 1, "250 tokens (tiles of 4 tokens), block size 32"),
 ])
 def test_paged_append_against_oracle(dtype, NB, bs, H, D, T, phase, desc):
     say(f"paged append: {desc}")
@@ -478,6 +482,34 @@ def test_paged_append_strided_sources_random_slots_and_golden(golden_dir):
     assert torch.equal(kc_g2, kc_g)
 
 
+@pytest.mark.parametrize("T,fp8", [(700, False), (200, False), (700, True), (200, True)])
+def test_paged_append_unaligned_sources_with_whole_runs(T, fp8):
+    """Sources that do not allow 16-byte loads (odd row stride, base off by one element) with prompts that
+    fill blocks: the element-wise source path feeds both the staged whole runs and the direct stores, with
+    tiles of 16 (700 tokens) and of 4 tokens (200)."""
+    NB, bs, H, D = 64, 16, 2, 128
+    g = torch.Generator().manual_seed(T)
+    qkv = (torch.randn((T, 2 * H * D + 3), generator=g) * 3).to(torch.bfloat16)
+    slots = paged_slots(NB, bs, T, seed=T + 1, phase=3)
+    key, value = qkv[:, 1:1 + H * D], qkv[:, 1 + H * D:1 + 2 * H * D]
+    cdt = torch.uint8 if fp8 else torch.bfloat16
+    kc, vc = paged_caches_cpu(NB, H, D, bs, cdt)
+    kc_g, vc_g = kc.to(DEV), vc.to(DEV)
+    qkv_g = qkv.to(DEV)
+    k_g, v_g = qkv_g[:, 1:1 + H * D].view(T, H, D), qkv_g[:, 1 + H * D:1 + 2 * H * D].view(T, H, D)
+    ks, vs = torch.tensor([0.07]), torch.tensor([0.3])
+    if fp8:
+        cache_ops.reshape_and_cache(k_g, v_g, kc_g.view(torch.float8_e4m3fn), vc_g.view(torch.float8_e4m3fn),
+                                    slots.to(DEV), "fp8", ks.to(DEV), vs.to(DEV))
+        orc.c_reshape_and_cache_paged(key.reshape(T, H, D).contiguous(), value.reshape(T, H, D).contiguous(), kc, vc,
+                                      slots, float(ks), float(vs))
+    else:
+        cache_ops.reshape_and_cache(k_g, v_g, kc_g, vc_g, slots.to(DEV))
+        orc.c_reshape_and_cache_paged(key.reshape(T, H, D).contiguous(), value.reshape(T, H, D).contiguous(), kc, vc,
+                                      slots)
+    assert same_bits(kc_g, kc) and same_bits(vc_g, vc)
+
+
 @pytest.mark.parametrize("fp8", [False, True])
 def test_paged_append_all_layers_in_one_launch(fp8):
     L, NB, bs, H, D, T = 5, 96, 16, 2, 128, 900
@@ -500,9 +532,10 @@ def test_paged_append_all_layers_in_one_launch(fp8):
         assert same_bits(kcs[l], kc) and same_bits(vcs[l], vc), f"layer {l}"
 
 
-@pytest.mark.parametrize("dtype,phase", [(torch.bfloat16, 0), (torch.float16, 2)])
-def test_paged_append_fp8(dtype, phase):
-    NB, bs, H, D, T = 200, 16, 4, 128, 2000
+@pytest.mark.parametrize("dtype,phase,T", [(torch.bfloat16, 0, 2000), (torch.float16, 2, 2000),
+                                           (torch.bfloat16, 3, 256), (torch.float16, 0, 77)])
+def test_paged_append_fp8(dtype, phase, T):
+    NB, bs, H, D = 200, 16, 4, 128
     g = torch.Generator().manual_seed(5)
     key = (torch.randn((T, H, D), generator=g) * 4).to(dtype)
     value = (torch.randn((T, H, D), generator=g) * 300).to(dtype)  # part of it overflows to NaN
@@ -517,7 +550,7 @@ def test_paged_append_fp8(dtype, phase):
     kr, vr = paged_caches_cpu(NB, H, D, bs, torch.uint8)
     orc.ref_reshape_and_cache_paged(key, value, kr, vr, slots, "fp8", ks, vs)
     assert same_bits(kc_g, kr) and same_bits(vc_g, vr)
-    assert int((vc_g.cpu() & 0x7F).eq(0x7F).sum()) > 100
+    assert int((vc_g.cpu() & 0x7F).eq(0x7F).sum()) > (100 if T >= 2000 else 3)
 
 
 def test_fp8_append_exhaustive_bf16_and_f16(golden_dir):
