@@ -516,6 +516,14 @@ def ceilings(src_w, dst_w, dev_tables, payload, dev):
                                    ("scatter_write_16KiB_chunks", _lib.EMM_PROBE_SCATTER_WRITE, dtab, all_di)):
         med, _ = timed(lambda: probe(kind, table, idx), 10)
         out[name] = rec(payload, med, 1, "emm_probe_kernel")
+    # what fetching the block id costs a pack: the same gather with ids computed in registers, and the whole pack
+    # (gathered read + sequential write, 2 x payload) with fetched and with computed ids
+    med, _ = timed(lambda: probe(_lib.EMM_PROBE_GATHER_READ_COMPUTED_IDS, stab, all_si), 10)
+    out["gather_read_computed_ids"] = rec(payload, med, 1, "emm_probe_kernel")
+    med, _ = timed(lambda: probe(_lib.EMM_PROBE_PACK, stab, all_si), 10)
+    out["pack_probe_fetched_ids"] = rec(2 * payload, med, 1, "emm_probe_kernel")
+    med, _ = timed(lambda: probe(_lib.EMM_PROBE_PACK_COMPUTED_IDS, stab, all_si), 10)
+    out["pack_probe_computed_ids"] = rec(2 * payload, med, 1, "emm_probe_kernel")
     r, w = out["sequential_read"]["GBps"], out["sequential_write"]["GBps"]
     g, s = out["gather_read_16KiB_chunks"]["GBps"], out["scatter_write_16KiB_chunks"]["GBps"]
     out["harmonic_seq_read_seq_write"] = round(2 / (1 / r + 1 / w), 1)

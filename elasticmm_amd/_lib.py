@@ -59,6 +59,7 @@ HOOK_SIGNATURES = {
     "emm_hook_fp8_quotient_sweep": (c_int, [c_int, c_int, ctypes.c_uint32, ctypes.c_uint32, _P, _P]),
 }
 EMM_PROBE_SEQ_READ, EMM_PROBE_SEQ_WRITE, EMM_PROBE_GATHER_READ, EMM_PROBE_SCATTER_WRITE = 0, 1, 2, 3
+EMM_PROBE_GATHER_READ_COMPUTED_IDS, EMM_PROBE_PACK_COMPUTED_IDS, EMM_PROBE_PACK = 4, 5, 6
 
 _lib = None
 _hooks = None

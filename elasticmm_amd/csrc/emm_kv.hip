@@ -1871,6 +1871,21 @@ __global__ __launch_bounds__(kThreads) void emm_probe_kernel(const int64_t *__re
     asm volatile("" : "+s"(b), "+s"(plane) : : "memory");
     if ((uint64_t)b >= (uint64_t)nb) return;
     p = plane + b * chunk + tile_off;
+  } else if constexpr (KIND == EMM_PROBE_GATHER_READ_COMPUTED_IDS || KIND == EMM_PROBE_PACK_COMPUTED_IDS ||
+                       KIND == EMM_PROBE_PACK) {
+    // pack with the id taken from the table, or computed (a multiplicative hash of j into [0, nb): no memory
+    // round trip before the data can be requested); gathered read alone with the computed id
+    int64_t b = KIND == EMM_PROBE_PACK ? idx[j] : (int64_t)(((uint64_t)(j * 2654435761u) * nb) >> 32);
+    char *plane = tables.t[0].base[pl];
+    asm volatile("" : "+s"(b), "+s"(plane) : : "memory");
+    if ((uint64_t)b >= (uint64_t)nb) return;
+    const u32x4 v = ld_stream<u32x4, 1>(plane + b * chunk + tile_off);
+    if constexpr (KIND == EMM_PROBE_GATHER_READ_COMPUTED_IDS) {
+      if ((v[0] ^ v[1] ^ v[2] ^ v[3]) == 0x9e3779b9u && sink) sink[threadIdx.x] = v[0];
+    } else {
+      st_stream<u32x4, 1>(lin + (int64_t)pl * lin_plane_stride + (int64_t)j * chunk + tile_off, v);
+    }
+    return;
   } else {
     p = lin + (int64_t)pl * lin_plane_stride + (int64_t)j * chunk + tile_off;
   }
@@ -1945,15 +1960,18 @@ int emm_hook_probe(int kind, void *const *layer_ptrs, int num_layers, int num_kv
                    int64_t chunk_bytes, const int64_t *block_idx, int64_t n, void *linear, uint32_t *sink,
                    emm_stream_t stream) {
   const char *what = "emm_hook_probe";
-  const bool pool = kind == EMM_PROBE_GATHER_READ || kind == EMM_PROBE_SCATTER_WRITE;
-  if (kind < 0 || kind > 3) return fail(EMM_EINVAL, "%s: unknown kind %d", what, kind);
+  if (kind < 0 || kind > EMM_PROBE_PACK) return fail(EMM_EINVAL, "%s: unknown kind %d", what, kind);
+  const bool pool = kind >= EMM_PROBE_GATHER_READ; // every kind but the two sequential ones walks the pool's planes
+  const bool linear_too = kind == EMM_PROBE_PACK || kind == EMM_PROBE_PACK_COMPUTED_IDS;
   if (num_layers <= 0 || num_layers > EMM_MAX_LAYERS || num_kv <= 0 || n <= 0 || n > kMaxGridY || chunk_bytes <= 0 ||
       chunk_bytes % 16)
     return fail(EMM_EINVAL, "%s: bad geometry", what);
   if (pool && (!layer_ptrs || !block_idx || num_blocks <= 0 || num_blocks > 0x7fffffffLL))
     return fail(EMM_EINVAL, "%s: pool kinds need layer_ptrs, block_idx and num_blocks", what);
-  if (!pool && (!linear || !aligned(linear, 16))) return fail(EMM_EINVAL, "%s: linear kinds need a 16-byte aligned buffer", what);
+  if ((!pool || linear_too) && (!linear || !aligned(linear, 16)))
+    return fail(EMM_EINVAL, "%s: linear kinds need a 16-byte aligned buffer", what);
   PlaneTables<1> t;
+  memset(&t, 0, sizeof(t));
   const int planes = num_layers * num_kv;
   if (pool)
     for (int i = 0; i < planes; ++i) {
@@ -1968,7 +1986,11 @@ int emm_hook_probe(int kind, void *const *layer_ptrs, int num_layers, int num_kv
   case EMM_PROBE_SEQ_READ: emm_probe_kernel<EMM_PROBE_SEQ_READ><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
   case EMM_PROBE_SEQ_WRITE: emm_probe_kernel<EMM_PROBE_SEQ_WRITE><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
   case EMM_PROBE_GATHER_READ: emm_probe_kernel<EMM_PROBE_GATHER_READ><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
-  default: emm_probe_kernel<EMM_PROBE_SCATTER_WRITE><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
+  case EMM_PROBE_SCATTER_WRITE: emm_probe_kernel<EMM_PROBE_SCATTER_WRITE><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
+  case EMM_PROBE_GATHER_READ_COMPUTED_IDS: emm_probe_kernel<EMM_PROBE_GATHER_READ_COMPUTED_IDS><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
+  case EMM_PROBE_PACK_COMPUTED_IDS: emm_probe_kernel<EMM_PROBE_PACK_COMPUTED_IDS><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
+  case EMM_PROBE_PACK: emm_probe_kernel<EMM_PROBE_PACK><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
+  default: return fail(EMM_EINVAL, "%s: unknown kind %d", what, kind);
   }
   return check_launch(what);
 }

@@ -33,6 +33,12 @@ int emm_hook_set_move_variant(int variant);
 #define EMM_PROBE_SEQ_WRITE 1
 #define EMM_PROBE_GATHER_READ 2
 #define EMM_PROBE_SCATTER_WRITE 3
+/* what the block-id fetch costs: the gathered read and a whole pack (gathered read + sequential write to
+ * `linear`) with block ids computed from the block's position instead of fetched, and the pack with fetched
+ * ids through the same probe kernel */
+#define EMM_PROBE_GATHER_READ_COMPUTED_IDS 4
+#define EMM_PROBE_PACK_COMPUTED_IDS 5
+#define EMM_PROBE_PACK 6
 int emm_hook_probe(int kind, void *const *layer_ptrs, int num_layers, int num_kv, int64_t num_blocks,
                    int64_t chunk_bytes, const int64_t *block_idx, int64_t n, void *linear, uint32_t *sink,
                    emm_stream_t stream);
