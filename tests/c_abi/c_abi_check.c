@@ -121,6 +121,13 @@ int main(void) {
   orc_kv_pack((const void *const *)h_src, L, KV, NB, chunk, h_si, N, h_want);
   bad += same(h_packed, h_want, packed_bytes, "emm_kv_pack");
 
+  /* the same pack with the block table on the host (ids travel in the kernel argument block) */
+  HIP(hipMemset(d_packed, 0, packed_bytes));
+  EMM(emm_kv_pack_host_ids((const void *const *)d_src, L, KV, NB, chunk, h_si, N, d_packed, stream));
+  HIP(hipStreamSynchronize(stream));
+  HIP(hipMemcpy(h_packed, d_packed, packed_bytes, hipMemcpyDeviceToHost));
+  bad += same(h_packed, h_want, packed_bytes, "emm_kv_pack_host_ids");
+
   /* unpack under another table, then copy_blocks inside the destination pool */
   EMM(emm_kv_unpack(d_dst, L, KV, NB, chunk, d_di, N, d_packed, stream));
   orc_kv_unpack(h_dst, L, KV, NB, chunk, h_di, N, h_want);
