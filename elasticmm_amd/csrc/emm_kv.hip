@@ -1340,7 +1340,9 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
         }
       }
       if (kv == 1) {
-        // rows row0 + 8 * it of lanes 0-31 and 32-63: the wave wrote them itself, LDS keeps a wave's order
+        // rows row0 + 8 * it of lanes 0-31 and 32-63: the wave wrote them itself and LDS keeps a wave's order;
+        // the fence (wavefront scope: no cache action) keeps the compiler from moving the reads above the writes
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
         __builtin_amdgcn_wave_barrier();
         const int lane = tid & 63, first = (tid >> 6) * (64 / kPieces);
 #pragma unroll
@@ -1360,7 +1362,8 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
               st<uint8_t, false>(dst + (int64_t)e * bs, *reinterpret_cast<const uint8_t *>(stage + rl * ROW + e));
           }
         }
-        __builtin_amdgcn_wave_barrier(); // the next round overwrites the rows
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront"); // the next round overwrites the rows
+        __builtin_amdgcn_wave_barrier();
       }
     } else {
       const int end = base + kPagedRun < count ? base + kPagedRun : count;
