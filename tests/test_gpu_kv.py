@@ -309,6 +309,22 @@ def test_cfg3_append_reduced_pool():
     assert same_bits(pool_g[L - 1], ref)
 
 
+@pytest.mark.parametrize("T", [1, 3, 1536, 1537, 2051, 6144, 6145, 6147])
+def test_append_token_counts_around_the_wave_shape_thresholds(T):
+    """The per-layer append picks 1, 2 or 4 token rows per wave from the token count: both sides of each
+    threshold, and counts that leave the last wave partly empty."""
+    NB, bs, H, D = 512, 16, 4, 128
+    slots = make_slots(NB * bs, T, T, pad_frac=0.05)
+    g = torch.Generator().manual_seed(T)
+    key = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+    value = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+    pool_c = cpu_pool(1, NB, bs, H, D, torch.bfloat16, 0, fill=3.0)
+    pool_g = to_dev(pool_c)
+    cache_ops.reshape_and_cache_flash(key.to(DEV), value.to(DEV), pool_g[0][0], pool_g[0][1], slots.to(DEV), "auto")
+    orc.c_reshape_and_cache(key, value, pool_c[0][0], pool_c[0][1], slots)
+    assert same_bits(pool_g[0], pool_c[0])
+
+
 def test_append_strided_tokens_odd_rows_and_layers_variant():
     NB, bs, H, D, T, L = 16, 4, 3, 40, 37, 3  # 240-byte rows (16-B lanes), T not a multiple of 16
     g = torch.Generator().manual_seed(13)
