@@ -391,6 +391,8 @@ def main():
             modes[name] = {"value_GBps": round(mm["value"], 1), "frac": round(mm["value"] / HBM_PEAK_GBPS, 4),
                            "pack_GBps": round(mm["pack_GBps"], 1), "unpack_GBps": round(mm["unpack_GBps"], 1),
                            "avg_launch_us": round(mm["avg_launch_us"], 2)}
+            if mono:
+                modes["pack_probes_one_allocation"] = pack_chain_probes(sw, tabs, payload, dev)
             release(sw, dw)
             del tabs
         modes["what"] = ("the headline workload on pools allocated differently: 'one_allocation_per_pool' is "
@@ -532,6 +534,35 @@ def ceilings(src_w, dst_w, dev_tables, payload, dev):
     out["note"] = ("a copy alternates reads and writes on the same channels and stays below the harmonic mean of its two "
                    "halves (compare plain_copy_same_engine with harmonic_seq_read_seq_write); the scatter probe overwrote "
                    "the destination blocks of the batch")
+    del lin
+    return out
+
+
+def pack_chain_probes(src_w, dev_tables, payload, dev):
+    """What the scalar fetches in front of a pack's data loads cost (whole batch in one launch, probe kernels of the hooks
+    build on a pool in one allocation): ids and plane bases fetched (the product kernel's chain), ids computed in registers,
+    and ids and plane bases both computed — no load at all before the data."""
+    from elasticmm_amd import _lib
+
+    hooks = _lib.load_hooks()
+    sp = src_w.pool
+    all_si = torch.cat([s for s, _ in dev_tables]).contiguous()
+    n = all_si.numel()
+    lin = torch.empty(payload, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    stab = _lib.ptr_table(sp.ptrs)
+
+    def probe(kind):
+        rc = hooks.emm_hook_probe(kind, stab, sp.num_layers, sp.num_kv, sp.num_blocks, sp.chunk_bytes, all_si.data_ptr(), n,
+                                  lin.data_ptr(), None, stream)
+        if rc != 0:
+            raise RuntimeError(hooks.emm_last_error().decode())
+
+    out = {}
+    for name, kind in (("ids_and_plane_bases_fetched", _lib.EMM_PROBE_PACK), ("ids_computed", _lib.EMM_PROBE_PACK_COMPUTED_IDS),
+                       ("nothing_fetched", _lib.EMM_PROBE_PACK_NOTHING_FETCHED)):
+        med, _ = timed(lambda: probe(kind), 10)
+        out[name] = rec(2 * payload, med, 1, "emm_probe_kernel")
     del lin
     return out
 

@@ -60,6 +60,7 @@ HOOK_SIGNATURES = {
 }
 EMM_PROBE_SEQ_READ, EMM_PROBE_SEQ_WRITE, EMM_PROBE_GATHER_READ, EMM_PROBE_SCATTER_WRITE = 0, 1, 2, 3
 EMM_PROBE_GATHER_READ_COMPUTED_IDS, EMM_PROBE_PACK_COMPUTED_IDS, EMM_PROBE_PACK = 4, 5, 6
+EMM_PROBE_PACK_NOTHING_FETCHED = 7
 
 _lib = None
 _hooks = None

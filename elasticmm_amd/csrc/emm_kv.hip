@@ -1875,11 +1875,14 @@ __global__ __launch_bounds__(kThreads) void emm_probe_kernel(const int64_t *__re
     if ((uint64_t)b >= (uint64_t)nb) return;
     p = plane + b * chunk + tile_off;
   } else if constexpr (KIND == EMM_PROBE_GATHER_READ_COMPUTED_IDS || KIND == EMM_PROBE_PACK_COMPUTED_IDS ||
-                       KIND == EMM_PROBE_PACK) {
+                       KIND == EMM_PROBE_PACK || KIND == EMM_PROBE_PACK_NOTHING_FETCHED) {
     // pack with the id taken from the table, or computed (a multiplicative hash of j into [0, nb): no memory
-    // round trip before the data can be requested); gathered read alone with the computed id
+    // round trip before the data can be requested); gathered read alone with the computed id; and the pack
+    // with the plane base computed as well (planes evenly spaced from the first, whose pointer arrives
+    // preloaded with the leading arguments): no scalar load at all in front of the data
     int64_t b = KIND == EMM_PROBE_PACK ? idx[j] : (int64_t)(((uint64_t)(j * 2654435761u) * nb) >> 32);
-    char *plane = tables.t[0].base[pl];
+    char *plane = KIND == EMM_PROBE_PACK_NOTHING_FETCHED ? tables.t[0].base[0] + (int64_t)pl * nb * chunk
+                                                         : tables.t[0].base[pl];
     asm volatile("" : "+s"(b), "+s"(plane) : : "memory");
     if ((uint64_t)b >= (uint64_t)nb) return;
     const u32x4 v = ld_stream<u32x4, 1>(plane + b * chunk + tile_off);
@@ -1963,9 +1966,9 @@ int emm_hook_probe(int kind, void *const *layer_ptrs, int num_layers, int num_kv
                    int64_t chunk_bytes, const int64_t *block_idx, int64_t n, void *linear, uint32_t *sink,
                    emm_stream_t stream) {
   const char *what = "emm_hook_probe";
-  if (kind < 0 || kind > EMM_PROBE_PACK) return fail(EMM_EINVAL, "%s: unknown kind %d", what, kind);
+  if (kind < 0 || kind > EMM_PROBE_PACK_NOTHING_FETCHED) return fail(EMM_EINVAL, "%s: unknown kind %d", what, kind);
   const bool pool = kind >= EMM_PROBE_GATHER_READ; // every kind but the two sequential ones walks the pool's planes
-  const bool linear_too = kind == EMM_PROBE_PACK || kind == EMM_PROBE_PACK_COMPUTED_IDS;
+  const bool linear_too = kind == EMM_PROBE_PACK || kind == EMM_PROBE_PACK_COMPUTED_IDS || kind == EMM_PROBE_PACK_NOTHING_FETCHED;
   if (num_layers <= 0 || num_layers > EMM_MAX_LAYERS || num_kv <= 0 || n <= 0 || n > kMaxGridY || chunk_bytes <= 0 ||
       chunk_bytes % 16)
     return fail(EMM_EINVAL, "%s: bad geometry", what);
@@ -1981,6 +1984,10 @@ int emm_hook_probe(int kind, void *const *layer_ptrs, int num_layers, int num_kv
       if (!layer_ptrs[i / num_kv] || !aligned(layer_ptrs[i / num_kv], 16)) return fail(EMM_EINVAL, "%s: bad layer pointer", what);
       t.t[0].base[i] = (char *)layer_ptrs[i / num_kv] + (int64_t)(i % num_kv) * num_blocks * chunk_bytes;
     }
+  if (kind == EMM_PROBE_PACK_NOTHING_FETCHED)
+    for (int i = 0; i < planes; ++i)
+      if (t.t[0].base[i] != t.t[0].base[0] + (int64_t)i * num_blocks * chunk_bytes)
+        return fail(EMM_EINVAL, "%s: this kind needs a pool whose planes are evenly spaced (one allocation)", what);
   const dim3 grid((uint32_t)((chunk_bytes + kThreads * 16 - 1) / (kThreads * 16)), (uint32_t)n, (uint32_t)planes);
   hipStream_t s = as_stream(stream);
   char *lin = (char *)linear;
@@ -1993,6 +2000,7 @@ int emm_hook_probe(int kind, void *const *layer_ptrs, int num_layers, int num_kv
   case EMM_PROBE_GATHER_READ_COMPUTED_IDS: emm_probe_kernel<EMM_PROBE_GATHER_READ_COMPUTED_IDS><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
   case EMM_PROBE_PACK_COMPUTED_IDS: emm_probe_kernel<EMM_PROBE_PACK_COMPUTED_IDS><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
   case EMM_PROBE_PACK: emm_probe_kernel<EMM_PROBE_PACK><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
+  case EMM_PROBE_PACK_NOTHING_FETCHED: emm_probe_kernel<EMM_PROBE_PACK_NOTHING_FETCHED><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
   default: return fail(EMM_EINVAL, "%s: unknown kind %d", what, kind);
   }
   return check_launch(what);

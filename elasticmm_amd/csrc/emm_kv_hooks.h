@@ -39,6 +39,8 @@ int emm_hook_set_move_variant(int variant);
 #define EMM_PROBE_GATHER_READ_COMPUTED_IDS 4
 #define EMM_PROBE_PACK_COMPUTED_IDS 5
 #define EMM_PROBE_PACK 6
+/* the pack with computed ids and computed plane bases (pool in one allocation): no scalar load before the data */
+#define EMM_PROBE_PACK_NOTHING_FETCHED 7
 int emm_hook_probe(int kind, void *const *layer_ptrs, int num_layers, int num_kv, int64_t num_blocks,
                    int64_t chunk_bytes, const int64_t *block_idx, int64_t n, void *linear, uint32_t *sink,
                    emm_stream_t stream);
