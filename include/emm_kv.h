@@ -270,6 +270,8 @@ int emm_reshape_and_cache_strided(const void *const *key_ptrs,
  * PagedAttention backend (its default on ROCm) instead of flash-attn; the pool
  * bound at worker.py:408-412 is then [2, num_blocks, block_size * H * D] per layer,
  * which pack / unpack / copy_blocks move unchanged (one block is still one chunk).
+ * Limits: num_tokens and num_heads * head_size below 2^31, token strides below 2^32
+ * elements (EMM_EINVAL otherwise).
  */
 int emm_reshape_and_cache_paged(const void *key, const void *value,
                                 void *key_cache, void *value_cache,
