@@ -446,10 +446,12 @@ int move_planes(const void *const *src_layers, int64_t src_nb, void *const *dst_
         if (pairs) launch_move_vec<KIND, kOrderRuns, true>(a, (uint32_t)ny, runs / cnt, grid, vec, policy, full, t, s);
         else launch_move_vec<KIND, kOrderRuns, false>(a, (uint32_t)ny, runs / cnt, grid, vec, policy, full, t, s);
       } else {
-        // long scatters (unpack) are walked in groups of 128 blocks per plane visit; short tables
+        // long scatters (unpack) are walked in groups of 256 blocks per plane visit (6712 blocks in one
+        // launch: 6.41-6.50 TB/s; groups of 128: 6.16-6.29, of 512: 6.34, of 64: 5.73; plain order 6.40-6.46 on a
+        // pool spread over the device but 5.65 on one that lies in one stretch of memory); short tables
         // already leave a plane after a few hundred blocks, and gathers (pack) measured faster in
         // the plain order
-        int glog = (KIND == kUnpack && ny >= 1024) ? 7 : 0;
+        int glog = (KIND == kUnpack && ny >= 1024) ? 8 : 0;
         const int forced = (move_variant() >> 16) & 0xf;
         if (forced) glog = forced == 0xf ? 0 : forced;
         if (glog > 0 && ((int64_t)cnt << glog) <= kMaxGridY) {
@@ -1708,12 +1710,12 @@ int emm_kv_unpack_dequant_fp8(void *const *layer_ptrs, int num_layers, int64_t n
     const char *packed = (const char *)packed_fp8 + j0 * chunk_elems;
     const int64_t *idx = block_idx + j0;
     const int64_t stride = n * chunk_elems;
-    const bool grouped = ny >= 1024 && ((2 * num_layers) << 7) <= kMaxGridY;
-    const dim3 grid = grouped ? dim3((uint32_t)tpc, (uint32_t)((2 * num_layers) << 7), (uint32_t)((ny + 127) >> 7))
+    const bool grouped = ny >= 1024 && ((2 * num_layers) << 8) <= kMaxGridY; // groups of 256 blocks, as in unpack
+    const dim3 grid = grouped ? dim3((uint32_t)tpc, (uint32_t)((2 * num_layers) << 8), (uint32_t)((ny + 255) >> 8))
                               : dim3((uint32_t)tpc, (uint32_t)ny, (uint32_t)(2 * num_layers));
 #define EMM_DQ_LAUNCH(DT, G) \
   emm_unpack_dequant_fp8_kernel<DT, G><<<grid, kThreads, 0, s>>>(packed, idx, k_scales, v_scales, stride, \
-      (uint32_t)chunk_elems, (uint32_t)num_blocks, (uint32_t)ny, 7u, t)
+      (uint32_t)chunk_elems, (uint32_t)num_blocks, (uint32_t)ny, 8u, t)
     if (out_dtype == EMM_DTYPE_BF16) { if (grouped) EMM_DQ_LAUNCH(EMM_DTYPE_BF16, true); else EMM_DQ_LAUNCH(EMM_DTYPE_BF16, false); }
     else { if (grouped) EMM_DQ_LAUNCH(EMM_DTYPE_F16, true); else EMM_DQ_LAUNCH(EMM_DTYPE_F16, false); }
 #undef EMM_DQ_LAUNCH
