@@ -48,9 +48,13 @@ def host_block_ids(block_indices: IndexLike, num_blocks: int) -> Optional[np.nda
         arr = t.numpy()
     else:
         arr = np.asarray(block_indices, dtype=np.int64)
+    flat_list = arr.ndim == 1 and isinstance(block_indices, (list, tuple))
     arr = np.ascontiguousarray(arr.reshape(-1))
     if arr.size:
-        lo, hi = int(arr.min()), int(arr.max())
+        if arr.size <= 64 and flat_list:  # numpy's reductions cost more than the list's
+            lo, hi = min(block_indices), max(block_indices)
+        else:
+            lo, hi = int(arr.min()), int(arr.max())
         if lo < -num_blocks or hi >= num_blocks:
             bad = lo if lo < -num_blocks else hi
             raise IndexError(f"index {bad} is out of bounds for dimension 1 with size {num_blocks}")
@@ -122,6 +126,9 @@ class PoolView:
         self.chunk_elems = int(np.prod(self.block_shape, dtype=np.int64)) if self.block_shape else 1
         self.chunk_bytes = self.chunk_elems * self.elem_bytes
         self.ptrs = [t.data_ptr() for t in layers]
+        # the host pointer tables the entry points take, built once (the layers stay where they are)
+        self._groups = [(l0, ptr_table(self.ptrs[l0:l0 + EMM_MAX_LAYERS]))
+                        for l0 in range(0, len(layers), EMM_MAX_LAYERS)]
 
     @property
     def num_layers(self) -> int:
@@ -129,8 +136,7 @@ class PoolView:
 
     def layer_groups(self):
         """(first_layer, ctypes pointer table) per group of at most EMM_MAX_LAYERS layers."""
-        for l0 in range(0, self.num_layers, EMM_MAX_LAYERS):
-            yield l0, ptr_table(self.ptrs[l0:l0 + EMM_MAX_LAYERS])
+        return self._groups
 
     def packed_shape(self, n: int):
         return (self.num_layers, self.num_kv, n) + self.block_shape
@@ -277,23 +283,28 @@ def kv_unpack_dequant_fp8(pool: PoolView, block_indices: IndexLike, packed_fp8: 
 
 def _row_geometry(x: torch.Tensor, what: str):
     """(num_tokens, row_elems, token_stride_elems) of a [T, ...] tensor whose rows are contiguous."""
-    nd = x.dim()
+    shape = x.shape
+    nd = len(shape)
     if nd < 1:
         raise ValueError(f"{what}: expected [num_tokens, ...]")
-    T = x.shape[0]
+    T = shape[0]
+    if T > 0 and x.is_contiguous():  # the common case, kept short: this runs once per layer and call
+        row = x.numel() // T
+        return T, row, row
     if nd == 1:
         return T, 1, (x.stride(0) if T > 1 else 1)
     row = 1
-    for d in x.shape[1:]:
+    for d in shape[1:]:
         row *= d
+    strides = x.stride()
     if T > 0:
         # rows must be dense: walk the trailing dimensions from the innermost outwards
         expect = 1
         for d in range(nd - 1, 0, -1):
-            if x.shape[d] != 1 and x.stride(d) != expect:
+            if shape[d] != 1 and strides[d] != expect:
                 raise ValueError(f"{what}: rows must be contiguous (only the token dimension may be strided)")
-            expect *= x.shape[d]
-    return T, row, (x.stride(0) if T > 1 else row)
+            expect *= shape[d]
+    return T, row, (strides[0] if T > 1 else row)
 
 
 def _cache_slots(cache: torch.Tensor, row_elems: int, what: str) -> int:
