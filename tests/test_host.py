@@ -25,6 +25,26 @@ def test_block_index_tensor_follows_torch_indexing_rules():
         kv_ops.block_index_tensor(torch.tensor([1], dtype=torch.int32), 8, cpu)
 
 
+def test_row_geometry_and_host_ids_short_paths():
+    """The per-call checks have short paths (contiguous tensors, short lists); both paths give what the
+    definitions say."""
+    qkv = torch.zeros((7, 3 * 24))
+    for x, want in ((torch.zeros((7, 4, 6)), (7, 24, 24)), (qkv[:, 24:48].view(7, 4, 6), (7, 24, 72)),
+                    (torch.zeros((1, 4, 6)), (1, 24, 24)), (torch.zeros((0, 4, 6)), (0, 24, 24)),
+                    (torch.zeros(5), (5, 1, 1)), (torch.zeros(10)[::2], (5, 1, 2)),
+                    (torch.zeros((3, 1, 8)), (3, 8, 8))):
+        assert kv_ops._row_geometry(x, "x") == want
+    with pytest.raises(ValueError):
+        kv_ops._row_geometry(torch.zeros((7, 6, 4)).transpose(1, 2), "x")  # rows not dense
+    for ids in ([3, -1, 5], list(range(100)) + [-100], (2, 0), [[1, 2], [3, -4]], [], np.array([4, -2])):
+        got = kv_ops.host_block_ids(ids, 100)
+        want = np.asarray(ids, dtype=np.int64).reshape(-1)
+        assert got.dtype == np.int64 and got.tolist() == np.where(want < 0, want + 100, want).tolist()
+    for bad in ([3, 100], [-101], list(range(70)) + [100]):
+        with pytest.raises(IndexError):
+            kv_ops.host_block_ids(bad, 100)
+
+
 def test_ops_refuse_cpu_tensors():
     pool = [torch.zeros((2, 4, 2, 1, 8), dtype=torch.float16)]
     with pytest.raises(RuntimeError, match="GPU only"):
