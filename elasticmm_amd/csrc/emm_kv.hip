@@ -101,12 +101,6 @@ __device__ __forceinline__ void st_stream(char *p, V v) {
     asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
   } else if constexpr (sizeof(V) == 16 && POLICY == 2) {
     asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
-  } else if constexpr (sizeof(V) == 2 && POLICY == 1) {
-    const uint32_t w = v;
-    asm volatile("global_store_short %0, %1, off sc0 sc1" ::"v"(p), "v"(w) : "memory");
-  } else if constexpr (sizeof(V) == 1 && POLICY == 1) {
-    const uint32_t w = v;
-    asm volatile("global_store_byte %0, %1, off sc0 sc1" ::"v"(p), "v"(w) : "memory");
   } else {
     st<V, POLICY != 3>(p, v);
   }
@@ -1364,12 +1358,12 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
           for (int m = 0; m < kPagedSeg / 64; ++m) {
             const int e = m * 64 + lane;
             if (e >= seg_elems) continue;
-            // written through like every other store of the kernel: lines left dirty in the L2 would have to be
-            // written back when the kernel ends
+            // plain stores: the tokens of a partial run write neighbouring elements of the same sectors, which the
+            // L2 merges before they go to memory (written through, a step with an 11-token tail wrote 1 % more)
             if constexpr (CE == 2)
-              st_stream<uint16_t, 1>(dst + (int64_t)e * bs * 2, *reinterpret_cast<const uint16_t *>(stage + rl * ROW + e * 2));
+              st<uint16_t, false>(dst + (int64_t)e * bs * 2, *reinterpret_cast<const uint16_t *>(stage + rl * ROW + e * 2));
             else
-              st_stream<uint8_t, 1>(dst + (int64_t)e * bs, *reinterpret_cast<const uint8_t *>(stage + rl * ROW + e));
+              st<uint8_t, false>(dst + (int64_t)e * bs, *reinterpret_cast<const uint8_t *>(stage + rl * ROW + e));
           }
         }
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront"); // the next round overwrites the rows
