@@ -21,15 +21,17 @@ cores for bounded samples of the same workloads.
 ``extra`` holds the other shapes of the path, each with its own algorithmic bytes, rate,
 fraction of the 8 TB/s peak, kernel name and average launch time:
   allocation_modes   the headline again with each pool in one allocation and with one
-                     allocation per layer (what a pool adopted from vLLM looks like)
+                     allocation per layer (what a pool adopted from vLLM looks like); probes of
+                     what the scalar fetches in front of a pack's loads cost
   list_indices       the headline with block tables passed as Python lists (the reference's
-                     call shape: one pinned staging + H2D copy per call)
+                     call shape; the ids travel in the kernel argument block)
   batched / fused    one launch for the whole batch; fused pool-to-pool migrate; copy_blocks
   ceilings           what this memory system does for the same access patterns without the
                      other half of the copy (sequential / gathered reads, sequential /
                      scattered writes, plain copy), from the hooks build of the library
   append             reshape_and_cache for one step (config 3): per-layer calls eager / from a
-                     HIP graph, one launch for all layers, and the launch-bound yardsticks
+                     HIP graph, one launch for all layers, a 256-token decode step, and the
+                     launch-bound yardsticks (plain copy of the same bytes, empty launch)
   append_paged_layout, cfg1_latency, fp8_70b_shape (config 4), rebalance_200GB (config 5,
   with the vision gather on the same and on a second stream), swap_pcie
 """
