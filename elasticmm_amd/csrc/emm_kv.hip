@@ -1144,7 +1144,7 @@ constexpr int kPagedSeg = 256;   // row elements per workgroup
 //
 // Runs. Consecutive tokens with consecutive slots inside one 16-slot-aligned window of a block
 // form a run (at most 16 tokens). A run belongs to the tile its first token lies in, so a tile
-// of 16 tokens owns runs that may extend up to 15 tokens into the next tile, and leaves the
+// of TT tokens owns runs that may extend up to 15 tokens past its end, and leaves the
 // head of a run that started in the previous tile to that tile: prompts written in order give
 // whole 16-token runs no matter where they start in the token list. Wave 0 finds the runs in
 // registers from the 32 slots after the tile start (lane = token position, three ballots) and
@@ -1152,18 +1152,19 @@ constexpr int kPagedSeg = 256;   // row elements per workgroup
 // one per tile) starts and lands, and a compact list of the other owned tokens. One wave only:
 // the instructions of this step are a visible part of a launch that lasts a few microseconds.
 //
-// Rows. Item q of a round of 16 tokens is (row q / 32, 16-byte source piece q % 32), two per
-// thread, both requested before either is used.
+// Rows. Item q of a round of 16 tokens is (row q / 32, 16-byte source piece q % 32), two per thread.
 //  * The whole run goes to LDS (quantised to e4m3fn on the way when the cache is fp8; rows padded
-//    by 16 bytes so that a column walk touches every bank once) and, after a barrier, to the cache.
-//    K: lane q moves (group q / 16, token q % 16), one 16-byte LDS read and one 16-byte store; 16
-//    neighbouring lanes cover one group, a wave instruction 1 KiB of contiguous cache. V: lane q
-//    gathers one 16-byte piece of the run's [element][16 tokens] region from a column of the tile
-//    (8 or 16 element-sized LDS reads).
-//  * Every other owned token (decode tokens, heads and tails of prompts) is stored straight from
-//    the registers, K as 16-byte (fp8 cache: 8-byte) pieces, V element by element. Each such store
-//    is a partial write of a 32-byte sector — what the layout costs for tokens that do not fill a
-//    block — but no barrier and no LDS latency is spent on them.
+//    by 16 bytes so that a column walk touches every bank once), one row after the other, and,
+//    after a barrier, to the cache. K: lane q moves (group q / 16, token q % 16), one 16-byte LDS
+//    read and one 16-byte store; 16 neighbouring lanes cover one group, a wave instruction 1 KiB of
+//    contiguous cache. V: lane q gathers one 16-byte piece of the run's [element][16 tokens] region
+//    from a column of the tile (8 or 16 element-sized LDS reads).
+//  * Every other owned token (decode tokens, heads and tails of prompts) skips the barrier: both rows
+//    of a thread are requested together; K is stored straight from the registers as 16-byte (fp8
+//    cache: 8-byte) pieces; V passes through rows of a second LDS tile that only the wave itself
+//    reads back, so that a store instruction covers 64 consecutive elements of one token (64 sectors
+//    in 16 consecutive lines). Each such store is a partial write of a 32-byte sector — what the
+//    layout costs for tokens that do not fill a block.
 // The scalar arguments are explicit and ordered by first use: the 14 dwords up to value_stride
 // arrive preloaded in scalar registers.
 // TT = tokens per tile (the runs that start in a tile are its own): 16, or 4 for launches of few tokens — a
