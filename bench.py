@@ -627,6 +627,15 @@ def paged_append_bench(kv, NB, bs, H, D, dev, T=8448, decode=256):
         for l in range(L):
             cache_ops.reshape_and_cache(keys[l][:Td], values[l][:Td], kcs[l], vcs[l], dslots, "auto")
 
+    # the flash layout behind a head-major pool [NB, H, bs, D], handed over as the permuted view vLLM builds: the
+    # strided append kernel, all layers in one launch
+    from elasticmm_amd import kv_ops
+    hk = [kv[l][0].view(NB, H, bs, D).permute(0, 2, 1, 3) for l in range(L)]
+    hv = [kv[l][1].view(NB, H, bs, D).permute(0, 2, 1, 3) for l in range(L)]
+    med, _ = timed(lambda: kv_ops.reshape_and_cache_strided(keys, values, hk, hv, slots), 20)
+    res["head_major_pool_one_launch_all_layers"] = rec(step_bytes, med, 1, "emm_append_strided_kernel",
+                                                       tokens_per_s=round(T / (med * 1e-3)))
+
     dgraph = torch.cuda.CUDAGraph()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):

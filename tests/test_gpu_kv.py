@@ -371,7 +371,13 @@ def test_append_into_head_major_and_padded_caches():
     blocks are padded. The oracle appends into the same views on the CPU; the whole underlying
     storage is compared, so the padding must stay untouched."""
     g = torch.Generator().manual_seed(41)
-    for dtype, NB, bs, H, D, T, L in ((torch.bfloat16, 48, 16, 4, 128, 500, 3), (torch.float16, 20, 8, 3, 20, 77, 1)):
+    # (..., T, L): 500 / 77 tokens: one row per wave; 2000: two, rows of 2 KiB (two passes per row); 6500: four;
+    # block size 12 and 40-byte head rows: the division paths (also with two rows per wave: 1700 tokens); 6 heads of
+    # 512 bytes: rows of 3 KiB
+    for dtype, NB, bs, H, D, T, L in ((torch.bfloat16, 48, 16, 4, 128, 500, 3), (torch.float16, 20, 8, 3, 20, 77, 1),
+                                      (torch.bfloat16, 300, 16, 8, 128, 2000, 2), (torch.bfloat16, 500, 16, 4, 128, 6500, 1),
+                                      (torch.float16, 30, 12, 2, 64, 100, 2), (torch.float16, 200, 12, 2, 64, 1700, 2),
+                                      (torch.bfloat16, 128, 16, 6, 256, 1601, 1)):
         slots = make_slots(NB * bs, T, 41, pad_frac=0.1)
         keys = [torch.randn((T, H, D), generator=g).to(dtype) for _ in range(L)]
         values = [torch.randn((T, H, D), generator=g).to(dtype) for _ in range(L)]
