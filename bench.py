@@ -393,6 +393,8 @@ def main():
             modes[name] = {"value_GBps": round(mm["value"], 1), "frac": round(mm["value"] / HBM_PEAK_GBPS, 4),
                            "pack_GBps": round(mm["pack_GBps"], 1), "unpack_GBps": round(mm["unpack_GBps"], 1),
                            "avg_launch_us": round(mm["avg_launch_us"], 2)}
+            ab = append_bench(dw.kv_cache, NB, bs, H, D, None, None, dev)
+            modes[name]["append"] = {k: ab[k] for k in ("per_layer_calls_hip_graph", "one_launch_all_layers")}
             if mono:
                 modes["pack_probes_one_allocation"] = pack_chain_probes(sw, tabs, payload, dev)
             release(sw, dw)
