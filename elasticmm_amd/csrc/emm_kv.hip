@@ -380,11 +380,6 @@ int move_planes(const void *const *src_layers, int64_t src_nb, void *const *dst_
   constexpr bool SP = KIND != kUnpack, DP = KIND != kPack;
   if (n == 0 || num_layers == 0 || num_kv == 0 || chunk == 0) return EMM_OK;
   InlineIds inline_ids;
-  if (host_ids) { // ids travel in the argument block; what the device path would skip becomes the skip mark
-    const int64_t nb = SP ? src_nb : dst_nb;
-    for (int64_t j = 0; j < n; ++j)
-      inline_ids.id[j] = (host_ids[j] >= 0 && host_ids[j] < nb) ? (uint32_t)host_ids[j] : 0xffffffffu;
-  }
   int al = 16;
   if (KIND != kPoolToPool) al = common_align(al, linear);
   for (int l = 0; l < num_layers; ++l) {
@@ -412,8 +407,15 @@ int move_planes(const void *const *src_layers, int64_t src_nb, void *const *dst_
       if (SP) t.t[0].base[i] = (char *)src_layers[l] + kv * src_nb * chunk;
       if (DP) t.t[KIND == kPoolToPool ? 1 : 0].base[i] = (char *)dst_layers[l] + kv * dst_nb * chunk;
     }
-    for (int64_t j0 = 0; j0 < n; j0 += kMaxGridY) {
-      const int64_t ny = (n - j0 < kMaxGridY) ? (n - j0) : kMaxGridY;
+    // blocks per launch: what the grid allows, or what the argument block holds (host tables)
+    const int64_t step = host_ids ? EMM_MAX_INLINE_IDS : kMaxGridY;
+    for (int64_t j0 = 0; j0 < n; j0 += step) {
+      const int64_t ny = (n - j0 < step) ? (n - j0) : step;
+      if (host_ids) { // ids travel in the argument block; what the device path would skip becomes the skip mark
+        const int64_t nb = SP ? src_nb : dst_nb;
+        for (int64_t j = 0; j < ny; ++j)
+          inline_ids.id[j] = (host_ids[j0 + j] >= 0 && host_ids[j0 + j] < nb) ? (uint32_t)host_ids[j0 + j] : 0xffffffffu;
+      }
       MoveArgs a;
       a.idx_a = idx_a ? idx_a + (pairs ? 2 * j0 : j0) : nullptr;
       a.idx_b = idx_b ? idx_b + j0 : nullptr;
@@ -423,7 +425,7 @@ int move_planes(const void *const *src_layers, int64_t src_nb, void *const *dst_
       a.src_nb = (uint32_t)src_nb;
       a.dst_nb = (uint32_t)dst_nb;
       if constexpr (KIND != kPoolToPool) {
-        if (host_ids) { // n <= EMM_MAX_INLINE_IDS: one launch, plain order
+        if (host_ids) { // at most EMM_MAX_INLINE_IDS blocks per launch, plain order
           const dim3 grid((uint32_t)tpc, (uint32_t)ny, (uint32_t)cnt);
           if (vec == 16) launch_move_inline<u32x4, 1, KIND, 1>(a, (uint32_t)ny, grid, full, t, inline_ids, s);
           else if (vec == 4) launch_move_inline<uint32_t, 4, KIND, 0>(a, (uint32_t)ny, grid, false, t, inline_ids, s);
@@ -1652,7 +1654,6 @@ int emm_kv_pack_host_ids(const void *const *layer_ptrs, int num_layers, int num_
   const char *what = "emm_kv_pack_host_ids";
   int rc = check_pool_args(what, layer_ptrs, num_layers, num_kv, num_blocks, chunk_bytes, n);
   if (rc != EMM_OK) return rc;
-  if (n > EMM_MAX_INLINE_IDS) return fail(EMM_EINVAL, "%s: n=%lld exceeds EMM_MAX_INLINE_IDS=%d", what, (long long)n, EMM_MAX_INLINE_IDS);
   if (n == 0 || num_layers == 0 || num_kv == 0 || chunk_bytes == 0) return EMM_OK;
   if (!host_block_idx || !packed) return fail(EMM_EINVAL, "%s: null host_block_idx / packed", what);
   return move_planes<kPack>(layer_ptrs, num_blocks, nullptr, 0, num_layers, num_kv, chunk_bytes,
@@ -1665,7 +1666,6 @@ int emm_kv_unpack_host_ids(void *const *layer_ptrs, int num_layers, int num_kv,
   const char *what = "emm_kv_unpack_host_ids";
   int rc = check_pool_args(what, (const void *const *)layer_ptrs, num_layers, num_kv, num_blocks, chunk_bytes, n);
   if (rc != EMM_OK) return rc;
-  if (n > EMM_MAX_INLINE_IDS) return fail(EMM_EINVAL, "%s: n=%lld exceeds EMM_MAX_INLINE_IDS=%d", what, (long long)n, EMM_MAX_INLINE_IDS);
   if (n == 0 || num_layers == 0 || num_kv == 0 || chunk_bytes == 0) return EMM_OK;
   if (!host_block_idx || !packed) return fail(EMM_EINVAL, "%s: null host_block_idx / packed", what);
   return move_planes<kUnpack>(nullptr, 0, layer_ptrs, num_blocks, num_layers, num_kv, chunk_bytes,

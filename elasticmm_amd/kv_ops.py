@@ -145,10 +145,10 @@ class PoolView:
 def kv_pack(pool: PoolView, block_indices: IndexLike, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Gather ``n`` blocks of every layer into ``[L, num_kv, n, *block_shape]``."""
     lib = _lib.load()
-    # a table of up to EMM_MAX_INLINE_IDS ids held on the host (the reference's List[int]) travels in the
-    # kernel argument block: no staging, no host-to-device copy
+    # a table held on the host (the reference's List[int]) travels in the kernel argument block, EMM_MAX_INLINE_IDS
+    # ids per launch: no staging, no host-to-device copy
     host = host_block_ids(block_indices, pool.num_blocks)
-    inline = host is not None and host.size <= EMM_MAX_INLINE_IDS and not pool.on_host
+    inline = host is not None and not pool.on_host
     idx = None if inline else block_index_tensor(host if host is not None else block_indices, pool.num_blocks,
                                                  pool.device)
     n = host.size if inline else idx.numel()
@@ -177,7 +177,7 @@ def kv_unpack(pool: PoolView, block_indices: IndexLike, packed: torch.Tensor) ->
     lib = _lib.load()
     _require_gpu(packed, "kv_unpack")
     host = host_block_ids(block_indices, pool.num_blocks)
-    inline = host is not None and host.size <= EMM_MAX_INLINE_IDS and not pool.on_host
+    inline = host is not None and not pool.on_host
     idx = None if inline else block_index_tensor(host if host is not None else block_indices, pool.num_blocks,
                                                  pool.device)
     n = host.size if inline else idx.numel()

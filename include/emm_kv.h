@@ -42,7 +42,7 @@ extern "C" {
 #define EMM_KV_ABI_VERSION 2
 #define EMM_MAX_LAYERS 96   /* layer pointers carried in one kernel argument block */
 #define EMM_MAX_SEGMENTS 128 /* ragged segments carried by one emm_concat_rows launch */
-#define EMM_MAX_INLINE_IDS 512 /* block ids carried by one emm_kv_*_host_ids launch */
+#define EMM_MAX_INLINE_IDS 512 /* block ids carried by one launch of emm_kv_*_host_ids (longer tables: several launches) */
 
 /* error codes */
 #define EMM_OK 0
@@ -92,15 +92,17 @@ int emm_kv_unpack(void *const *layer_ptrs, int num_layers, int num_kv,
                   emm_stream_t stream);
 
 /*
- * pack / unpack with the block table given as a HOST array of n <= EMM_MAX_INLINE_IDS
- * ids — the form in which the reference holds a request's table (a Python
+ * pack / unpack with the block table given as a HOST array of n ids — the form in
+ * which the reference holds a request's table (a Python
  * List[int] from V0BlockManager, elasticmm/engine/v0/block_manager.py:264-266,
  * passed to extract_kv_blocks / write_kv_blocks, worker.py:578, :612). The ids are
  * copied into the kernel argument block at launch: no device-side table, no
  * host-to-device copy, nothing to keep alive after the call returns, and the kernels
  * fetch an id with a scalar load from the argument block that the whole launch
- * shares. Same results as emm_kv_pack / emm_kv_unpack (negative and too-large ids are
- * skipped). A launch recorded into a HIP graph keeps the ids it was recorded with.
+ * shares (EMM_MAX_INLINE_IDS ids per launch; a longer table takes one launch per
+ * EMM_MAX_INLINE_IDS ids). Same results as emm_kv_pack / emm_kv_unpack (negative and
+ * too-large ids are skipped). A launch recorded into a HIP graph keeps the ids it was
+ * recorded with.
  */
 int emm_kv_pack_host_ids(const void *const *layer_ptrs, int num_layers, int num_kv,
                          int64_t num_blocks, int64_t chunk_bytes,

@@ -735,13 +735,13 @@ def test_concat_rows_non_contiguous_segments():
 
 def test_host_id_entry_points_match_the_device_table_ones():
     """emm_kv_pack_host_ids / emm_kv_unpack_host_ids carry the block table in the kernel argument block. Same
-    bytes as the device-table entry points for tables of 1, 37 and 512 ids (the limit), odd chunk sizes
-    included; ids that the device path skips (negative, too large) are skipped; 513 ids are refused; the
-    Python layer picks the path by where the table lives and how long it is."""
+    bytes as the device-table entry points for tables of 1, 37, 512 (one launch's worth), 513 and 1300 ids
+    (several launches), odd chunk sizes included; ids that the device path skips (negative, too large) are
+    skipped; the Python layer picks the path by where the table lives."""
     import ctypes
 
     lib = _lib.load()
-    L, NB = 3, 700
+    L, NB = 3, 1400
     for block_shape, dtype in (((16, 4, 128), torch.bfloat16), ((3, 5), torch.float16), ((7,), torch.uint8)):
         g = torch.Generator().manual_seed(21)
         pool_c = [torch.randint(0, 255, (2, NB) + block_shape, generator=g).to(torch.uint8).view(torch.uint8)
@@ -750,7 +750,7 @@ def test_host_id_entry_points_match_the_device_table_ones():
             pool_c = [torch.randn((2, NB) + block_shape, generator=g).to(dtype) for _ in range(L)]
         pool_g = to_dev(pool_c)
         pv = PoolView(pool_g)
-        for n in (1, 37, 512):
+        for n in (1, 37, 512, 513, 1300):
             ids = torch.randperm(NB, generator=g)[:n]
             via_list = kv_ops.kv_pack(pv, ids.tolist())              # host table: argument-block path
             via_dev = kv_ops.kv_pack(pv, ids.to(DEV))                # device table
@@ -761,9 +761,6 @@ def test_host_id_entry_points_match_the_device_table_ones():
             kv_ops.kv_unpack(PoolView(d1), dst_ids.tolist(), via_list)
             kv_ops.kv_unpack(PoolView(d2), dst_ids.to(DEV), via_list)
             assert same_bits(torch.stack(d1), torch.stack(d2))
-        # longer host tables fall back to the staged device table
-        ids = torch.randperm(NB, generator=g)[:600]
-        assert same_bits(kv_ops.kv_pack(pv, ids.tolist()), kv_ops.kv_pack(pv, ids.to(DEV)))
     # the C ABI directly: skipped ids, the limit
     pool_g = to_dev(cpu_pool(2, 32, 16, 2, 64, torch.bfloat16, 5))
     pv = PoolView(pool_g)
@@ -779,9 +776,6 @@ def test_host_id_entry_points_match_the_device_table_ones():
             if 0 <= b < 32:
                 want[l, :, j] = pool_g[l][:, b].cpu()
     assert same_bits(out, want)
-    many = np.zeros(513, dtype=np.int64)
-    rc = lib.emm_kv_pack_host_ids(table, 2, 2, 32, pv.chunk_bytes, many.ctypes.data, 513, out.data_ptr(), None)
-    assert rc == -1 and b"EMM_MAX_INLINE_IDS" in lib.emm_last_error()
     rc = lib.emm_kv_unpack_host_ids(table, 2, 2, 32, pv.chunk_bytes, None, 4, out.data_ptr(), None)
     assert rc == -1 and b"null" in lib.emm_last_error()
 
