@@ -1459,22 +1459,27 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
   }
   // ---- V, whole run: 16-byte pieces of the run's [element][16 tokens] region ----
   if constexpr (CE == 2) {
-    // Lanes 0-31 of a wave gather tokens 0-7 of 32 consecutive elements, lanes 32-63 tokens 8-15 of
-    // the same elements: the two half-waves read different tile rows at the same column (the same
-    // LDS banks) in different passes, and one store instruction still covers the 32 elements'
-    // 1 KiB of output completely.
-    const int lane = tid & 63, half = lane >> 5;
+    // The transposing LDS read of gfx950 (ds_read_b64_tr_b16) does the [4 tokens][16 elements] ->
+    // [16 elements][4 tokens] step by itself: in every group of 16 lanes, lane 4 j + q points at elements
+    // c .. c + 3 of token j (c = first element of the group + 4 q), and lane l receives element
+    // (first element + l) of tokens 0 .. 3. Two such reads give a lane 8 tokens of its element = 16 bytes.
+    // Lanes 0-31 of a wave take tokens 0-7 of 32 consecutive elements, lanes 32-63 tokens 8-15 of the same
+    // elements, so that one store instruction covers the 32 elements' 1 KiB of output completely (whole
+    // sectors). Every lane stays active through the reads (its address serves other lanes).
+    typedef short v4i16 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) v4i16 lds_v4i16;
+    const int lane = tid & 63, half = lane >> 5, grp = (lane >> 4) & 1, sub = lane & 15;
     for (int q0 = (tid >> 6) * 32; q0 < seg_elems; q0 += (kThreads >> 6) * 32) {
-      const int e = q0 + (lane & 31);
-      if (e >= seg_elems) continue;
-      const char *col = tile + half * 8 * ROW + e * 2;
+      const char *from = tile + (8 * half + (sub >> 2)) * ROW + (q0 + 16 * grp + 4 * (sub & 3)) * 2;
       uint32_t w[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint32_t lo = *reinterpret_cast<const uint16_t *>(col + (2 * j) * ROW);
-        const uint32_t hi = *reinterpret_cast<const uint16_t *>(col + (2 * j + 1) * ROW);
-        w[j] = lo | (hi << 16);
+      for (int m = 0; m < 2; ++m) {
+        const v4i16 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16 *)(from + 4 * m * ROW));
+        w[2 * m] = (uint32_t)(uint16_t)r[0] | ((uint32_t)(uint16_t)r[1] << 16);
+        w[2 * m + 1] = (uint32_t)(uint16_t)r[2] | ((uint32_t)(uint16_t)r[3] << 16);
       }
+      const int e = q0 + 16 * grp + sub;
+      if (e >= seg_elems) continue;
       char *dst = cache + ((wblk * row_elems + e0 + e) * bs + woff) * 2 + half * 16;
       st_stream<u32x4, 1>(dst, u32x4{w[0], w[1], w[2], w[3]});
     }
