@@ -256,6 +256,49 @@ def test_migrate_equals_pack_then_unpack():
         kv_ops.kv_migrate(PoolView(src_g), si, PoolView(a), di[:-1])
 
 
+def test_block_moves_seeded_sweep_of_shapes():
+    """Thirty seeded draws of (dtype, block size, heads, head size, layers, pool size, table length, table as a list
+    or on the device, one allocation or one per layer): pack, unpack, migrate and copy_blocks against the C
+    restatement. Table lengths straddle the 512 ids that one launch carries in its argument block."""
+    g = torch.Generator().manual_seed(977)
+    pick = lambda xs: xs[int(torch.randint(len(xs), (1,), generator=g))]  # noqa: E731
+    for case in range(30):
+        dtype = pick([torch.bfloat16, torch.float16, torch.float32, torch.uint8])
+        bs, H, D = pick([1, 2, 8, 16, 32]), pick([1, 2, 3, 5, 8]), pick([3, 7, 16, 40, 64, 128])
+        L = pick([1, 2, 7, 33])
+        n = pick([1, 2, 31, 511, 512, 513, 700])
+        if bs * H * D * L * n > (48 << 20):
+            n = 31
+        NB = n + pick([1, 5, 64])
+        as_list, mono = pick([True, False]), pick([True, False])
+        say(f"block-move sweep {case}: {dtype} bs={bs} H={H} D={D} L={L} NB={NB} n={n} list={as_list} mono={mono}")
+        if dtype == torch.uint8:
+            src_c = [torch.randint(0, 255, (2, NB, bs, H, D), generator=g, dtype=torch.uint8) for _ in range(L)]
+        else:
+            src_c = [torch.randint(-30000, 30000, (2, NB, bs, H, D), generator=g).to(dtype) for _ in range(L)]
+        dst_c = [torch.zeros_like(t) for t in src_c]
+        si_t, di_t = torch.randperm(NB, generator=g)[:n], torch.randperm(NB, generator=g)[:n]
+        si, di = (si_t.tolist(), di_t.tolist()) if as_list else (si_t.to(DEV), di_t.to(DEV))
+        src_g, dst_g, mig_g = to_dev(src_c, mono), to_dev(dst_c, mono), to_dev(dst_c, mono)
+        buf = kv_ops.kv_pack(PoolView(src_g), si)
+        assert same_bits(buf, orc.c_kv_pack(src_c, si_t.tolist())), f"pack, case {case}"
+        kv_ops.kv_unpack(PoolView(dst_g), di, buf)
+        orc.c_kv_unpack(dst_c, di_t.tolist(), raw(buf))
+        assert same_bits(torch.stack(dst_g), torch.stack(dst_c)), f"unpack, case {case}"
+        kv_ops.kv_migrate(PoolView(src_g), si, PoolView(mig_g), di)
+        assert same_bits(torch.stack(mig_g), torch.stack(dst_c)), f"migrate, case {case}"
+        half = n // 2
+        if half:
+            perm = torch.randperm(NB, generator=g)
+            mapping = torch.stack([perm[:half], perm[half:2 * half]], 1).contiguous()
+            if as_list:
+                kv_ops.copy_blocks(PoolView(src_g), mapping.tolist())
+            else:
+                cache_ops.copy_blocks(src_g, mapping.to(DEV))
+            orc.c_copy_blocks(src_c, mapping.numpy())
+            assert same_bits(torch.stack(src_g), torch.stack(src_c)), f"copy_blocks, case {case}"
+
+
 # ------------------------------------------------------------------ legacy pools
 def test_monolithic_6d_pool_and_vision_pool():
     L, NB, bs, H, D = 3, 20, 16, 2, 64
@@ -353,6 +396,48 @@ def test_append_strided_tokens_odd_rows_and_layers_variant():
     vcc = torch.zeros_like(kcc)
     orc.c_reshape_and_cache(x[:, 1:2, :].contiguous(), x[:, 1:2, :].contiguous(), kcc, vcc, sl)
     assert same_bits(kc, kcc) and same_bits(vc, vcc)
+
+
+def test_flash_append_seeded_sweep_of_shapes():
+    """Thirty seeded draws of (dtype, block size, heads, head size, tokens, source row stride, fp8 or not, one call per
+    layer or one for all): the flash-layout append against the C restatement."""
+    g = torch.Generator().manual_seed(4242)
+    pick = lambda xs: xs[int(torch.randint(len(xs), (1,), generator=g))]  # noqa: E731
+    for case in range(30):
+        dtype = pick([torch.bfloat16, torch.float16])
+        bs, H, D = pick([1, 4, 16, 32]), pick([1, 2, 3, 4, 8]), pick([3, 8, 40, 64, 80, 128, 256])
+        T = pick([1, 2, 17, 64, 255, 256, 257, 1000, 1537, 3000])
+        L = pick([1, 2, 5])
+        fp8 = pick([False, False, True])
+        pad = pick([0, 0, 8, 3])  # extra elements per source row
+        fused = pick([True, False])
+        NB = T // bs + 9
+        say(f"flash append sweep {case}: {dtype} bs={bs} H={H} D={D} T={T} L={L} fp8={fp8} row pad={pad} "
+            f"one call for all layers={fused}")
+        slots = make_slots(NB * bs, T, 500 + case, pad_frac=0.07)
+        src = (torch.randn((L, T, 2 * H * D + pad), generator=g) * 5).to(dtype)
+        src_g = src.to(DEV)
+        keys = [src_g[l, :, :H * D].view(T, H, D) for l in range(L)]
+        values = [src_g[l, :, H * D:2 * H * D].view(T, H, D) for l in range(L)]
+        cdt = torch.uint8 if fp8 else dtype
+        pool_c = [(torch.arange(2 * NB * bs * H * D) % 53).to(cdt).view(2, NB, bs, H, D).clone() for _ in range(L)]
+        pool_g = to_dev(pool_c)
+        ks, vs = torch.linspace(0.03, 0.2, L), torch.linspace(0.8, 0.1, L)
+        mode = ("fp8", ks, vs) if fp8 else ()
+        if fused:
+            cache_ops.reshape_and_cache_flash_layers(keys, values, pool_g, slots.to(DEV), *mode)
+        else:
+            for l in range(L):
+                per = ("fp8", ks[l:l + 1].to(DEV), vs[l:l + 1].to(DEV)) if fp8 else ()
+                cache_ops.reshape_and_cache_flash(keys[l], values[l], pool_g[l][0], pool_g[l][1], slots.to(DEV), *per)
+        for l in range(L):
+            k = src[l, :, :H * D].reshape(T, H, D).contiguous()
+            v = src[l, :, H * D:2 * H * D].reshape(T, H, D).contiguous()
+            if fp8:
+                orc.c_reshape_and_cache_fp8(k, v, pool_c[l][0], pool_c[l][1], slots, float(ks[l]), float(vs[l]))
+            else:
+                orc.c_reshape_and_cache(k, v, pool_c[l][0], pool_c[l][1], slots)
+            assert same_bits(pool_g[l], pool_c[l]), f"case {case}, layer {l}"
 
 
 def test_append_out_of_range_slot_is_skipped():
@@ -530,6 +615,67 @@ def test_paged_append_unaligned_sources_with_whole_runs(T, fp8):
         orc.c_reshape_and_cache_paged(key.reshape(T, H, D).contiguous(), value.reshape(T, H, D).contiguous(), kc, vc,
                                       slots)
     assert same_bits(kc_g, kc) and same_bits(vc_g, vc)
+
+
+@pytest.mark.parametrize("bs,T,first", [(16, 2048, 0), (16, 2048, 11), (8, 900, 3), (32, 1500, 17), (16, 250, 9)])
+def test_paged_append_slots_in_pool_order(bs, T, first):
+    """A fresh block manager hands out blocks 0, 1, 2, ...: the slots of a prompt are then consecutive across
+    block boundaries, and a run of consecutive slots must still end at every block's end. Also the same
+    slots backwards (consecutive downwards: no runs at all), and every other slot."""
+    NB, H, D = 160, 4, 128
+    g = torch.Generator().manual_seed(bs + T)
+    key = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+    value = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+    up = torch.arange(first, first + T, dtype=torch.long)
+    for name, slots in (("ascending", up), ("descending", up.flip(0).contiguous()),
+                        ("every other slot", (up * 2) % (NB * bs - 1))):
+        say(f"paged append, slots in pool order: block size {bs}, {T} tokens from slot {first}, {name}")
+        if name == "every other slot":
+            slots = torch.unique(slots, sorted=False)[:T]  # no slot twice: the order of two writes is not defined
+        n = len(slots)
+        kc, vc = paged_caches_cpu(NB, H, D, bs, torch.bfloat16)
+        kc_g, vc_g = kc.to(DEV), vc.to(DEV)
+        cache_ops.reshape_and_cache(key[:n].to(DEV), value[:n].to(DEV), kc_g, vc_g, slots.to(DEV))
+        orc.c_reshape_and_cache_paged(key[:n].contiguous(), value[:n].contiguous(), kc, vc, slots)
+        assert same_bits(kc_g, kc) and same_bits(vc_g, vc), name
+
+
+def test_paged_append_seeded_sweep_of_shapes():
+    """Forty seeded draws of (dtype, block size, heads, head size, tokens, slot pattern, fp8 or not, source
+    row stride), each against the C restatement: shapes nobody picked by hand."""
+    g = torch.Generator().manual_seed(20240607)
+    pick = lambda xs: xs[int(torch.randint(len(xs), (1,), generator=g))]  # noqa: E731
+    for case in range(40):
+        dtype = pick([torch.bfloat16, torch.float16])
+        bs = pick([8, 16, 16, 16, 32])
+        H = pick([1, 2, 3, 4, 8])
+        D = pick([32, 64, 80, 96, 128, 256])
+        T = pick([1, 2, 15, 16, 17, 63, 255, 256, 257, 600, 1100])
+        fp8 = pick([False, False, True])
+        pad = pick([0, 0, 8, 5])  # extra elements per source row: 5 forbids 16-byte loads
+        phase = pick([0, 1, 7, 15])
+        whole = pick([0.0, 0.5, 1.0])
+        NB = 3 * T // bs + 60
+        say(f"paged sweep {case}: {dtype} bs={bs} H={H} D={D} T={T} fp8={fp8} row pad={pad} phase={phase} "
+            f"whole={whole}")
+        slots = paged_slots(NB, bs, T, seed=1000 + case, whole_frac=whole, phase=min(phase, T))
+        src = (torch.randn((T, 2 * H * D + pad), generator=g) * 3).to(dtype)
+        key, value = src[:, :H * D], src[:, H * D:2 * H * D]
+        src_g = src.to(DEV)
+        k_g, v_g = src_g[:, :H * D].view(T, H, D), src_g[:, H * D:2 * H * D].view(T, H, D)
+        cdt = torch.uint8 if fp8 else dtype
+        kc, vc = paged_caches_cpu(NB, H, D, bs, cdt)
+        kc_g, vc_g = kc.to(DEV), vc.to(DEV)
+        kh, vh = key.reshape(T, H, D).contiguous(), value.reshape(T, H, D).contiguous()
+        if fp8:
+            ks, vs = torch.tensor([0.04 + 0.01 * case]), torch.tensor([0.9 - 0.02 * case])
+            cache_ops.reshape_and_cache(k_g, v_g, kc_g.view(torch.float8_e4m3fn), vc_g.view(torch.float8_e4m3fn),
+                                        slots.to(DEV), "fp8", ks.to(DEV), vs.to(DEV))
+            orc.c_reshape_and_cache_paged(kh, vh, kc, vc, slots, float(ks), float(vs))
+        else:
+            cache_ops.reshape_and_cache(k_g, v_g, kc_g, vc_g, slots.to(DEV))
+            orc.c_reshape_and_cache_paged(kh, vh, kc, vc, slots)
+        assert same_bits(kc_g, kc) and same_bits(vc_g, vc), f"case {case}"
 
 
 @pytest.mark.parametrize("fp8", [False, True])
