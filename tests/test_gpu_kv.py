@@ -640,6 +640,30 @@ def test_paged_append_slots_in_pool_order(bs, T, first):
         assert same_bits(kc_g, kc) and same_bits(vc_g, vc), name
 
 
+@pytest.mark.parametrize("bs", [1, 4, 24, 40, 64, 128])
+@pytest.mark.parametrize("fp8", [False, True])
+def test_paged_append_unusual_block_sizes(bs, fp8):
+    """Block sizes outside 8 / 16 / 32, not all powers of two: runs still end at every block's end and at every
+    16th slot of a block, and a 16-token run is staged as a whole only where its V region is 16-byte aligned."""
+    NB, H, D, T = 2200 // bs + 30, 2, 128, 900
+    g = torch.Generator().manual_seed(bs)
+    key = (torch.randn((T, H, D), generator=g) * 2).to(torch.bfloat16)
+    value = (torch.randn((T, H, D), generator=g) * 2).to(torch.bfloat16)
+    slots = paged_slots(NB, bs, T, seed=bs, phase=2)
+    assert len(slots) == T
+    kc, vc = paged_caches_cpu(NB, H, D, bs, torch.uint8 if fp8 else torch.bfloat16)
+    kc_g, vc_g = kc.to(DEV), vc.to(DEV)
+    if fp8:
+        ks, vs = torch.tensor([0.05]), torch.tensor([0.2])
+        cache_ops.reshape_and_cache(key.to(DEV), value.to(DEV), kc_g.view(torch.float8_e4m3fn),
+                                    vc_g.view(torch.float8_e4m3fn), slots.to(DEV), "fp8", ks.to(DEV), vs.to(DEV))
+        orc.c_reshape_and_cache_paged(key, value, kc, vc, slots, float(ks), float(vs))
+    else:
+        cache_ops.reshape_and_cache(key.to(DEV), value.to(DEV), kc_g, vc_g, slots.to(DEV))
+        orc.c_reshape_and_cache_paged(key, value, kc, vc, slots)
+    assert same_bits(kc_g, kc) and same_bits(vc_g, vc)
+
+
 def test_paged_append_seeded_sweep_of_shapes():
     """Forty seeded draws of (dtype, block size, heads, head size, tokens, slot pattern, fp8 or not, source
     row stride), each against the C restatement: shapes nobody picked by hand."""
