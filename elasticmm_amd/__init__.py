@@ -12,6 +12,7 @@ the Python surface of the reference worker on top of it.
   worker           ``KVWorker``: the data-path methods of the reference's V0Worker
   pool_transfer    gather/scatter on the legacy monolithic 6-D pool and the vision block pool
   block_manager    host-side free-list block tables (index producer)
+  kv_transfer      ``KVTransferManager`` / ``KVMigrationManager``: the callers that move requests between workers
 """
 from .build import build_library, library_path  # noqa: F401
 

@@ -137,6 +137,8 @@ class KVTransferManager:
             return self._transfer_via_p2p_copy(request_id, src_rank, src_blocks, dst_rank, dst_blocks)
         if self.transfer_method == TransferMethod.CUDA_IPC:
             return self._transfer_via_device_migrate(request_id, src_rank, src_blocks, dst_rank, dst_blocks)
+        if self.transfer_method == TransferMethod.STAGED_COPY:
+            return self._transfer_via_staged_copy(request_id, src_rank, src_blocks, dst_rank, dst_blocks)
         return False
 
     def _workers(self, src_rank: int, dst_rank: int):
@@ -215,6 +217,31 @@ class KVTransferManager:
             return True
         except Exception as e:
             print(f"[KVTransferManager] device migrate failed: {e}")
+            return False
+
+    def _transfer_via_staged_copy(self, request_id, src_rank, src_blocks, dst_rank, dst_blocks) -> bool:
+        """Through host memory (kv_transfer.py:821-840, a placeholder that sleeps there): pack on the source, one
+        copy into page-locked host memory, one copy onto the destination's device, unpack. For workers whose
+        devices cannot reach each other; PCIe-bound."""
+        import torch
+
+        src_worker, dst_worker = self._workers(src_rank, dst_rank)
+        if src_worker is None:
+            return False
+        try:
+            start_time = time.perf_counter()
+            kv_data = src_worker.extract_kv_blocks(src_blocks)
+            staged = torch.empty(kv_data.shape, dtype=kv_data.dtype, pin_memory=True)
+            staged.copy_(kv_data, non_blocking=True)
+            torch.cuda.current_stream(kv_data.device).synchronize()  # the host copy is complete
+            dst_worker.write_kv_blocks(dst_blocks, staged.to(dst_worker.device, non_blocking=True))
+            elapsed = time.perf_counter() - start_time
+            self.transfer_count += 1
+            if self.metrics_callback:
+                self.metrics_callback(transfer_time_sec=elapsed, num_blocks=len(src_blocks))
+            return True
+        except Exception as e:
+            print(f"[KVTransferManager] staged copy failed: {e}")
             return False
 
     # ----- migration of whole requests (backend.py:674-737) -----------------------
@@ -348,3 +375,82 @@ class KVTransferManager:
         self.transfer_count = 0
         self.total_transfer_time = 0.0
         self.total_bytes_transferred = 0
+
+
+class KVMigrationManager:
+    """Cross-stage moves addressed by (stage, worker id) (kv_transfer.py:867-980, ``V0KVMigrationManager``):
+    extract on the source worker, write on the destination worker, for KV blocks and for a request's vision
+    embeddings. The reference's worker lookup is a placeholder that finds nobody (:961-969), so its moves always
+    report failure; here workers are registered under (stage, worker id)."""
+
+    def __init__(self):
+        self.migration_count = 0
+        self.total_migration_time = 0.0
+        self._workers_by_stage: Dict[Tuple[str, int], Any] = {}
+
+    def register_worker(self, stage: str, worker_id: int, worker: Any) -> None:
+        self._workers_by_stage[(stage.lower(), worker_id)] = worker
+
+    def unregister_worker(self, stage: str, worker_id: int) -> None:
+        self._workers_by_stage.pop((stage.lower(), worker_id), None)
+
+    def _get_worker_ref(self, stage: str, worker_id: int):
+        return self._workers_by_stage.get((stage.lower(), worker_id))
+
+    def _pair(self, src_stage, src_worker_id, dst_stage, dst_worker_id):
+        src_worker = self._get_worker_ref(src_stage, src_worker_id)
+        dst_worker = self._get_worker_ref(dst_stage, dst_worker_id)
+        if src_worker is None or dst_worker is None:
+            print(f"[KVMigrationManager] Worker not found: src={src_stage}/{src_worker_id}, "
+                  f"dst={dst_stage}/{dst_worker_id}")
+            return None, None
+        return src_worker, dst_worker
+
+    def migrate_kv_blocks_sync(self, request_id: str, src_stage: str, src_worker_id: int, src_blocks: List[int],
+                               dst_stage: str, dst_worker_id: int, dst_blocks: List[int]) -> bool:
+        start_time = time.time()
+        try:
+            src_worker, dst_worker = self._pair(src_stage, src_worker_id, dst_stage, dst_worker_id)
+            if src_worker is None:
+                return False
+            kv_data = src_worker.extract_kv_blocks(src_blocks)
+            dst_worker.write_kv_blocks(dst_blocks, kv_data)
+            self.migration_count += 1
+            self.total_migration_time += time.time() - start_time
+            return True
+        except Exception as e:
+            print(f"[KVMigrationManager] KV migration failed: {e}")
+            return False
+
+    def migrate_vision_embeddings_sync(self, request_id: str, src_stage: str, src_worker_id: int, dst_stage: str,
+                                       dst_worker_id: int) -> bool:
+        start_time = time.time()
+        try:
+            src_worker, dst_worker = self._pair(src_stage, src_worker_id, dst_stage, dst_worker_id)
+            if src_worker is None:
+                return False
+            ve_data = src_worker.extract_vision_blocks(request_id)
+            dst_worker.write_vision_blocks(request_id, ve_data)
+            self.migration_count += 1
+            self.total_migration_time += time.time() - start_time
+            return True
+        except Exception as e:
+            print(f"[KVMigrationManager] Vision embedding migration failed: {e}")
+            return False
+
+    async def migrate_kv_blocks(self, request_id: str, src_stage: str, src_worker_id: int, src_blocks: List[int],
+                                dst_stage: str, dst_worker_id: int, dst_blocks: List[int]) -> bool:
+        return self.migrate_kv_blocks_sync(request_id, src_stage, src_worker_id, src_blocks, dst_stage,
+                                           dst_worker_id, dst_blocks)
+
+    async def migrate_vision_embeddings(self, request_id: str, src_stage: str, src_worker_id: int, dst_stage: str,
+                                        dst_worker_id: int) -> bool:
+        return self.migrate_vision_embeddings_sync(request_id, src_stage, src_worker_id, dst_stage, dst_worker_id)
+
+    def get_stats(self) -> Dict[str, Any]:
+        return {
+            "migration_count": self.migration_count,
+            "total_migration_time": self.total_migration_time,
+            "avg_migration_time": (self.total_migration_time / self.migration_count
+                                   if self.migration_count > 0 else 0.0),
+        }

@@ -509,6 +509,40 @@ class KVWorker:
         """worker.py:528-532: forget the request's swap event."""
         self.swap_event_table.pop(request_id, None)
 
+    def clear_request_resource_batched(self, request_ids: List[str]) -> None:
+        """worker.py:534-537."""
+        for request_id in request_ids:
+            self.clear_request_resource(request_id)
+
+    def clear_all_requests(self) -> None:
+        """worker.py:1114-1132: drop every cached vision embedding (before a role switch); the KV pool
+        stays allocated, its blocks belong to the block manager."""
+        if self.ve_cache is not None:
+            self.ve_cache.clear()
+        self._ve_sources.clear()
+        self.swap_event_table.clear()
+
+    # ----- shapes (worker.py:1038-1064) ---------------------------------------
+    def get_kv_cache_shape(self) -> tuple:
+        """``(num_layers, 2, num_blocks, block_size, num_kv_heads, head_size)``, or ``()`` without a pool.
+        The reference asks the per-layer list for ``.shape`` (worker.py:1042), which a list does not have; this
+        is the shape its 6-D consumers (nccl_transfer.py:215) expect."""
+        if self.kv_cache is None:
+            return ()
+        return (len(self.kv_cache),) + tuple(self.kv_cache[0].shape)
+
+    def get_ve_cache_shape(self) -> tuple:
+        """``()``: vision embeddings are kept per request id, not in one tensor (worker.py:431-437)."""
+        return ()
+
+    def get_ve_cache_keys(self) -> List[str]:
+        return [] if self.ve_cache is None else list(self.ve_cache.keys())
+
+    def get_ve_shape(self, request_id: str) -> Optional[tuple]:
+        if self.ve_cache and request_id in self.ve_cache:
+            return tuple(self.ve_cache[request_id].shape)
+        return None
+
     # ----- vision embeddings (worker.py:1007-1036, worker_steps.py:252-267) --
     def extract_vision_blocks(self, request_id: str) -> torch.Tensor:
         if self.ve_cache is None:

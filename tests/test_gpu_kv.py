@@ -1650,7 +1650,8 @@ def test_transfer_manager_methods_move_the_same_bytes():
 
     si, di = [3, 30, 7, 12], [0, 1, 29, 15]
     for method, batching in ((TransferMethod.P2P_COPY, False), (TransferMethod.NCCL, False),
-                             (TransferMethod.CUDA_IPC, False), (TransferMethod.NCCL, True)):
+                             (TransferMethod.CUDA_IPC, False), (TransferMethod.STAGED_COPY, False),
+                             (TransferMethod.NCCL, True)):
         src, dst = make_pair()
         m = KVTransferManager(method, enable_batching=batching, batch_size=2, batch_timeout=1e9)
         m.register_workers("prefill", [src], [0])
@@ -1664,6 +1665,34 @@ def test_transfer_manager_methods_move_the_same_bytes():
         torch.cuda.synchronize()
         check_moved(src, dst, si, di)
         assert m.transfer_kv_cache_sync("bad", 0, 1, [999], [0]) is (True if batching else False)
+
+
+def test_migration_manager_moves_blocks_and_vision_embeddings():
+    """The (stage, worker id)-addressed manager: KV blocks and a request's vision embeddings move from the
+    prefill worker to the decoding worker; an unknown worker or a bad block id reports failure."""
+    import asyncio
+    from elasticmm_amd.kv_transfer import KVMigrationManager
+
+    si, di = [3, 30, 7, 12], [0, 1, 29, 15]
+    src, dst = make_pair()
+    m = KVMigrationManager()
+    assert m.migrate_kv_blocks_sync("a", "prefill", 0, si, "decoding", 0, di) is False  # nobody registered
+    m.register_worker("prefill", 0, src)
+    m.register_worker("Decoding", 0, dst)
+    assert asyncio.run(m.migrate_kv_blocks("a", "prefill", 0, si, "decoding", 0, di)) is True
+    torch.cuda.synchronize()
+    check_moved(src, dst, si, di)
+    assert m.migrate_kv_blocks_sync("bad", "prefill", 0, [999], "decoding", 0, [0]) is False
+    src.init_vecache()
+    dst.init_vecache()
+    e = torch.randn((11, 64), device=DEV)
+    src.write_vision_blocks("a", e)
+    assert asyncio.run(m.migrate_vision_embeddings("a", "prefill", 0, "decoding", 0)) is True
+    assert dst.get_ve_shape("a") == (11, 64) and dst.extract_vision_blocks("a") is e
+    assert m.migrate_vision_embeddings_sync("missing", "prefill", 0, "decoding", 0) is False
+    assert m.get_stats()["migration_count"] == 2
+    m.unregister_worker("prefill", 0)
+    assert m.migrate_kv_blocks_sync("a", "prefill", 0, si, "decoding", 0, di) is False
 
 
 def test_migrate_requests_between_two_workers():

@@ -92,6 +92,60 @@ def test_worker_error_conventions_without_pool():
     assert w.gather_vision_embeddings(["missing"]) is None
 
 
+def test_worker_shape_accessors_and_request_cleanup():
+    w = KVWorker(device="cpu")
+    assert w.get_kv_cache_shape() == () and w.get_ve_cache_shape() == ()
+    assert w.get_ve_cache_keys() == [] and w.get_ve_shape("r") is None
+    w.kv_cache = [torch.zeros((2, 5, 16, 4, 8)) for _ in range(3)]  # shape only: no kernel runs here
+    assert w.get_kv_cache_shape() == (3, 2, 5, 16, 4, 8)
+    w.init_vecache()
+    w.write_vision_blocks("r", torch.zeros((3, 4)))
+    w.write_vision_blocks("q", torch.zeros((7, 4)))
+    assert w.get_ve_cache_keys() == ["r", "q"] and w.get_ve_shape("q") == (7, 4)
+    w.swap_event_table.update({"r": object(), "q": object(), "z": object()})
+    w.clear_request_resource_batched(["r", "q", "never seen"])
+    assert list(w.swap_event_table) == ["z"]
+    w.clear_all_requests()
+    assert w.get_ve_cache_keys() == [] and w.swap_event_table == {} and w.ve_cache == {}
+
+
+def test_migration_manager_registry_and_failures():
+    import asyncio
+    from elasticmm_amd.kv_transfer import KVMigrationManager
+
+    class Fake:
+        def __init__(self):
+            self.blocks, self.ve = {}, {}
+
+        def extract_kv_blocks(self, ids):
+            return [self.blocks[i] for i in ids]  # KeyError for an unknown block
+
+        def write_kv_blocks(self, ids, data):
+            self.blocks.update(zip(ids, data))
+
+        def extract_vision_blocks(self, rid):
+            return self.ve[rid]
+
+        def write_vision_blocks(self, rid, data):
+            self.ve[rid] = data
+
+    a, b = Fake(), Fake()
+    a.blocks = {1: "x", 2: "y"}
+    a.ve = {"r": "emb"}
+    m = KVMigrationManager()
+    assert asyncio.run(m.migrate_kv_blocks("r", "prefill", 0, [1], "decoding", 0, [5])) is False
+    m.register_worker("PREFILL", 0, a)
+    m.register_worker("decoding", 0, b)
+    assert asyncio.run(m.migrate_kv_blocks("r", "prefill", 0, [2, 1], "decoding", 0, [5, 6])) is True
+    assert b.blocks == {5: "y", 6: "x"}
+    assert asyncio.run(m.migrate_vision_embeddings("r", "prefill", 0, "decoding", 0)) is True and b.ve == {"r": "emb"}
+    assert m.migrate_kv_blocks_sync("r", "prefill", 0, [9], "decoding", 0, [5]) is False
+    assert m.migrate_vision_embeddings_sync("nope", "prefill", 0, "decoding", 0) is False
+    st = m.get_stats()
+    assert st["migration_count"] == 2 and st["avg_migration_time"] >= 0.0
+    assert KVMigrationManager().get_stats()["avg_migration_time"] == 0.0
+
+
 def test_coordinated_transfer_preflight():
     link = LoopbackLink(world_size=2)
     w = KVWorker(device="cpu", link=link, global_rank=1)
