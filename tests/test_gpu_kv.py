@@ -323,6 +323,45 @@ def test_monolithic_6d_pool_and_vision_pool():
     assert same_bits(ve_dst_g, ve_dst_c)
 
 
+def test_pool_transfer_manager_sender_and_receiver_halves():
+    """The legacy manager's two halves over the loopback link: what the receiver's pool holds afterwards is the
+    torch statement of the reference's stack / per-block assignment, for the 6-D KV pool and the vision pool."""
+    import asyncio
+    from elasticmm_amd.worker import LoopbackLink
+
+    L, NB, bs, H, D = 3, 20, 16, 2, 64
+    g = torch.Generator().manual_seed(12)
+    pool6 = torch.randn((L, 2, NB, bs, H, D), generator=g).to(torch.bfloat16)
+    si, di = [7, 0, 19, 3, 11], [1, 2, 18, 5, 0]
+    link = LoopbackLink(2)
+    sender, receiver = pool_transfer.PoolTransferManager(link), pool_transfer.PoolTransferManager(link)
+    with pytest.raises(ValueError, match="Group 'g' not found"):
+        sender.transfer_kv_cache_blocks_sync("g", 0, 1, pool6.to(DEV), si, di, True)
+    sender.create_transfer_group("g", 0, 2)
+    receiver.create_transfer_group("g", 1, 2)
+    src_g, dst_c = pool6.to(DEV), torch.zeros_like(pool6)
+    dst_g = dst_c.to(DEV)
+    assert asyncio.run(sender.transfer_kv_cache_blocks("g", 0, 1, src_g, si, di, True)) is None
+    kv_data = asyncio.run(receiver.transfer_kv_cache_blocks("g", 0, 1, dst_g, si, di, False))
+    assert kv_data.shape == (L, 2, len(si), bs, H, D)
+    orc.ref_pool6d_scatter(dst_c, di, orc.ref_pool6d_gather(pool6, si))
+    assert same_bits(dst_g, dst_c) and same_bits(src_g, pool6)
+    st = sender.get_stats()
+    assert st["total_transfers"] == 1 and st["total_bytes_transferred"] == kv_data.numel() * 2 and st["num_groups"] == 1
+    ve = torch.randn((12, 9, 48), generator=g).to(torch.float16)
+    ve_dst_c = torch.zeros_like(ve)
+    ve_dst_g = ve_dst_c.to(DEV)
+    assert sender.transfer_vision_embeddings_sync("g", 0, 1, ve.to(DEV), [5, 11, 0], [2, 3, 4], True) is None
+    got = receiver.transfer_vision_embeddings_sync("g", 0, 1, ve_dst_g, [5, 11, 0], [2, 3, 4], False)
+    assert got.shape == (3, 9, 48)
+    orc.ref_vision_scatter(ve_dst_c, [2, 3, 4], orc.ref_vision_gather(ve, [5, 11, 0]))
+    assert same_bits(ve_dst_g, ve_dst_c)
+    # a message of the wrong type is refused before anything is written
+    sender.transfer_vision_embeddings_sync("g", 0, 1, ve.to(DEV), [1], [1], True)
+    with pytest.raises(ValueError, match="differs from the pool's"):
+        receiver.transfer_vision_embeddings_sync("g", 0, 1, ve_dst_g.to(torch.bfloat16), [1], [1], False)
+
+
 # ------------------------------------------------------------------ append
 def make_slots(num_slots, T, seed, pad_frac=0.05):
     g = torch.Generator().manual_seed(seed)
