@@ -104,7 +104,9 @@ class BlockManager:
         assert self.request_location.get(rid) == BlockLocation.GPU, f"Request {rid} is not on GPU"
         return max(0, self.get_num_blocks_needed(request) - len(self.block_table[rid]))
 
-    def get_max_blocks_needed(self, requests: Iterable[Any]) -> int:
+    def get_max_blocks_needed(self, requests: Any) -> int:
+        """block_manager.py:487-501; takes a BatchedRequests-like object (``.requests``) or an iterable."""
+        requests = getattr(requests, "requests", requests)
         return max((self.get_num_blocks_needed(r) for r in requests), default=0)
 
     def can_allocate(self, request: Any) -> bool:
@@ -238,6 +240,24 @@ class BlockManager:
         return {"gpu": share(gpu_used, self.max_num_gpu_blocks), "cpu": share(cpu_used, self.max_num_cpu_blocks),
                 "swap": f"{len(self.swapping_gpu_blocks_list)} -> {len(self.swapping_cpu_blocks_list)}",
                 "#req": f"{len(self.block_table)}"}
+
+
+    def print_block_usage(self) -> None:
+        usage = self.get_block_usage()
+        print(f"({self.stage}) Block usage: GPU={usage['gpu']}, CPU={usage['cpu']}, "
+              f"Swapping={usage['swap']}, Requests={usage['#req']}")
+
+    # ----- pool tensors sized for a batch (block_manager.py:443-485) ---------------------------
+    def create_kv_cache_tensors(self, batched_requests: Any, num_layers: int, num_heads: int, head_size: int,
+                                dtype: Any, device: str = "cuda") -> List[Any]:
+        """One ``[2, max_blocks, block_size, num_heads, head_size]`` tensor per layer, ``max_blocks`` = the most
+        blocks any request of the batch needs: the layout every kernel of this package takes as a pool.
+        ``batched_requests`` is a BatchedRequests-like object (``.requests``) or an iterable of requests."""
+        import torch
+
+        max_blocks_needed = self.get_max_blocks_needed(batched_requests)
+        shape = (2, max_blocks_needed, self.block_size, num_heads, head_size)
+        return [torch.empty(shape, dtype=dtype, device=device) for _ in range(num_layers)]
 
 
 class VisionBlockManager(BlockManager):

@@ -239,6 +239,20 @@ def test_block_manager_requests_growth_and_queries():
     assert vb.get_num_blocks_needed(_Req("v", 5, images=["i0", "i1"])) == 72 and vb.get_num_blocks_needed(_Req("t", 5)) == 0
 
 
+def test_block_manager_pool_tensors_for_a_batch(capsys):
+    from types import SimpleNamespace as NS
+
+    bm = BlockManager(64, block_size=16, max_num_cpu_blocks=8, stage="decoding")
+    batch = NS(requests=[40, 17, 100])  # token counts stand for requests
+    assert bm.get_max_blocks_needed(batch) == 7 and bm.get_max_blocks_needed([1]) == 1
+    layers = bm.create_kv_cache_tensors(batch, num_layers=3, num_heads=2, head_size=8, dtype=torch.float16, device="cpu")
+    assert len(layers) == 3 and all(t.shape == (2, 7, 16, 2, 8) and t.dtype == torch.float16 for t in layers)
+    assert bm.create_kv_cache_tensors([], 2, 1, 8, torch.float16, "cpu")[0].shape == (2, 0, 16, 1, 8)
+    bm.allocate_blocks("a", 16)
+    bm.print_block_usage()
+    assert capsys.readouterr().out.strip() == "(decoding) Block usage: GPU=25% (16/64), CPU=0% (0/8), Swapping=0 -> 0, Requests=1"
+
+
 def test_block_manager_swap_bookkeeping_and_worker_calls():
     rec = _SwapRecorder()
     bm = BlockManager(6, block_size=16, max_num_cpu_blocks=5, workers=[rec])
