@@ -106,13 +106,6 @@ __device__ __forceinline__ void st_stream(char *p, V v) {
   }
 }
 
-// A value that is the same in every lane, moved to scalar registers.
-__device__ __forceinline__ int64_t uniform64(int64_t x) {
-  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)x);
-  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)x >> 32));
-  return (int64_t)(((uint64_t)hi << 32) | lo);
-}
-
 constexpr int kThreads = 256; // 4 wavefronts of 64 lanes (append / dequant / concat kernels)
 
 // A tile is U * T vectors; lane `tid` owns vectors (u * T + tid). All U loads of a
