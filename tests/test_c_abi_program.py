@@ -1,6 +1,7 @@
 """The C ABI used from C: tests/c_abi/c_abi_check.c (no Python, no torch on its path) is compiled with gcc
-against include/emm_kv.h, libemm_kv.so and the HIP runtime, and checks pack / unpack / copy_blocks / append /
-concat against the loops of oracle/kv_oracle.c."""
+against include/emm_kv.h, libemm_kv.so and the HIP runtime, and checks every data-moving entry point of the header
+(block moves with device and host tables, migrate, the appends of all three layouts in 16-bit and fp8, the
+dequantising unpack, concat, the plain copy) against the loops of oracle/kv_oracle.c."""
 import os
 import subprocess
 
