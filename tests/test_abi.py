@@ -112,6 +112,33 @@ def test_argument_errors_of_the_layout_variants_without_gpu():
     assert lib.emm_reshape_and_cache_strided(t, t, t, t, 0, P, 4, 2, 64, 16, 8, 128, 128, 4096, 128, 64, None) == 0
 
 
+def test_last_error_is_kept_per_thread():
+    """Two host threads that fail in different ways each read their own message (the text lives in
+    thread-local storage; the transfer manager calls the library from a thread of its own)."""
+    import threading
+
+    lib = _lib.load()
+    table = _lib.ptr_table([0x1000])
+    seen, start = {}, threading.Barrier(2)
+
+    def worker(name, layers, want):
+        start.wait()
+        for _ in range(200):
+            rc = lib.emm_kv_pack(table, layers, 2, 4, 64 if layers == 200 else -64, 0x1000, 1, 0x1000, None)
+            msg = lib.emm_last_error()
+            if rc != -1 or want not in msg:
+                seen[name] = msg
+                return
+        seen[name] = b"ok"
+
+    a = threading.Thread(target=worker, args=("a", 200, b"num_layers"))
+    b = threading.Thread(target=worker, args=("b", 1, b"negative"))
+    a.start(), b.start()
+    a.join(), b.join()
+    assert seen == {"a": b"ok", "b": b"ok"}
+    assert lib.emm_kv_pack(table, 1, 2, 4, 64, None, 0, None, None) == 0
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "_lib", None)
     monkeypatch.setattr(_lib, "library_path", lambda: str(tmp_path / "nope.so"))
