@@ -241,7 +241,6 @@ class BlockManager:
                 "swap": f"{len(self.swapping_gpu_blocks_list)} -> {len(self.swapping_cpu_blocks_list)}",
                 "#req": f"{len(self.block_table)}"}
 
-
     def print_block_usage(self) -> None:
         usage = self.get_block_usage()
         print(f"({self.stage}) Block usage: GPU={usage['gpu']}, CPU={usage['cpu']}, "

@@ -253,6 +253,75 @@ def test_block_manager_pool_tensors_for_a_batch(capsys):
     assert capsys.readouterr().out.strip() == "(decoding) Block usage: GPU=25% (16/64), CPU=0% (0/8), Swapping=0 -> 0, Requests=1"
 
 
+def test_block_manager_conserves_blocks_under_random_operations():
+    """2000 seeded random operations (allocate, grow, free, swap out, swap in, with a worker that records the
+    copies it is asked for): after every one of them each GPU block id and each CPU block id is in exactly one
+    place: a request's table, the free list, or the list of blocks whose copy is still in flight."""
+    import random
+
+    class Recorder:
+        def __init__(self):
+            self.copies = 0
+
+        def swap_blocks(self, request_ids, src, dst, is_swap_in):
+            assert len(src) == len(dst) and len(set(dst)) == len(dst)
+            self.copies += len(src)
+
+        def wait_for_all_swap_in(self):
+            pass
+
+        def wait_for_all_swap_out(self):
+            pass
+
+        def clear_request_resource(self, request_id):
+            pass
+
+    rng = random.Random(1234)
+    G, C = 48, 32
+    rec = Recorder()
+    bm = BlockManager(G, block_size=16, max_num_cpu_blocks=C, workers=[rec])
+    live, next_id = [], 0
+
+    def check():
+        gpu = list(bm.free_gpu_blocks_list) + list(bm.swapping_gpu_blocks_list)
+        cpu = list(bm.free_cpu_blocks_list) + list(bm.swapping_cpu_blocks_list)
+        for rid, table in bm.block_table.items():
+            (gpu if bm.get_location(rid) == BlockLocation.GPU else cpu).extend(table)
+        assert sorted(gpu) == list(range(G)) and sorted(cpu) == list(range(C))
+        assert set(bm.block_table) == set(live) == set(bm.request_location)
+
+    for _ in range(2000):
+        op = rng.choice(["alloc", "alloc", "grow", "free", "out", "in"])
+        on_gpu = [r for r in live if bm.get_location(r) == BlockLocation.GPU]
+        on_cpu = [r for r in live if bm.get_location(r) == BlockLocation.CPU]
+        if op == "alloc":
+            n = rng.randint(1, 9)
+            if bm.get_num_avail_gpu_blocks() >= n:
+                rid = f"r{next_id}"
+                next_id += 1
+                assert len(bm.allocate_blocks(rid, n)) == n
+                live.append(rid)
+        elif op == "grow" and on_gpu:
+            rid = rng.choice(on_gpu)
+            want = bm.get_allocated_num_blocks(rid) + rng.randint(0, 3)
+            if bm.get_num_avail_gpu_blocks() >= want - bm.get_allocated_num_blocks(rid):
+                assert len(bm.expand_blocks_for_seq_len(rid, want * 16)) == want
+        elif op == "free" and live:
+            rid = rng.choice(live)
+            bm.free_blocks(rid)
+            live.remove(rid)
+        elif op == "out" and on_gpu:
+            rids = rng.sample(on_gpu, min(len(on_gpu), rng.randint(1, 3)))
+            if bm.get_num_avail_cpu_blocks() >= sum(bm.get_allocated_num_blocks(r) for r in rids):
+                bm.swap_out_requests(rids)
+        elif op == "in" and on_cpu:
+            rids = rng.sample(on_cpu, min(len(on_cpu), rng.randint(1, 3)))
+            if bm.get_num_avail_gpu_blocks() >= sum(bm.get_allocated_num_blocks(r) for r in rids):
+                bm.swap_in_requests(rids)
+        check()
+    assert rec.copies > 100 and next_id > 100
+
+
 def test_block_manager_swap_bookkeeping_and_worker_calls():
     rec = _SwapRecorder()
     bm = BlockManager(6, block_size=16, max_num_cpu_blocks=5, workers=[rec])
