@@ -210,6 +210,7 @@ constexpr int kPack = 0, kUnpack = 1, kPoolToPool = 2;
 //           sides are pools (about 12 % faster there; slower with a linear side, which would be
 //           read as one stream per plane).
 constexpr int kOrderPlain = 0, kOrderGrouped = 1, kOrderRuns = 2;
+constexpr uint32_t kXcdRemap = 0x80000000u; // flag in `order_arg`: keep the tiles of a chunk on one XCD
 
 // idx_a / idx_b: source / destination ids (PAIRS: idx_a holds (src, dst) pairs, idx_b unused).
 // `n` = blocks of this launch (ids and linear buffer already offset to its first block),
@@ -223,21 +224,38 @@ __global__ __launch_bounds__(kThreads) void emm_block_move_kernel(
     const std::conditional_t<INLINE, InlineIds, NoIds> ids) {
   constexpr int64_t TILE = (int64_t)U * kThreads * sizeof(V);
   constexpr bool SRC_POOL = KIND != kUnpack, DST_POOL = KIND != kPack;
+  // The tiles of one chunk on one XCD. Workgroups go to the 8 XCDs round-robin in dispatch order (x fastest), so
+  // the tiles of a 16 KiB chunk would land on 4 different XCDs, and each XCD's translation cache (UTCL2) would fetch
+  // the same page entry by itself: a table of random blocks hits a different page with almost every chunk.
+  // Inside every group of 8 chunks (8 * tiles-per-chunk consecutive workgroups) workgroup q takes tile q / 8 of
+  // chunk q % 8: workgroups 8 apart in dispatch order, hence on one XCD, share a chunk. A bijection on (x, y)
+  // inside the group; what is left of y past the last whole group keeps the plain mapping.
+  uint32_t bx = blockIdx.x, by = blockIdx.y;
+  if (order_arg & kXcdRemap) {
+    const uint32_t tpc = (uint32_t)((chunk + TILE - 1) / TILE); // = gridDim.x (TILE is a power of two)
+    const uint32_t whole = ORDER == kOrderPlain ? (n & ~7u) : ~7u; // grouped / runs: y is a multiple of 8 per plane
+    if (by < whole) {
+      const uint32_t q = bx + tpc * (by & 7u);
+      by = (by & ~7u) | (q & 7u);
+      bx = q >> 3;
+    }
+  }
+  order_arg &= ~kXcdRemap;
   uint32_t pl, j;
   if constexpr (ORDER == kOrderRuns) {
-    pl = blockIdx.y / kRun;
+    pl = by / kRun;
     const uint32_t runs = (n + kRun - 1) / kRun;
     uint32_t run = blockIdx.z + pl * order_arg; // order_arg = runs / planes
     if (run >= runs) run -= runs;
-    j = run * kRun + (blockIdx.y % kRun);
+    j = run * kRun + (by % kRun);
     if (j >= n) return;
   } else if constexpr (ORDER == kOrderGrouped) {
-    pl = blockIdx.y >> order_arg;
-    j = (blockIdx.z << order_arg) + (blockIdx.y & ((1u << order_arg) - 1u));
+    pl = by >> order_arg;
+    j = (blockIdx.z << order_arg) + (by & ((1u << order_arg) - 1u));
     if (j >= n) return;
   } else {
     pl = blockIdx.z;
-    j = blockIdx.y;
+    j = by;
   }
   // round trip 1: ids and plane bases, all issued before the one wait below
   int64_t sb = 0, db = 0;
@@ -257,7 +275,7 @@ __global__ __launch_bounds__(kThreads) void emm_block_move_kernel(
   if constexpr (SRC_POOL) src_plane = tables.t[0].base[pl];
   if constexpr (DST_POOL) dst_plane = tables.t[KIND == kPoolToPool ? 1 : 0].base[pl];
 
-  const int64_t tile_off = (int64_t)blockIdx.x * TILE;
+  const int64_t tile_off = (int64_t)bx * TILE;
   const int64_t limit = FULL ? TILE : chunk - tile_off;
   char *linp = nullptr;
   if constexpr (KIND != kPoolToPool) linp = lin + (int64_t)pl * lin_plane_stride + (int64_t)j * chunk + tile_off;
@@ -306,6 +324,22 @@ struct MoveArgs {
   uint32_t src_nb, dst_nb;
 };
 
+// Whether a launch keeps the tiles of a chunk on one XCD (kXcdRemap). It pays where translations are the limiter and
+// costs where they are not (the workgroups that start together then read or write 8 chunks at once instead of 2):
+//  * both sides pools (migrate, copy_blocks): always; measured +0.3 .. +1.5 % on 16 KiB chunks of the Qwen2-7B pool,
+//    +2 .. +3 % on the 80-layer fp8 pool, +3 .. +6 % on 32 KiB chunks;
+//  * one side the transfer buffer (pack, unpack, dequantising unpack): only for a table so short that a visit to a
+//    plane touches most of its 2 MiB pages once: blocks * 2 MiB <= 3/4 of the plane's bytes. There per-request packs
+//    gain +0.3 .. +1.9 % and unpacks +0.1 .. +1.0 %; above (ratio 1 .. 16) packs lose 1 .. 8 % and unpacks up to 2 %.
+//    Launches of fewer than 96 blocks are left alone (their time is the launch ramp).
+// Benchmark builds can switch it off (bit 25) or on (bit 26) everywhere.
+bool xcd_remap_pays(bool pool_to_pool, int64_t n, int64_t pool_blocks, int64_t chunk) {
+  if (move_variant() & 0x2000000) return false;
+  if (move_variant() & 0x4000000) return true;
+  if (pool_to_pool) return true;
+  return n >= 96 && (n << 21) / 3 <= pool_blocks * chunk / 4;
+}
+
 template <typename V, int U, int KIND, int ORDER, bool PAIRS, int POLICY>
 void launch_move_full(const MoveArgs &a, uint32_t n, uint32_t order_arg, dim3 grid, bool full,
                       const PlaneTables<KIND == kPoolToPool ? 2 : 1> &t, hipStream_t s) {
@@ -318,14 +352,14 @@ void launch_move_full(const MoveArgs &a, uint32_t n, uint32_t order_arg, dim3 gr
 }
 
 template <typename V, int U, int KIND, int POLICY>
-void launch_move_inline(const MoveArgs &a, uint32_t n, dim3 grid, bool full, const PlaneTables<1> &t,
-                        const InlineIds &ids, hipStream_t s) {
+void launch_move_inline(const MoveArgs &a, uint32_t n, uint32_t order_arg, dim3 grid, bool full,
+                        const PlaneTables<1> &t, const InlineIds &ids, hipStream_t s) {
   if (full)
     emm_block_move_kernel<V, U, KIND, kOrderPlain, true, false, POLICY, true><<<grid, kThreads, 0, s>>>(
-        nullptr, nullptr, a.lin, a.lin_plane_stride, a.chunk, a.src_nb, a.dst_nb, n, 0, t, ids);
+        nullptr, nullptr, a.lin, a.lin_plane_stride, a.chunk, a.src_nb, a.dst_nb, n, order_arg, t, ids);
   else
     emm_block_move_kernel<V, U, KIND, kOrderPlain, false, false, POLICY, true><<<grid, kThreads, 0, s>>>(
-        nullptr, nullptr, a.lin, a.lin_plane_stride, a.chunk, a.src_nb, a.dst_nb, n, 0, t, ids);
+        nullptr, nullptr, a.lin, a.lin_plane_stride, a.chunk, a.src_nb, a.dst_nb, n, order_arg, t, ids);
 }
 
 template <int KIND, int ORDER, bool PAIRS>
@@ -417,13 +451,14 @@ int move_planes(const void *const *src_layers, int64_t src_nb, void *const *dst_
       a.chunk = chunk;
       a.src_nb = (uint32_t)src_nb;
       a.dst_nb = (uint32_t)dst_nb;
+      const uint32_t remap = xcd_remap_pays(KIND == kPoolToPool, ny, SP ? src_nb : dst_nb, chunk) ? kXcdRemap : 0u;
       if constexpr (KIND != kPoolToPool) {
         if (host_ids) { // at most EMM_MAX_INLINE_IDS blocks per launch, plain order
           const dim3 grid((uint32_t)tpc, (uint32_t)ny, (uint32_t)cnt);
-          if (vec == 16) launch_move_inline<u32x4, 1, KIND, 1>(a, (uint32_t)ny, grid, full, t, inline_ids, s);
-          else if (vec == 4) launch_move_inline<uint32_t, 4, KIND, 0>(a, (uint32_t)ny, grid, false, t, inline_ids, s);
-          else if (vec == 2) launch_move_inline<uint16_t, 4, KIND, 0>(a, (uint32_t)ny, grid, false, t, inline_ids, s);
-          else launch_move_inline<uint8_t, 4, KIND, 0>(a, (uint32_t)ny, grid, false, t, inline_ids, s);
+          if (vec == 16) launch_move_inline<u32x4, 1, KIND, 1>(a, (uint32_t)ny, remap, grid, full, t, inline_ids, s);
+          else if (vec == 4) launch_move_inline<uint32_t, 4, KIND, 0>(a, (uint32_t)ny, remap, grid, false, t, inline_ids, s);
+          else if (vec == 2) launch_move_inline<uint16_t, 4, KIND, 0>(a, (uint32_t)ny, remap, grid, false, t, inline_ids, s);
+          else launch_move_inline<uint8_t, 4, KIND, 0>(a, (uint32_t)ny, remap, grid, false, t, inline_ids, s);
           const int rc = check_launch(what);
           if (rc != EMM_OK) return rc;
           continue;
@@ -432,8 +467,8 @@ int move_planes(const void *const *src_layers, int64_t src_nb, void *const *dst_
       if constexpr (KIND == kPoolToPool) {
         const uint32_t runs = (uint32_t)((ny + kRun - 1) / kRun);
         const dim3 grid((uint32_t)tpc, (uint32_t)(cnt * kRun), runs);
-        if (pairs) launch_move_vec<KIND, kOrderRuns, true>(a, (uint32_t)ny, runs / cnt, grid, vec, policy, full, t, s);
-        else launch_move_vec<KIND, kOrderRuns, false>(a, (uint32_t)ny, runs / cnt, grid, vec, policy, full, t, s);
+        if (pairs) launch_move_vec<KIND, kOrderRuns, true>(a, (uint32_t)ny, runs / cnt | remap, grid, vec, policy, full, t, s);
+        else launch_move_vec<KIND, kOrderRuns, false>(a, (uint32_t)ny, runs / cnt | remap, grid, vec, policy, full, t, s);
       } else {
         // long scatters (unpack) are walked in groups of 256 blocks per plane visit (6712 blocks in one
         // launch: 6.41-6.50 TB/s; groups of 128: 6.16-6.29, of 512: 6.34, of 64: 5.73; plain order 6.40-6.46 on a
@@ -445,10 +480,11 @@ int move_planes(const void *const *src_layers, int64_t src_nb, void *const *dst_
         if (forced) glog = forced == 0xf ? 0 : forced;
         if (glog > 0 && ((int64_t)cnt << glog) <= kMaxGridY) {
           const dim3 grid((uint32_t)tpc, (uint32_t)(cnt << glog), (uint32_t)((ny + (1 << glog) - 1) >> glog));
-          launch_move_vec<KIND, kOrderGrouped, false>(a, (uint32_t)ny, (uint32_t)glog, grid, vec, policy, full, t, s);
+          launch_move_vec<KIND, kOrderGrouped, false>(a, (uint32_t)ny, (uint32_t)glog | (glog >= 3 ? remap : 0u), grid, vec, policy, full, t,
+                                                          s);
         } else {
           const dim3 grid((uint32_t)tpc, (uint32_t)ny, (uint32_t)cnt);
-          launch_move_vec<KIND, kOrderPlain, false>(a, (uint32_t)ny, 0, grid, vec, policy, full, t, s);
+          launch_move_vec<KIND, kOrderPlain, false>(a, (uint32_t)ny, remap, grid, vec, policy, full, t, s);
         }
       }
       const int rc = check_launch(what);
@@ -678,17 +714,29 @@ __global__ __launch_bounds__(kThreads) void emm_unpack_dequant_fp8_kernel(
     uint32_t n, uint32_t group_log2, const LayerTable layers) {
   constexpr uint32_t TILE = kThreads * 16;
   const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // the tiles of one chunk on one XCD, as in emm_block_move_kernel
+  uint32_t bx = blockIdx.x, by = blockIdx.y;
+  if (group_log2 & kXcdRemap) {
+    const uint32_t tpc = (chunk + TILE - 1) / TILE;
+    const uint32_t whole = GROUPED ? ~7u : (n & ~7u);
+    if (by < whole) {
+      const uint32_t q = bx + tpc * (by & 7u);
+      by = (by & ~7u) | (q & 7u);
+      bx = q >> 3;
+    }
+  }
+  group_log2 &= ~kXcdRemap;
   uint32_t pl, j;
   if constexpr (GROUPED) {
-    pl = blockIdx.y >> group_log2;
-    j = (blockIdx.z << group_log2) + (blockIdx.y & ((1u << group_log2) - 1u));
+    pl = by >> group_log2;
+    j = (blockIdx.z << group_log2) + (by & ((1u << group_log2) - 1u));
     if (j >= n) return;
   } else {
     pl = blockIdx.z;
-    j = blockIdx.y;
+    j = by;
   }
   const uint32_t l = pl >> 1, kv = pl & 1;
-  const uint32_t off0 = blockIdx.x * TILE + wave * 1024 + lane * 8;
+  const uint32_t off0 = bx * TILE + wave * 1024 + lane * 8;
   const uint32_t off1 = off0 + 512;
   const bool live0 = off0 < chunk, live1 = off1 < chunk; // chunk is a multiple of 16
   const char *src = packed + (int64_t)pl * plane_stride + (uint64_t)j * chunk;
@@ -1754,11 +1802,12 @@ int emm_kv_unpack_dequant_fp8(void *const *layer_ptrs, int num_layers, int64_t n
     const int64_t *idx = block_idx + j0;
     const int64_t stride = n * chunk_elems;
     const bool grouped = ny >= 1024 && ((2 * num_layers) << 8) <= kMaxGridY; // groups of 256 blocks, as in unpack
+    const uint32_t remap = xcd_remap_pays(false, ny, num_blocks, 2 * chunk_elems) ? kXcdRemap : 0u;
     const dim3 grid = grouped ? dim3((uint32_t)tpc, (uint32_t)((2 * num_layers) << 8), (uint32_t)((ny + 255) >> 8))
                               : dim3((uint32_t)tpc, (uint32_t)ny, (uint32_t)(2 * num_layers));
 #define EMM_DQ_LAUNCH(DT, G) \
   emm_unpack_dequant_fp8_kernel<DT, G><<<grid, kThreads, 0, s>>>(packed, idx, k_scales, v_scales, stride, \
-      (uint32_t)chunk_elems, (uint32_t)num_blocks, (uint32_t)ny, 8u, t)
+      (uint32_t)chunk_elems, (uint32_t)num_blocks, (uint32_t)ny, 8u | remap, t)
     if (out_dtype == EMM_DTYPE_BF16) { if (grouped) EMM_DQ_LAUNCH(EMM_DTYPE_BF16, true); else EMM_DQ_LAUNCH(EMM_DTYPE_BF16, false); }
     else { if (grouped) EMM_DQ_LAUNCH(EMM_DTYPE_F16, true); else EMM_DQ_LAUNCH(EMM_DTYPE_F16, false); }
 #undef EMM_DQ_LAUNCH
@@ -2011,7 +2060,7 @@ extern "C" {
 
 int emm_hook_set_move_variant(int variant) {
   const int old = g_move_variant;
-  g_move_variant = variant & 0x13fff00;
+  g_move_variant = variant & 0x73fff00;
   return old;
 }
 

@@ -22,7 +22,10 @@ extern "C" {
  *   0 = default ((4, 1) for a per-layer launch, (1, 1) for a whole-step launch), 1 = (1, 4), 2 = (2, 4),
  *   3 = (4, 1), 4 = (1, 1), 5 = (2, 1);
  * bits 16-19: log2 of the blocks per plane visit of pack / unpack (15 = plain order);
- * bit 24: fp8 append with the IEEE division instead of the reciprocal form.
+ * bits 20-21: token tile of the paged-layout append (1 = 16 tokens, 2 = 4 tokens; 0 = by token count);
+ * bit 24: fp8 append with the IEEE division instead of the reciprocal form;
+ * bit 25 / bit 26: never / always keep the tiles of a chunk on one XCD in the block moves (default: by table
+ *   length and plane size).
  * Process-wide, not thread-safe. Returns the previous value. */
 int emm_hook_set_move_variant(int variant);
 
