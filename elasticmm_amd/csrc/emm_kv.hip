@@ -225,11 +225,11 @@ __global__ __launch_bounds__(kThreads) void emm_block_move_kernel(
   constexpr int64_t TILE = (int64_t)U * kThreads * sizeof(V);
   constexpr bool SRC_POOL = KIND != kUnpack, DST_POOL = KIND != kPack;
   // The tiles of one chunk on one XCD. Workgroups go to the 8 XCDs round-robin in dispatch order (x fastest), so
-  // the tiles of a 16 KiB chunk would land on 4 different XCDs, and each XCD's translation cache (UTCL2) would fetch
-  // the same page entry by itself: a table of random blocks hits a different page with almost every chunk.
-  // Inside every group of 8 chunks (8 * tiles-per-chunk consecutive workgroups) workgroup q takes tile q / 8 of
-  // chunk q % 8: workgroups 8 apart in dispatch order, hence on one XCD, share a chunk. A bijection on (x, y)
-  // inside the group; what is left of y past the last whole group keeps the plain mapping.
+  // the tiles of a 16 KiB chunk would land on 4 different XCDs. Inside every group of 8 chunks (8 * tiles-per-chunk
+  // consecutive workgroups) workgroup q takes tile q / 8 of chunk q % 8 instead: workgroups 8 apart in dispatch
+  // order, hence on one XCD, share a chunk, and every XCD asks the memory for whole chunks. A bijection on (x, y)
+  // inside the group; what is left of y past the last whole group keeps the plain mapping. The host decides per
+  // launch (xcd_remap_pays below).
   uint32_t bx = blockIdx.x, by = blockIdx.y;
   if (order_arg & kXcdRemap) {
     const uint32_t tpc = (uint32_t)((chunk + TILE - 1) / TILE); // = gridDim.x (TILE is a power of two)
@@ -324,14 +324,17 @@ struct MoveArgs {
   uint32_t src_nb, dst_nb;
 };
 
-// Whether a launch keeps the tiles of a chunk on one XCD (kXcdRemap). It pays where translations are the limiter and
-// costs where they are not (the workgroups that start together then read or write 8 chunks at once instead of 2):
-//  * both sides pools (migrate, copy_blocks): always; measured +0.3 .. +1.5 % on 16 KiB chunks of the Qwen2-7B pool,
-//    +2 .. +3 % on the 80-layer fp8 pool, +3 .. +6 % on 32 KiB chunks;
-//  * one side the transfer buffer (pack, unpack, dequantising unpack): only for a table so short that a visit to a
-//    plane touches most of its 2 MiB pages once: blocks * 2 MiB <= 3/4 of the plane's bytes. There per-request packs
-//    gain +0.3 .. +1.9 % and unpacks +0.1 .. +1.0 %; above (ratio 1 .. 16) packs lose 1 .. 8 % and unpacks up to 2 %.
-//    Launches of fewer than 96 blocks are left alone (their time is the launch ramp).
+// Whether a launch keeps the tiles of a chunk on one XCD (kXcdRemap). Measured by alternating both mappings on the
+// same pools in one process:
+//  * both sides pools (migrate, copy_blocks): always; +0.3 .. +1.5 % on 16 KiB chunks of the Qwen2-7B pool,
+//    +2 .. +3 % on the 80-layer fp8 pool, +3 .. +6 % on 32 KiB chunks, never a loss;
+//  * one side the transfer buffer (pack, unpack, dequantising unpack): only for a table that is short against the
+//    plane it indexes: blocks * 2 MiB <= 3/4 of the plane's bytes. There per-request packs gain +0.3 .. +1.9 % and
+//    unpacks +0.1 .. +1.0 %; above (ratio 1 .. 16) the remap loses 1 .. 8 % on packs and up to 2 % on unpacks (the
+//    workgroups that start together then touch 8 places of the transfer buffer instead of 2). Launches of fewer
+//    than 96 blocks are left alone (their time is the launch ramp).
+// The translation counters (UTCL1 misses, UTCL2 busy) read the same with both mappings, so the gain is not fewer
+// page-table fetches; what changes is that each XCD requests 16 KiB contiguous instead of 4 KiB.
 // Benchmark builds can switch it off (bit 25) or on (bit 26) everywhere.
 bool xcd_remap_pays(bool pool_to_pool, int64_t n, int64_t pool_blocks, int64_t chunk) {
   if (move_variant() & 0x2000000) return false;
