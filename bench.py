@@ -473,6 +473,32 @@ def batched(src_w, dst_w, dev_tables, payload, L, chunk, NB, dev):
     out["per_request_pack_then_unpack_interleaved"] = rec(
         4 * payload, med, 2 * len(dev_tables), note="each buffer unpacked right after its pack: partly read back from "
                                                     "the 256 MB last-level cache, not the headline")
+    # per-request launches alternating over two streams of the same priority: the drain of one launch overlaps the
+    # ramp of the next (the kernels take the current stream, so a caller can do this with the product as it is)
+    bufs2 = [torch.empty(sp.packed_shape(s.numel()), dtype=sp.dtype, device=dev) for s, _ in dev_tables]
+    side = torch.cuda.Stream()
+
+    def fan_out(fn):
+        main = torch.cuda.current_stream()
+        side.wait_stream(main)
+        for i, (tab, b) in enumerate(zip(dev_tables, bufs2)):
+            if i & 1:
+                with torch.cuda.stream(side):
+                    fn(tab, b)
+            else:
+                fn(tab, b)
+        main.wait_stream(side)
+
+    med_p, _ = timed(lambda: fan_out(lambda tab, b: kv_ops.kv_pack(sp, tab[0], out=b)), 10)
+    med_u, _ = timed(lambda: fan_out(lambda tab, b: kv_ops.kv_unpack(dp, tab[1], b)), 10)
+    med_p1, _ = timed(lambda: [kv_ops.kv_pack(sp, tab[0], out=b) for tab, b in zip(dev_tables, bufs2)], 10)
+    med_u1, _ = timed(lambda: [kv_ops.kv_unpack(dp, tab[1], b) for tab, b in zip(dev_tables, bufs2)], 10)
+    out["per_request_two_streams"] = {
+        "pack": rec(2 * payload, med_p, len(dev_tables)), "unpack": rec(2 * payload, med_u, len(dev_tables)),
+        "pack_one_stream": rec(2 * payload, med_p1, len(dev_tables)),
+        "unpack_one_stream": rec(2 * payload, med_u1, len(dev_tables)),
+        "note": "the same 32 per-request launches alternating over two streams against one stream, same buffers"}
+    del bufs2
     flat = buf.view(-1)
     other = torch.empty_like(flat)
     med, _ = timed(lambda: kv_ops.stream_copy(flat, other), 10)
