@@ -25,7 +25,8 @@ fraction of the 8 TB/s peak, kernel name and average launch time:
                      what the scalar fetches in front of a pack's loads cost
   list_indices       the headline with block tables passed as Python lists (the reference's
                      call shape; the ids travel in the kernel argument block)
-  batched / fused    one launch for the whole batch; fused pool-to-pool migrate; copy_blocks
+  batched / fused    one launch for the whole batch; fused pool-to-pool migrate; copy_blocks;
+                     the per-request launches alternating over two streams against one
   ceilings           what this memory system does for the same access patterns without the
                      other half of the copy (sequential / gathered reads, sequential /
                      scattered writes, plain copy), from the hooks build of the library
