@@ -340,7 +340,7 @@ bool xcd_remap_pays(bool pool_to_pool, int64_t n, int64_t pool_blocks, int64_t c
   if (move_variant() & 0x2000000) return false;
   if (move_variant() & 0x4000000) return true;
   if (pool_to_pool) return true;
-  return n >= 96 && (n << 21) / 3 <= pool_blocks * chunk / 4;
+  return n >= 96 && (double)n * 2097152.0 * 4.0 <= (double)pool_blocks * (double)chunk * 3.0; // no overflow for any sizes
 }
 
 template <typename V, int U, int KIND, int ORDER, bool PAIRS, int POLICY>
