@@ -210,7 +210,30 @@ constexpr int kPack = 0, kUnpack = 1, kPoolToPool = 2;
 //           sides are pools (about 12 % faster there; slower with a linear side, which would be
 //           read as one stream per plane).
 constexpr int kOrderPlain = 0, kOrderGrouped = 1, kOrderRuns = 2;
-constexpr uint32_t kXcdRemap = 0x80000000u; // flag in `order_arg`: keep the tiles of a chunk on one XCD
+// Tile -> XCD mappings, flags in the top bits of `order_arg`. Workgroups go to the 8 XCDs round-robin in dispatch
+// order (x fastest), so with the plain mapping every XCD takes every eighth 4 KiB tile and the tiles of a 16 KiB
+// chunk land on 4 XCDs. Inside every window of 8 chunks (8 * tiles-per-chunk consecutive workgroups):
+//   kXcdPairs  the workgroups q and q + 8 of every 16 take two neighbouring tiles: every XCD requests 8 KiB
+//              contiguous (tiles per chunk must be even);
+//   kXcdChunk  workgroup q takes tile q / 8 of chunk q % 8: every XCD requests whole chunks.
+// Both are bijections on the window's (x, y); what is left of y past the last whole window keeps the plain
+// mapping. The host decides per launch (xcd_mapping below).
+constexpr uint32_t kXcdChunk = 0x80000000u, kXcdPairs = 0x40000000u, kXcdMask = kXcdChunk | kXcdPairs;
+
+// (bx, by) of the tile this workgroup moves. `whole` = the y covered by whole windows of 8.
+__device__ __forceinline__ void xcd_map(uint32_t mode, uint32_t tpc, uint32_t whole, uint32_t &bx, uint32_t &by) {
+  if (!(mode & kXcdMask) || by >= whole) return;
+  const uint32_t lin = bx + tpc * (by & 7u); // position in the window
+  if (mode & kXcdChunk) {
+    by = (by & ~7u) | (lin & 7u);
+    bx = lin >> 3;
+  } else {
+    const uint32_t t = (lin & ~15u) + 2u * (lin & 7u) + ((lin >> 3) & 1u); // 8 * tpc is a multiple of 16
+    const uint32_t c = (tpc & (tpc - 1u)) == 0u ? t >> __builtin_ctz(tpc) : t / tpc;
+    by = (by & ~7u) + c;
+    bx = t - c * tpc;
+  }
+}
 
 // idx_a / idx_b: source / destination ids (PAIRS: idx_a holds (src, dst) pairs, idx_b unused).
 // `n` = blocks of this launch (ids and linear buffer already offset to its first block),
@@ -224,23 +247,10 @@ __global__ __launch_bounds__(kThreads) void emm_block_move_kernel(
     const std::conditional_t<INLINE, InlineIds, NoIds> ids) {
   constexpr int64_t TILE = (int64_t)U * kThreads * sizeof(V);
   constexpr bool SRC_POOL = KIND != kUnpack, DST_POOL = KIND != kPack;
-  // The tiles of one chunk on one XCD. Workgroups go to the 8 XCDs round-robin in dispatch order (x fastest), so
-  // the tiles of a 16 KiB chunk would land on 4 different XCDs. Inside every group of 8 chunks (8 * tiles-per-chunk
-  // consecutive workgroups) workgroup q takes tile q / 8 of chunk q % 8 instead: workgroups 8 apart in dispatch
-  // order, hence on one XCD, share a chunk, and every XCD asks the memory for whole chunks. A bijection on (x, y)
-  // inside the group; what is left of y past the last whole group keeps the plain mapping. The host decides per
-  // launch (xcd_remap_pays below).
   uint32_t bx = blockIdx.x, by = blockIdx.y;
-  if (order_arg & kXcdRemap) {
-    const uint32_t tpc = (uint32_t)((chunk + TILE - 1) / TILE); // = gridDim.x (TILE is a power of two)
-    const uint32_t whole = ORDER == kOrderPlain ? (n & ~7u) : ~7u; // grouped / runs: y is a multiple of 8 per plane
-    if (by < whole) {
-      const uint32_t q = bx + tpc * (by & 7u);
-      by = (by & ~7u) | (q & 7u);
-      bx = q >> 3;
-    }
-  }
-  order_arg &= ~kXcdRemap;
+  xcd_map(order_arg, (uint32_t)((chunk + TILE - 1) / TILE) /* = gridDim.x */,
+          ORDER == kOrderPlain ? (n & ~7u) : ~7u /* grouped / runs: y is a multiple of 8 per plane */, bx, by);
+  order_arg &= ~kXcdMask;
   uint32_t pl, j;
   if constexpr (ORDER == kOrderRuns) {
     pl = by / kRun;
@@ -324,23 +334,32 @@ struct MoveArgs {
   uint32_t src_nb, dst_nb;
 };
 
-// Whether a launch keeps the tiles of a chunk on one XCD (kXcdRemap). Measured by alternating both mappings on the
-// same pools in one process:
-//  * both sides pools (migrate, copy_blocks): always; +0.3 .. +1.5 % on 16 KiB chunks of the Qwen2-7B pool,
-//    +2 .. +3 % on the 80-layer fp8 pool, +3 .. +6 % on 32 KiB chunks, never a loss;
-//  * one side the transfer buffer (pack, unpack, dequantising unpack): only for a table that is short against the
-//    plane it indexes: blocks * 2 MiB <= 3/4 of the plane's bytes. There per-request packs gain +0.3 .. +1.9 % and
-//    unpacks +0.1 .. +1.0 %; above (ratio 1 .. 16) the remap loses 1 .. 8 % on packs and up to 2 % on unpacks (the
-//    workgroups that start together then touch 8 places of the transfer buffer instead of 2). Launches of fewer
-//    than 96 blocks are left alone (their time is the launch ramp).
-// The translation counters (UTCL1 misses, UTCL2 busy) read the same with both mappings, so the gain is not fewer
-// page-table fetches; what changes is that each XCD requests 16 KiB contiguous instead of 4 KiB.
-// Benchmark builds can switch it off (bit 25) or on (bit 26) everywhere.
-bool xcd_remap_pays(bool pool_to_pool, int64_t n, int64_t pool_blocks, int64_t chunk) {
-  if (move_variant() & 0x2000000) return false;
-  if (move_variant() & 0x4000000) return true;
-  if (pool_to_pool) return true;
-  return n >= 96 && (double)n * 2097152.0 * 4.0 <= (double)pool_blocks * (double)chunk * 3.0; // no overflow for any sizes
+// The tile -> XCD mapping of a launch (kXcdPairs, kXcdChunk or 0). Measured by alternating the mappings on the same
+// pools in one process, tables of 32 .. 4096 random blocks, against the plain mapping:
+//  * unpack: pairs +0.5 .. +1.6 % on the Qwen2-7B pool (16 KiB chunks, 983 MB planes), +0.7 .. +3.0 % on the 80-layer
+//    fp8 pool (327 MB planes); two cells of -0.6 / -0.7 % on other shapes;
+//  * both sides pools (migrate, copy_blocks): pairs +0.2 .. +1.3 % on the Qwen2-7B pool, +1.3 .. +2.9 % on the 80-layer
+//    fp8 pool; from 32 KiB chunks on whole chunks do better (+2 .. +6.9 % against +1.2 .. +4.5 %); copy_blocks in a
+//    200 GB pool +1.2 .. +1.5 % at 512 and 4096 pairs, -0.3 % at 54 500;
+//  * pack: pairs gain while the table is short against the plane it indexes and lose when it is not: Qwen2-7B pool
+//    +1.0 / +2.1 / +2.3 / +1.6 / +0.7 % at 128 / 256 / 512 / 1000 / 2048 blocks, 80-layer fp8 pool +1.3 / -0.6 / -1.5 /
+//    -1.6 / -2.2 %. The transfer-buffer side of a pack is a sequential stream, which wants the XCDs side by side on
+//    4 KiB pieces (a plain copy loses 3 % with 8 KiB per XCD and 9 % with 16 KiB); the sparser the gather, the more
+//    its side counts. Pairs are used up to blocks * 2 MiB = 1.25 x the plane's bytes. Whole chunks lose up to 8 %.
+//  * the dequantising unpack keeps the plain mapping (pairs: 0 .. -0.4 % on the 80-layer pool).
+// Launches of fewer than 96 blocks are left alone (their time is the launch ramp). The translation counters (UTCL1
+// misses, UTCL2 busy) read the same with every mapping: the gain is not fewer page-table fetches; what changes is
+// what each XCD requests at a time. Benchmark builds can force plain (bit 25), whole chunks (26) or pairs (27).
+constexpr int kMapPack = 0, kMapUnpack = 1, kMapPoolToPool = 2, kMapDequant = 3;
+uint32_t xcd_mapping(int kind, int64_t n, int64_t tpc, int64_t pool_blocks, int64_t chunk) {
+  if (move_variant() & 0x2000000) return 0u;
+  if (move_variant() & 0x4000000) return kXcdChunk;
+  if (move_variant() & 0x8000000) return tpc % 2 == 0 ? kXcdPairs : 0u;
+  if (n < 96 || tpc < 2 || kind == kMapDequant) return 0u;
+  if (kind == kMapPoolToPool) return tpc >= 8 || tpc % 2 ? kXcdChunk : kXcdPairs;
+  if (tpc % 2) return 0u;
+  if (kind == kMapPack && (double)n * 2097152.0 > 1.25 * (double)pool_blocks * (double)chunk) return 0u;
+  return kXcdPairs;
 }
 
 template <typename V, int U, int KIND, int ORDER, bool PAIRS, int POLICY>
@@ -454,7 +473,8 @@ int move_planes(const void *const *src_layers, int64_t src_nb, void *const *dst_
       a.chunk = chunk;
       a.src_nb = (uint32_t)src_nb;
       a.dst_nb = (uint32_t)dst_nb;
-      const uint32_t remap = xcd_remap_pays(KIND == kPoolToPool, ny, SP ? src_nb : dst_nb, chunk) ? kXcdRemap : 0u;
+      const uint32_t remap = xcd_mapping(KIND == kPoolToPool ? kMapPoolToPool : KIND == kPack ? kMapPack : kMapUnpack, ny, tpc,
+                                          SP ? src_nb : dst_nb, chunk);
       if constexpr (KIND != kPoolToPool) {
         if (host_ids) { // at most EMM_MAX_INLINE_IDS blocks per launch, plain order
           const dim3 grid((uint32_t)tpc, (uint32_t)ny, (uint32_t)cnt);
@@ -717,18 +737,9 @@ __global__ __launch_bounds__(kThreads) void emm_unpack_dequant_fp8_kernel(
     uint32_t n, uint32_t group_log2, const LayerTable layers) {
   constexpr uint32_t TILE = kThreads * 16;
   const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  // the tiles of one chunk on one XCD, as in emm_block_move_kernel
   uint32_t bx = blockIdx.x, by = blockIdx.y;
-  if (group_log2 & kXcdRemap) {
-    const uint32_t tpc = (chunk + TILE - 1) / TILE;
-    const uint32_t whole = GROUPED ? ~7u : (n & ~7u);
-    if (by < whole) {
-      const uint32_t q = bx + tpc * (by & 7u);
-      by = (by & ~7u) | (q & 7u);
-      bx = q >> 3;
-    }
-  }
-  group_log2 &= ~kXcdRemap;
+  xcd_map(group_log2, (chunk + TILE - 1) / TILE, GROUPED ? ~7u : (n & ~7u), bx, by); // as in emm_block_move_kernel
+  group_log2 &= ~kXcdMask;
   uint32_t pl, j;
   if constexpr (GROUPED) {
     pl = by >> group_log2;
@@ -1805,7 +1816,7 @@ int emm_kv_unpack_dequant_fp8(void *const *layer_ptrs, int num_layers, int64_t n
     const int64_t *idx = block_idx + j0;
     const int64_t stride = n * chunk_elems;
     const bool grouped = ny >= 1024 && ((2 * num_layers) << 8) <= kMaxGridY; // groups of 256 blocks, as in unpack
-    const uint32_t remap = xcd_remap_pays(false, ny, num_blocks, 2 * chunk_elems) ? kXcdRemap : 0u;
+    const uint32_t remap = xcd_mapping(kMapDequant, ny, tpc, num_blocks, 2 * chunk_elems);
     const dim3 grid = grouped ? dim3((uint32_t)tpc, (uint32_t)((2 * num_layers) << 8), (uint32_t)((ny + 255) >> 8))
                               : dim3((uint32_t)tpc, (uint32_t)ny, (uint32_t)(2 * num_layers));
 #define EMM_DQ_LAUNCH(DT, G) \
@@ -2063,7 +2074,7 @@ extern "C" {
 
 int emm_hook_set_move_variant(int variant) {
   const int old = g_move_variant;
-  g_move_variant = variant & 0x73fff00;
+  g_move_variant = variant & 0xf3fff00;
   return old;
 }
 

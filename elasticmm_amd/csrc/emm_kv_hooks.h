@@ -24,8 +24,8 @@ extern "C" {
  * bits 16-19: log2 of the blocks per plane visit of pack / unpack (15 = plain order);
  * bits 20-21: token tile of the paged-layout append (1 = 16 tokens, 2 = 4 tokens; 0 = by token count);
  * bit 24: fp8 append with the IEEE division instead of the reciprocal form;
- * bit 25 / bit 26: never / always keep the tiles of a chunk on one XCD in the block moves (default: by table
- *   length and plane size).
+ * bits 25 / 26 / 27: tile-to-XCD mapping of the block moves forced to plain / whole chunks per XCD / pairs of tiles
+ *   per XCD (default: chosen per launch by kind, table length, tiles per chunk and plane size).
  * Process-wide, not thread-safe. Returns the previous value. */
 int emm_hook_set_move_variant(int variant);
 

@@ -299,6 +299,76 @@ def test_block_moves_seeded_sweep_of_shapes():
             assert same_bits(torch.stack(src_g), torch.stack(src_c)), f"copy_blocks, case {case}"
 
 
+@pytest.mark.parametrize("bs,H,D,desc", [
+    (16, 1, 128, "4 KiB chunks: one tile"), (16, 2, 128, "8 KiB: two tiles"), (16, 3, 128, "12 KiB: three tiles"),
+    (16, 4, 128, "16 KiB"), (16, 5, 128, "20 KiB: five tiles"), (16, 6, 128, "24 KiB: six tiles"),
+    (11, 8, 128, "22 KiB: six tiles, the last one partly filled"), (16, 8, 128, "32 KiB"), (16, 9, 128, "36 KiB: nine tiles"),
+    (16, 10, 128, "40 KiB: ten tiles"), (16, 40, 128, "160 KiB: forty tiles"),
+])
+def test_block_moves_of_a_hundred_blocks_over_tiles_per_chunk(bs, H, D, desc):
+    """Tables of 96 blocks and more choose a tile-to-XCD mapping by the number of tiles per chunk (pairs of tiles for
+    an even count, whole chunks for pool-to-pool moves of 8 tiles and more or of an odd count, none otherwise); the
+    mapping works on windows of 8 blocks, so the table lengths here leave 4, 3 and 0 blocks past the last window."""
+    L = 3
+    g = torch.Generator().manual_seed(bs * 1000 + H)
+    for n in (100, 131, 96):
+        NB = n + 40
+        say(f"block moves, {desc}, {n} blocks")
+        src_c = [torch.randint(-30000, 30000, (2, NB, bs, H, D), generator=g).to(torch.bfloat16) for _ in range(L)]
+        dst_c = [torch.zeros_like(t) for t in src_c]
+        si_t, di_t = torch.randperm(NB, generator=g)[:n], torch.randperm(NB, generator=g)[:n]
+        src_g, dst_g, dst2_g, mig_g = to_dev(src_c), to_dev(dst_c), to_dev(dst_c), to_dev(dst_c)
+        want = orc.c_kv_pack(src_c, si_t.tolist())
+        buf = kv_ops.kv_pack(PoolView(src_g), si_t.to(DEV))
+        assert same_bits(buf, want), "pack, device table"
+        assert same_bits(kv_ops.kv_pack(PoolView(src_g), si_t.tolist()), want), "pack, list"
+        kv_ops.kv_unpack(PoolView(dst_g), di_t.to(DEV), buf)
+        kv_ops.kv_unpack(PoolView(dst2_g), di_t.tolist(), buf)
+        orc.c_kv_unpack(dst_c, di_t.tolist(), raw(buf))
+        assert same_bits(torch.stack(dst_g), torch.stack(dst_c)), "unpack, device table"
+        assert same_bits(torch.stack(dst2_g), torch.stack(dst_c)), "unpack, list"
+        kv_ops.kv_migrate(PoolView(src_g), si_t.to(DEV), PoolView(mig_g), di_t.to(DEV))
+        assert same_bits(torch.stack(mig_g), torch.stack(dst_c)), "migrate"
+        perm = torch.randperm(NB, generator=g)
+        mapping = torch.stack([perm[:n // 2 + 20], perm[n // 2 + 20:2 * (n // 2 + 20)]], 1).contiguous()
+        cache_ops.copy_blocks(src_g, mapping.to(DEV))
+        orc.c_copy_blocks(src_c, mapping.numpy())
+        assert same_bits(torch.stack(src_g), torch.stack(src_c)), "copy_blocks"
+
+
+@pytest.mark.parametrize("H,NB,n", [(4, 10400, 100), (4, 14000, 131), (40, 1100, 100), (6, 7000, 99), (2, 25000, 120)])
+def test_pack_of_a_short_table_from_large_planes(H, NB, n):
+    """A pack pairs its tiles per XCD only when the table is short against the plane it indexes (blocks * 2 MiB up to
+    1.25 x the plane's bytes): planes of 160 MB and more here, with 4, 40, 6 and 2 tiles per chunk (a power of two
+    and not)."""
+    bs, D = 16, 128
+    assert n * (2 << 20) <= 1.25 * NB * bs * H * D * 2
+    g = torch.Generator().manual_seed(NB + n)
+    src_c = [torch.randint(-30000, 30000, (2, NB, bs, H, D), generator=g, dtype=torch.int16).view(torch.bfloat16)]
+    si = torch.randperm(NB, generator=g)[:n]
+    src_g = to_dev(src_c)
+    want = orc.c_kv_pack(src_c, si.tolist())
+    assert same_bits(kv_ops.kv_pack(PoolView(src_g), si.to(DEV)), want), "device table"
+    assert same_bits(kv_ops.kv_pack(PoolView(src_g), si.tolist()), want), "list"
+
+
+@pytest.mark.parametrize("bs,H,D,n", [(16, 8, 128, 100), (16, 4, 128, 131), (16, 5, 128, 100), (16, 1, 128, 97),
+                                      (16, 8, 128, 1100)])
+def test_dequant_unpack_of_a_hundred_blocks_over_tiles_per_chunk(bs, H, D, n):
+    L, NB = 2, n + 30
+    g = torch.Generator().manual_seed(n + H)
+    packed = torch.randint(0, 0x78, (L, 2, n, bs, H, D), generator=g, dtype=torch.uint8)  # finite positive e4m3
+    packed[:, :, ::3] |= 0x80
+    ks, vs = torch.tensor([0.03, 0.4]), torch.tensor([0.9, 0.011])
+    di = torch.randperm(NB, generator=g)[:n]
+    for dt in (torch.bfloat16, torch.float16):
+        dq_g = [torch.full((2, NB, bs, H, D), 9.0, dtype=dt, device=DEV) for _ in range(L)]
+        dq_c = [torch.full((2, NB, bs, H, D), 9.0, dtype=dt) for _ in range(L)]
+        kv_ops.kv_unpack_dequant_fp8(PoolView(dq_g), di.to(DEV), packed.to(DEV), ks, vs)
+        orc.c_unpack_dequant_fp8(dq_c, di.tolist(), raw(packed), ks.numpy(), vs.numpy())
+        assert same_bits(torch.stack(dq_g), torch.stack(dq_c)), str(dt)
+
+
 # ------------------------------------------------------------------ legacy pools
 def test_monolithic_6d_pool_and_vision_pool():
     L, NB, bs, H, D = 3, 20, 16, 2, 64
