@@ -1245,9 +1245,10 @@ int append_strided(const void *const *k, const void *const *v, void *const *kc, 
 // of block_size * 16 bytes resp. block_size elements.
 constexpr int kPagedRun = 16;    // tokens of a whole run = rows staged through LDS = rows of a round of direct stores
 constexpr int kPagedRows = 32;   // token positions a tile looks at: an owned run may reach 15 tokens past the tile
-constexpr int kPagedSeg = 256;   // row elements per workgroup
+constexpr int kPagedSeg = 256;   // row elements per workgroup (template parameter SEG); 128 for short launches, see append_paged
+constexpr int kPagedSegShort = 128;
 
-// One workgroup handles the rows of up to 31 tokens x up to 256 row elements of K or V.
+// One workgroup handles the rows of up to 31 tokens x up to SEG (256 or 128) row elements of K or V.
 //
 // Runs. Consecutive tokens with consecutive slots inside one 16-slot-aligned window of a block
 // form a run (at most 16 tokens). A run belongs to the tile its first token lies in, so a tile
@@ -1259,7 +1260,8 @@ constexpr int kPagedSeg = 256;   // row elements per workgroup
 // one per tile) starts and lands, and a compact list of the other owned tokens. One wave only:
 // the instructions of this step are a visible part of a launch that lasts a few microseconds.
 //
-// Rows. Item q of a round of 16 tokens is (row q / 32, 16-byte source piece q % 32), two per thread.
+// Rows. Item q of a round of 16 tokens is (row q / (SEG / 8), 16-byte source piece q % (SEG / 8)): two per thread
+// for SEG = 256, one for SEG = 128.
 //  * The whole run goes to LDS (quantised to e4m3fn on the way when the cache is fp8; rows padded
 //    by 16 bytes so that a column walk touches every bank once), one row after the other, and,
 //    after a barrier, to the cache. K: lane q moves (group q / 16, token q % 16), one 16-byte LDS
@@ -1279,16 +1281,18 @@ constexpr int kPagedSeg = 256;   // row elements per workgroup
 // element-sized stores is what such a launch waits for; finding the runs four times as often costs
 // long launches more than that gains.
 // grid: x = token tiles, y = 2 * row segments (bit 0: K | V), z = layers.
-template <int CE, int SRC_DTYPE, bool SAT, int TT, bool TABLES>
+template <int CE, int SRC_DTYPE, bool SAT, int TT, int SEG, bool TABLES>
 __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
     const int64_t *__restrict__ slot_mapping, const char *key, const char *value, char *key_cache,
     char *value_cache, uint32_t num_tokens, uint32_t row_elems, uint32_t key_stride, uint32_t value_stride,
     uint32_t block_size, uint32_t vec_src, int64_t num_blocks, const float *k_scales, const float *v_scales,
     const std::conditional_t<TABLES, AppendTables, NoTables> tables) {
   constexpr int X = 16 / CE;               // elements per 16-byte piece of the cache
-  constexpr int ROW = kPagedSeg * CE + 16; // LDS row stride in bytes
-  constexpr int kPieces = kPagedSeg / 8;   // 16-byte source pieces per full row
+  constexpr int ROW = SEG * CE + 16; // LDS row stride in bytes
+  constexpr int kPieces = SEG / 8;   // 16-byte source pieces per full row
   constexpr int N = kPagedRun * kPieces / kThreads; // items per thread in a round of 16 tokens
+  constexpr int kPass = kThreads / kPieces;         // rows the workgroup covers with one item per thread
+  static_assert(SEG % 64 == 0 && N >= 1 && N * kPass == kPagedRun, "tile width");
   __shared__ __attribute__((aligned(16))) char tile[kPagedRun * ROW];  // the whole run
   __shared__ __attribute__((aligned(16))) char stage[kPagedRun * ROW]; // V rows of the other tokens, wave-private
   __shared__ int64_t s_blk[kPagedRows];                                  // the other owned tokens
@@ -1355,9 +1359,9 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
     key_cache = tables.key_cache[l];
     value_cache = tables.value_cache[l];
   }
-  const uint32_t e0 = seg * kPagedSeg;
+  const uint32_t e0 = seg * SEG;
   const uint32_t left = row_elems - e0;
-  const int seg_elems = left < kPagedSeg ? (int)left : kPagedSeg; // multiple of X
+  const int seg_elems = left < SEG ? (int)left : SEG; // multiple of X
   const int pieces = seg_elems >> 3;
   const char *src = kv == 0 ? key : value;
   char *cache = kv == 0 ? key_cache : value_cache;
@@ -1371,7 +1375,7 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
   if (w0 < 0 && count == 0) return;
   const int c = tid % kPieces < pieces ? tid % kPieces : 0; // lanes past the row re-read its start; nothing of theirs is stored
   const bool live = tid % kPieces < pieces;
-  const int row0 = tid / kPieces; // rows of the thread's items in a round: row0 + 8 * it
+  const int row0 = tid / kPieces; // rows of the thread's items in a round: row0 + kPass * it
 
   // One element of a source row that does not allow 16-byte loads, converted for the cache.
   auto slow_elem = [&](int pos, int e) -> uint32_t {
@@ -1387,10 +1391,10 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
       // layer has every workgroup in the same phase, and spreading the requests measured faster than bunching them
 #pragma unroll
       for (int it = 0; it < N; ++it) {
-        u32x4 v = ld<u32x4, true>(src + ((uint64_t)(t0 + w0 + row0 + 8 * it) * stride + e0 + c * 8) * 2);
+        u32x4 v = ld<u32x4, true>(src + ((uint64_t)(t0 + w0 + row0 + kPass * it) * stride + e0 + c * 8) * 2);
         asm volatile("" : "+v"(v));
         if (live) {
-          char *dst = tile + (row0 + 8 * it) * ROW;
+          char *dst = tile + (row0 + kPass * it) * ROW;
           if constexpr (CE == 2)
             *reinterpret_cast<u32x4 *>(dst + (tid % kPieces) * 16) = v;
           else
@@ -1417,7 +1421,7 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
       int doff[N];
 #pragma unroll
       for (int it = 0; it < N; ++it) {
-        const int r = base + row0 + 8 * it;
+        const int r = base + row0 + kPass * it;
         const int rc = r < count ? r : count - 1; // rows past the list re-read its last row
         dblk[it] = s_blk[rc];
         doff[it] = s_off[rc];
@@ -1429,7 +1433,7 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
       for (int it = 0; it < N; ++it) asm volatile("" : "+v"(v[it]));
 #pragma unroll
       for (int it = 0; it < N; ++it) {
-        if (base + row0 + 8 * it >= count || !live) continue;
+        if (base + row0 + kPass * it >= count || !live) continue;
         const uint32_t e = e0 + (tid % kPieces) * 8; // first element of the piece
         u32x2 q8{0, 0};
         if constexpr (CE == 1) q8 = quant8<SRC_DTYPE, SAT>(v[it], div);
@@ -1442,7 +1446,7 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
         } else {
           // V: through the wave's own rows of the staging tile, so that a store instruction covers 64
           // consecutive elements of one token (64 sectors in 16 consecutive lines) instead of every eighth
-          char *dst = stage + (row0 + 8 * it) * ROW;
+          char *dst = stage + (row0 + kPass * it) * ROW;
           if constexpr (CE == 2)
             *reinterpret_cast<u32x4 *>(dst + (tid % kPieces) * 16) = v[it];
           else
@@ -1450,20 +1454,20 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
         }
       }
       if (kv == 1) {
-        // rows row0 + 8 * it of lanes 0-31 and 32-63: the wave wrote them itself and LDS keeps a wave's order;
+        // rows row0 + kPass * it of lanes 0-31 and 32-63: the wave wrote them itself and LDS keeps a wave's order;
         // the fence (wavefront scope: no cache action) keeps the compiler from moving the reads above the writes
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
         __builtin_amdgcn_wave_barrier();
         const int lane = tid & 63, first = (tid >> 6) * (64 / kPieces);
 #pragma unroll
         for (int rr = 0; rr < N * (64 / kPieces); ++rr) {
-          const int rl = first + (rr % (64 / kPieces)) + 8 * (rr / (64 / kPieces));
+          const int rl = first + (rr % (64 / kPieces)) + kPass * (rr / (64 / kPieces));
           if (base + rl >= count) continue;
           const int64_t rblk = s_blk[base + rl];
           const int roff = s_off[base + rl];
           char *dst = cache + ((rblk * row_elems + e0) * bs + roff) * CE;
 #pragma unroll
-          for (int m = 0; m < kPagedSeg / 64; ++m) {
+          for (int m = 0; m < SEG / 64; ++m) {
             const int e = m * 64 + lane;
             if (e >= seg_elems) continue;
             // plain stores: the tokens of a partial run write neighbouring elements of the same sectors, which the
@@ -1586,7 +1590,17 @@ int append_paged(const void *const *k, const void *const *v, void *const *kc, vo
   if (((move_variant() >> 20) & 3) == 1) tile_tokens = 16;
   if (((move_variant() >> 20) & 3) == 2) tile_tokens = 4;
   const int64_t tiles = (num_tokens + tile_tokens - 1) / tile_tokens;
-  const int64_t segs = (row_elems + kPagedSeg - 1) / kPagedSeg;
+  // Row elements per workgroup: 128 instead of 256 while the launch of one layer still fits the device at once
+  // (2048 resident workgroups: 256 compute units x 8). Each thread then moves one 16-byte piece instead of two, one
+  // memory round trip less per workgroup, and twice as many workgroups share the work: a 512 / 1000 / 2000 / 3000
+  // token prompt of Qwen2-7B rows takes 2.97 / 3.47 / 4.04 / 5.03 us per layer against 3.28 / 3.96 / 4.61 / 5.24,
+  // 64 lone tokens + a 1024-token prompt 4.40 against 5.30, 4096 tokens the same (5.62); beyond that the narrow tiles
+  // need a second round of workgroups and lose (5000 tokens: 7.8 against 6.3 us). Launches for several layers keep 256.
+  int seg_elems = kPagedSeg;
+  if (!(num_layers > 1) && tiles * 2 * ((row_elems + kPagedSegShort - 1) / kPagedSegShort) <= 2048) seg_elems = kPagedSegShort;
+  if (((move_variant() >> 22) & 3) == 1) seg_elems = kPagedSeg;
+  if (((move_variant() >> 22) & 3) == 2 && num_layers == 1) seg_elems = kPagedSegShort;
+  const int64_t segs = (row_elems + seg_elems - 1) / seg_elems;
   if (tiles > 0x7fffffffLL || segs * 2 > kMaxGridY) return fail(EMM_EINVAL, "%s: too many tokens / too long rows", what);
   if (num_tokens > 0x7fffffffLL || row_elems > 0x7fffffffLL || ks > 0xffffffffLL || vs > 0xffffffffLL)
     return fail(EMM_EINVAL, "%s: num_tokens / row / token stride too large", what);
@@ -1608,17 +1622,21 @@ int append_paged(const void *const *k, const void *const *v, void *const *kc, vo
     }
   }
   const dim3 grid((uint32_t)tiles, (uint32_t)(segs * 2), (uint32_t)num_layers);
+#define EMM_PAGED_LAUNCH3(CE_, DT_, SAT_, TT_, SEG_) \
+  emm_append_paged_kernel<CE_, DT_, SAT_, TT_, SEG_, false><<<grid, kThreads, 0, s>>>( \
+      slot_mapping, (const char *)k[0], (const char *)v[0], (char *)kc[0], (char *)vc[0], (uint32_t)num_tokens, \
+      (uint32_t)row_elems, (uint32_t)ks, (uint32_t)vs, (uint32_t)block_size, vec_src, num_blocks, k_scales, \
+      v_scales, NoTables{})
 #define EMM_PAGED_LAUNCH2(CE_, DT_, SAT_, TT_) \
   do { \
     if (tables) \
-      emm_append_paged_kernel<CE_, DT_, SAT_, TT_, true><<<grid, kThreads, 0, s>>>( \
+      emm_append_paged_kernel<CE_, DT_, SAT_, TT_, kPagedSeg, true><<<grid, kThreads, 0, s>>>( \
           slot_mapping, nullptr, nullptr, nullptr, nullptr, (uint32_t)num_tokens, (uint32_t)row_elems, (uint32_t)ks, \
           (uint32_t)vs, (uint32_t)block_size, vec_src, num_blocks, k_scales, v_scales, t); \
+    else if (seg_elems == kPagedSegShort) \
+      EMM_PAGED_LAUNCH3(CE_, DT_, SAT_, TT_, kPagedSegShort); \
     else \
-      emm_append_paged_kernel<CE_, DT_, SAT_, TT_, false><<<grid, kThreads, 0, s>>>( \
-          slot_mapping, (const char *)k[0], (const char *)v[0], (char *)kc[0], (char *)vc[0], (uint32_t)num_tokens, \
-          (uint32_t)row_elems, (uint32_t)ks, (uint32_t)vs, (uint32_t)block_size, vec_src, num_blocks, k_scales, \
-          v_scales, NoTables{}); \
+      EMM_PAGED_LAUNCH3(CE_, DT_, SAT_, TT_, kPagedSeg); \
   } while (0)
 #define EMM_PAGED_LAUNCH(CE_, DT_, SAT_) \
   do { \
@@ -1632,6 +1650,7 @@ int append_paged(const void *const *k, const void *const *v, void *const *kc, vo
   else EMM_PAGED_LAUNCH(1, EMM_DTYPE_F16, true);
 #undef EMM_PAGED_LAUNCH
 #undef EMM_PAGED_LAUNCH2
+#undef EMM_PAGED_LAUNCH3
   return check_launch(what);
 }
 
@@ -2074,7 +2093,7 @@ extern "C" {
 
 int emm_hook_set_move_variant(int variant) {
   const int old = g_move_variant;
-  g_move_variant = variant & 0xf3fff00;
+  g_move_variant = variant & 0xfffff00;
   return old;
 }
 

@@ -23,6 +23,7 @@ extern "C" {
  *   3 = (4, 1), 4 = (1, 1), 5 = (2, 1);
  * bits 16-19: log2 of the blocks per plane visit of pack / unpack (15 = plain order);
  * bits 20-21: token tile of the paged-layout append (1 = 16 tokens, 2 = 4 tokens; 0 = by token count);
+ * bits 22-23: row elements per workgroup of a one-layer paged-layout append (1 = 256, 2 = 128; 0 = by launch size);
  * bit 24: fp8 append with the IEEE division instead of the reciprocal form;
  * bits 25 / 26 / 27: tile-to-XCD mapping of the block moves forced to plain / whole chunks per XCD / pairs of tiles
  *   per XCD (default: chosen per launch by kind, table length, tiles per chunk and plane size).

@@ -773,6 +773,44 @@ def test_paged_append_unusual_block_sizes(bs, fp8):
     assert same_bits(kc_g, kc) and same_bits(vc_g, vc)
 
 
+@pytest.mark.parametrize("width", [1, 2], ids=["256 row elements per workgroup", "128 row elements per workgroup"])
+def test_paged_append_both_tile_widths(width, monkeypatch):
+    """A one-layer launch takes workgroups of 128 row elements while it fits the device at once and of 256 beyond;
+    here each width is forced (test hook of the hooks library) on launches of either size, tiles of 4 and of 16
+    tokens, 16-bit and fp8 caches, rows that end inside a workgroup's segment, misaligned sources."""
+    hooks = _lib.load_hooks()
+    monkeypatch.setattr(_lib, "_lib", hooks)
+    old = hooks.emm_hook_set_move_variant(width << 22)
+    try:
+        for (dtype, NB, bs, H, D, T, phase, fp8, pad) in [
+                (torch.bfloat16, 700, 16, 4, 128, 5000, 3, False, 0), (torch.float16, 300, 16, 8, 128, 2500, 0, True, 0),
+                (torch.bfloat16, 200, 16, 4, 128, 1000, 7, False, 0), (torch.bfloat16, 64, 16, 4, 128, 256, 5, False, 0),
+                (torch.float16, 96, 8, 3, 40, 333, 0, False, 0), (torch.bfloat16, 33, 16, 5, 112, 77, 2, True, 0), (torch.bfloat16, 33, 16, 5, 104, 77, 2, False, 0),
+                (torch.bfloat16, 48, 32, 2, 64, 700, 1, False, 8), (torch.float16, 80, 16, 3, 96, 300, 4, False, 5),
+                (torch.bfloat16, 40, 16, 1, 64, 130, 0, True, 5), (torch.bfloat16, 30, 16, 20, 128, 100, 1, False, 0)]:
+            say(f"paged append, width code {width}: {dtype} NB={NB} bs={bs} H={H} D={D} T={T} fp8={fp8} row pad={pad}")
+            g = torch.Generator().manual_seed(NB * 7 + T + width)
+            slots = paged_slots(NB, bs, T, seed=T + 1, phase=phase)
+            src = (torch.randn((T, 2 * H * D + pad), generator=g) * 3).to(dtype)
+            src_g = src.to(DEV)
+            k_g, v_g = src_g[:, :H * D].view(T, H, D), src_g[:, H * D:2 * H * D].view(T, H, D)
+            kh = src[:, :H * D].reshape(T, H, D).contiguous()
+            vh = src[:, H * D:2 * H * D].reshape(T, H, D).contiguous()
+            kc, vc = paged_caches_cpu(NB, H, D, bs, torch.uint8 if fp8 else dtype)
+            kc_g, vc_g = kc.to(DEV), vc.to(DEV)
+            if fp8:
+                ks, vs = torch.tensor([0.07]), torch.tensor([0.6])
+                cache_ops.reshape_and_cache(k_g, v_g, kc_g.view(torch.float8_e4m3fn), vc_g.view(torch.float8_e4m3fn),
+                                            slots.to(DEV), "fp8", ks.to(DEV), vs.to(DEV))
+                orc.c_reshape_and_cache_paged(kh, vh, kc, vc, slots, float(ks), float(vs))
+            else:
+                cache_ops.reshape_and_cache(k_g, v_g, kc_g, vc_g, slots.to(DEV))
+                orc.c_reshape_and_cache_paged(kh, vh, kc, vc, slots)
+            assert same_bits(kc_g, kc) and same_bits(vc_g, vc), f"T={T} H={H} D={D} fp8={fp8}"
+    finally:
+        hooks.emm_hook_set_move_variant(old)
+
+
 def test_paged_append_seeded_sweep_of_shapes():
     """Forty seeded draws of (dtype, block size, heads, head size, tokens, slot pattern, fp8 or not, source
     row stride), each against the C restatement: shapes nobody picked by hand."""
