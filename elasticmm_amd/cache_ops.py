@@ -1,4 +1,4 @@
-"""vLLM-shaped cache operators: ``reshape_and_cache_flash``, ``reshape_and_cache`` and ``copy_blocks``.
+"""vLLM-shaped cache operators: ``reshape_and_cache_flash``, ``reshape_and_cache``, ``copy_blocks`` and ``swap_blocks``.
 
 The reference reaches both inside vLLM (``vllm>=0.10.1``, V0 engine): the append
 from ``model_runner.execute_model`` (elasticmm/engine/v0/worker_steps.py:281, :438)
@@ -111,12 +111,51 @@ def paged_layered_append(keys: Sequence[torch.Tensor], values: Sequence[torch.Te
     raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
 
 
-def copy_blocks(kv_caches: List[torch.Tensor], block_mapping: torch.Tensor) -> None:
-    """``kv_caches``: list of ``[2, num_blocks, block_size, H, D]``; ``block_mapping``: int64
-    ``[num_pairs, 2]`` of (src, dst). One launch covers every layer, K and V."""
+def copy_blocks(kv_caches: Sequence[torch.Tensor], *args) -> None:
+    """Both call shapes vLLM has for this operator; one launch covers every layer, K and V.
+
+    ``copy_blocks(kv_caches, block_mapping)`` — the attention-backend form: ``kv_caches`` is the list of
+    per-layer ``[2, num_blocks, ...]`` pools, ``block_mapping`` int64 ``[num_pairs, 2]`` of (src, dst).
+
+    ``copy_blocks(key_caches, value_caches, block_mapping)`` — the form of ``vllm._custom_ops.copy_blocks``
+    that the backends hand their split pools to: per-layer key caches and value caches ``[num_blocks, ...]``
+    whose trailing shapes may differ (``[NB, H, D // x, bs, x]`` and ``[NB, H, D, bs]`` in the paged-attention
+    layout) as long as a block has the same number of bytes in both."""
+    if len(args) == 1:
+        (block_mapping,) = args
+        if len(kv_caches) == 0 or block_mapping.numel() == 0:
+            return
+        kv_ops.copy_blocks(PoolView(kv_caches), block_mapping)
+        return
+    if len(args) != 2:
+        raise TypeError("copy_blocks(kv_caches, block_mapping) or copy_blocks(key_caches, value_caches, block_mapping)")
+    value_caches, block_mapping = args
+    if len(kv_caches) != len(value_caches):
+        raise ValueError("key_caches and value_caches differ in length")
     if len(kv_caches) == 0 or block_mapping.numel() == 0:
         return
-    kv_ops.copy_blocks(PoolView(kv_caches), block_mapping)
+    planes = [t.view(t.shape[0], -1) for t in list(kv_caches) + list(value_caches)]  # one chunk per block and plane
+    kv_ops.copy_blocks(PoolView(planes, num_kv_dim=False), block_mapping)
+
+
+def swap_blocks(src_kv_cache: torch.Tensor, dst_kv_cache: torch.Tensor, src_to_dst) -> None:
+    """vLLM's backend-level ``swap_blocks(src_kv_cache, dst_kv_cache, src_to_dst)`` for one layer: block
+    ``src_to_dst[j, 0]`` of ``src_kv_cache`` ``[2, NB_src, ...]`` goes to block ``src_to_dst[j, 1]`` of
+    ``dst_kv_cache`` ``[2, NB_dst, ...]``, K and V in one launch. One of the two may be a page-locked host
+    tensor (vLLM's ``cpu_cache``): the kernel then reads / writes it over PCIe directly. ``src_to_dst`` is an
+    int64 ``[num_pairs, 2]`` tensor (vLLM passes it on the CPU) or a list of pairs. The worker-level form with
+    side streams and per-request events is ``KVWorker.swap_blocks`` (elasticmm/engine/v0/worker.py:467-526)."""
+    pairs = src_to_dst if isinstance(src_to_dst, torch.Tensor) else torch.as_tensor(list(src_to_dst), dtype=torch.long)
+    if pairs.numel() == 0:
+        return
+    if pairs.dim() != 2 or pairs.shape[1] != 2 or pairs.dtype != torch.long:
+        raise ValueError("src_to_dst must be int64 pairs [num_pairs, 2]")
+    if not (src_kv_cache.is_cuda or dst_kv_cache.is_cuda):
+        raise ValueError("swap_blocks: at least one cache must live in GPU memory")
+    gpu = src_kv_cache.device if src_kv_cache.is_cuda else dst_kv_cache.device
+    src = PoolView([src_kv_cache], pinned_host_for=None if src_kv_cache.is_cuda else gpu)
+    dst = PoolView([dst_kv_cache], pinned_host_for=None if dst_kv_cache.is_cuda else gpu)
+    kv_ops.kv_migrate(src, pairs[:, 0].contiguous(), dst, pairs[:, 1].contiguous())
 
 
 def compute_slot_mapping(block_tables: Sequence[Sequence[int]], context_lens: Sequence[int],

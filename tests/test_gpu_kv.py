@@ -240,6 +240,63 @@ def test_copy_blocks_against_oracle():
     assert same_bits(torch.stack(dev2), torch.stack(want))
 
 
+def test_copy_blocks_with_split_key_and_value_caches():
+    """The operator-level call shape: per-layer key caches and value caches of the paged-attention layout
+    (different trailing shapes, equal bytes per block), checked against the C restatement applied to the same
+    bytes viewed as [2, NB, chunk] pools and against torch's indexing."""
+    for dtype, L, NB, H, D, bs in [(torch.bfloat16, 3, 50, 4, 128, 16), (torch.uint8, 2, 40, 2, 64, 16),
+                                   (torch.float16, 100, 12, 1, 32, 8)]:  # 200 planes: more than one argument block
+        x = 16 // torch.empty((), dtype=dtype).element_size()
+        g = torch.Generator().manual_seed(NB + L)
+        kcs = [torch.randint(0, 250, (NB, H, D // x, bs, x), generator=g).to(dtype) for _ in range(L)]
+        vcs = [torch.randint(0, 250, (NB, H, D, bs), generator=g).to(dtype) for _ in range(L)]
+        perm = torch.randperm(NB, generator=g)
+        n = NB // 3
+        mapping = torch.stack([perm[:n], perm[n:2 * n]], 1).contiguous()
+        k_g, v_g = to_dev(kcs), to_dev(vcs)
+        cache_ops.copy_blocks(k_g, v_g, mapping.to(DEV))
+        pools = [torch.stack([kcs[l].reshape(NB, -1), vcs[l].reshape(NB, -1)]) for l in range(L)]
+        orc.c_copy_blocks(pools, mapping.numpy())
+        for l in range(L):
+            assert same_bits(k_g[l], pools[l][0]) and same_bits(v_g[l], pools[l][1]), f"layer {l}"
+            want_k = kcs[l].clone()
+            want_k[mapping[:, 1]] = kcs[l][mapping[:, 0]]
+            assert same_bits(k_g[l], want_k)
+    cache_ops.copy_blocks([], [], mapping.to(DEV))  # nothing to do
+    with pytest.raises(ValueError, match="differ in length"):
+        cache_ops.copy_blocks(k_g, v_g[:-1], mapping.to(DEV))
+
+
+def test_cache_ops_swap_blocks_between_gpu_and_pinned_host():
+    """vLLM's swap_blocks for one layer: GPU -> page-locked host -> another GPU cache, K and V per launch;
+    the pairs arrive as a CPU tensor (vLLM's form) or as a list."""
+    NBg, NBc, bs, H, D = 30, 20, 16, 4, 128
+    g = torch.Generator().manual_seed(77)
+    gpu_c = torch.randn((2, NBg, bs, H, D), generator=g).to(torch.bfloat16)
+    gpu = gpu_c.to(DEV)
+    cpu = torch.zeros((2, NBc, bs, H, D), dtype=torch.bfloat16).pin_memory()
+    out_pairs = torch.stack([torch.randperm(NBg, generator=g)[:12], torch.randperm(NBc, generator=g)[:12]], 1)
+    cache_ops.swap_blocks(gpu, cpu, out_pairs)
+    torch.cuda.synchronize()
+    want_cpu = torch.zeros_like(cpu)
+    want_cpu[:, out_pairs[:, 1]] = gpu_c[:, out_pairs[:, 0]]
+    assert same_bits(cpu, want_cpu)
+    back = torch.full((2, NBg, bs, H, D), 7.0, dtype=torch.bfloat16, device=DEV)
+    in_pairs = torch.stack([out_pairs[:, 1], torch.randperm(NBg, generator=g)[:12]], 1)
+    cache_ops.swap_blocks(cpu, back, in_pairs.tolist())
+    want_back = torch.full((2, NBg, bs, H, D), 7.0, dtype=torch.bfloat16)
+    want_back[:, in_pairs[:, 1]] = want_cpu[:, in_pairs[:, 0]]
+    assert same_bits(back, want_back)
+    gpu2 = torch.zeros_like(gpu)
+    cache_ops.swap_blocks(gpu, gpu2, out_pairs[:, [0, 0]].contiguous())  # device to device, same ids
+    want2 = torch.zeros_like(gpu_c)
+    want2[:, out_pairs[:, 0]] = gpu_c[:, out_pairs[:, 0]]
+    assert same_bits(gpu2, want2)
+    cache_ops.swap_blocks(gpu, gpu2, torch.empty((0, 2), dtype=torch.long))  # nothing to do
+    with pytest.raises(ValueError, match="GPU memory"):
+        cache_ops.swap_blocks(cpu, cpu, out_pairs)
+
+
 def test_migrate_equals_pack_then_unpack():
     L, NBs, NBd = 4, 40, 24
     src_c = cpu_pool(L, NBs, 16, 4, 128, torch.bfloat16, 10)
