@@ -381,12 +381,25 @@ class KVMigrationManager:
     """Cross-stage moves addressed by (stage, worker id) (kv_transfer.py:867-980, ``V0KVMigrationManager``):
     extract on the source worker, write on the destination worker, for KV blocks and for a request's vision
     embeddings. The reference's worker lookup is a placeholder that finds nobody (:961-969), so its moves always
-    report failure; here workers are registered under (stage, worker id)."""
+    report failure; here workers are registered under (stage, worker id). The coroutines run the blocking move on
+    the manager's own thread, like ``KVTransferManager``'s."""
 
     def __init__(self):
         self.migration_count = 0
         self.total_migration_time = 0.0
         self._workers_by_stage: Dict[Tuple[str, int], Any] = {}
+        self._executor: Optional[concurrent.futures.ThreadPoolExecutor] = None
+
+    async def _off_loop(self, fn, *args):
+        """Run a blocking move on this manager's own thread and await it (the event loop stays free)."""
+        if self._executor is None:
+            self._executor = concurrent.futures.ThreadPoolExecutor(max_workers=1, thread_name_prefix="kv-migration")
+        return await asyncio.get_running_loop().run_in_executor(self._executor, fn, *args)
+
+    def close(self) -> None:
+        if self._executor is not None:
+            self._executor.shutdown(wait=True)
+            self._executor = None
 
     def register_worker(self, stage: str, worker_id: int, worker: Any) -> None:
         self._workers_by_stage[(stage.lower(), worker_id)] = worker
@@ -440,12 +453,13 @@ class KVMigrationManager:
 
     async def migrate_kv_blocks(self, request_id: str, src_stage: str, src_worker_id: int, src_blocks: List[int],
                                 dst_stage: str, dst_worker_id: int, dst_blocks: List[int]) -> bool:
-        return self.migrate_kv_blocks_sync(request_id, src_stage, src_worker_id, src_blocks, dst_stage,
-                                           dst_worker_id, dst_blocks)
+        return await self._off_loop(self.migrate_kv_blocks_sync, request_id, src_stage, src_worker_id, src_blocks,
+                                    dst_stage, dst_worker_id, dst_blocks)
 
     async def migrate_vision_embeddings(self, request_id: str, src_stage: str, src_worker_id: int, dst_stage: str,
                                         dst_worker_id: int) -> bool:
-        return self.migrate_vision_embeddings_sync(request_id, src_stage, src_worker_id, dst_stage, dst_worker_id)
+        return await self._off_loop(self.migrate_vision_embeddings_sync, request_id, src_stage, src_worker_id,
+                                    dst_stage, dst_worker_id)
 
     def get_stats(self) -> Dict[str, Any]:
         return {
