@@ -62,7 +62,7 @@ def parse():
     ap.add_argument("--no-extra", action="store_true", help="headline only (same as --sections none)")
     ap.add_argument("--sections", default="all",
                     help="comma-separated secondary measurements to run: " + ",".join(ALL_SECTIONS) + " (all | none)")
-    ap.add_argument("--variant", type=int, default=0,
+    ap.add_argument("--variant", type=lambda v: int(v, 0), default=0,
                     help="launch variant of the hooks build (tuning; routes every call through libemm_kv_hooks.so)")
     ap.add_argument("--spread", type=int, default=4,
                     help="stripes per pool of the headline: each pool's layers are allocated in this many pieces spread "

@@ -1560,6 +1560,236 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
   }
 }
 
+// The paged-attention append for the usual shapes (16-bit cache, sources that allow 16-byte loads, block size a
+// power of two >= 16): workgroups of ONE wave, no block barrier.
+//
+// A wave owns a tile of 16 token positions x COLS row elements of K or of V (grid: x = 2 * column + (K | V),
+// y = tile, z = layer; x runs fastest, so the waves of one tile are dispatched side by side).
+//
+// Who stores what. 16 consecutive tokens whose slots fill one 16-slot-aligned window of a block are a whole run;
+// the run belongs to the tile its first token lies in (it may reach 15 tokens into the next tile). Every other
+// valid token is stored by its own tile, one token at a time. Both decisions need nothing but the 48 slots
+// around the tile: lane i (< 48) loads the slots of positions t0 - 16 + i and + 1, four lane compares become
+// four 64-bit masks (valid, consecutive, aligned, not at a window start), and the rest is scalar bit arithmetic:
+//   links   E = valid & valid >> 1 & consecutive & next-not-at-a-window-start        (bit p: p -> p + 1 is a link)
+//   15 links in a row from p: four shift-and steps; W = those & valid & aligned      (bit p: a whole run starts)
+//   bits 1..15 of W: a run of the previous tile covers this tile's tokens below that bit;
+//   bits 16..31: this tile's own run (at most one: two starts are at least 16 apart).
+// Every wave of a tile repeats this (a dozen vector and two dozen scalar instructions) instead of sharing it
+// through LDS and a barrier.
+//
+// Whole run: the 16 rows x COLS elements go to a wave-private LDS tile (rows padded by 16 bytes) and come back
+// transposed: K as 16-byte pieces, lane -> (group, token), every store instruction 1 KiB of contiguous cache;
+// V through the transposing LDS read ds_read_b64_tr_b16, lanes 0-31 the tokens 0-7 and lanes 32-63 the tokens
+// 8-15 of the same 32 elements, again 1 KiB of whole sectors per store instruction.
+// Other tokens: lane -> (token, piece) loads the row piece and the token's slot; K is stored from the registers
+// as 16-byte pieces; V passes through the LDS tile so that a store instruction writes 64 (COLS = 32: 2 x 32)
+// consecutive elements of a token — element-sized writes, each a partial sector: what this layout costs for a
+// token that does not fill a block.
+// COLS = 128 for long launches; 32 for launches of few tokens, which then spread over four times as many waves.
+// Measured on MI355X, Qwen2-7B rows, 28 layers (per-layer launches replayed from a HIP graph / one launch for all
+// layers; the flash-layout append on the same slots and memory beside it):
+//   8192-token prompt of whole runs   8.4-8.6 us per launch, 148 us (6.35 TB/s)     flash layout 7.0 us, 145 us
+//   256 single tokens                  4.8 us per launch, 39 us                      flash layout 2.2 us, 8 us
+//   256 single tokens + that prompt   12.6 us per launch, 251 us                     flash layout 7.2 us, 151 us
+// Whole runs move at the speed of the flash-layout append; what is left is the single tokens: each of a token's 512 V
+// elements and 64 K pieces is a write request of its own, whatever kernel issues it (K alone: 2.2 us for the 256
+// tokens, the launch floor; V alone: 4.6). Tried on the single tokens' V stores and not kept: reading the word first so
+// that the line is valid in the L2 (256 tokens x 28 layers in one launch: 69 us against 43), merging with a pair of
+// 32-bit atomics (151 us), write-through stores (45 us). Whole rows per wave (COLS = 512, benchmark builds) bring the
+// per-layer launch of a prompt of whole runs to 7.1-7.3 us but leave a tile of 16 single tokens to two waves (a
+// decode step: 9.5 us per launch); the tile order (tiles slowest, layers inside) is worth 4 % on the one-launch form.
+template <int COLS, bool TABLES>
+__global__ __launch_bounds__(64) void emm_append_paged_wave_kernel(
+    const int64_t *__restrict__ slot_mapping, const char *key, const char *value, char *key_cache,
+    char *value_cache, uint32_t num_tokens, uint32_t row_elems, uint32_t key_stride, uint32_t value_stride,
+    uint32_t bs_log2, uint64_t num_slots, const std::conditional_t<TABLES, AppendTables, NoTables> tables) {
+  constexpr int PC = COLS / 8;     // 16-byte source pieces per row segment
+  constexpr int RPI = 64 / PC;     // token rows one load instruction covers
+  constexpr int NL = 16 / RPI;     // load instructions for 16 rows
+  constexpr int ROW = COLS * 2 + 16; // LDS row stride in bytes
+  static_assert(COLS == 512 || COLS == 256 || COLS == 128 || COLS == 32, "column width");
+  __shared__ __attribute__((aligned(16))) char tile[16 * ROW];
+  const uint32_t lane = threadIdx.x;
+  // grid: x = the 2 * columns waves of a tile, then the layers (TABLES), tiles slowest. Workgroups go to the 8 XCDs
+  // round-robin in dispatch order; rotating the (column, K | V) assignment by the tile index spreads the V waves of
+  // consecutive tiles over all XCDs (the single tokens of V are eight times the write requests of K).
+  const uint32_t tile_idx = TABLES ? blockIdx.z : blockIdx.y;
+  const uint32_t rot_mask = bs_log2 >> 8;
+  bs_log2 &= 0xffu;
+  const uint32_t xi = rot_mask ? (blockIdx.x + tile_idx) & rot_mask : blockIdx.x;
+  const uint32_t kv = xi & 1u, col = xi >> 1;
+  const uint32_t t0 = tile_idx * 16u;
+
+  // ---- the 48 slots around the tile -> whole runs and single tokens (wave-uniform) ----
+  const int32_t pos = (int32_t)t0 - 16 + (int32_t)lane, last = (int32_t)num_tokens - 1;
+  const int32_t p0 = pos < 0 ? 0 : pos > last ? last : pos;
+  const int32_t p1 = pos + 1 < 0 ? 0 : pos + 1 > last ? last : pos + 1;
+  const int64_t s = slot_mapping[p0];
+  const int64_t sn = slot_mapping[p1];
+  if constexpr (TABLES) {
+    const uint32_t l = blockIdx.y;
+    key = tables.key[l];
+    value = tables.value[l];
+    key_cache = tables.key_cache[l];
+    value_cache = tables.value_cache[l];
+  }
+  const char *src = kv == 0 ? key : value;
+  char *cache = kv == 0 ? key_cache : value_cache;
+  const uint32_t stride = kv == 0 ? key_stride : value_stride;
+  const uint32_t e0 = col * COLS;
+  const uint32_t col_elems = row_elems - e0 < (uint32_t)COLS ? row_elems - e0 : (uint32_t)COLS; // multiple of 8
+  const uint32_t piece = lane % PC, rsub = lane / PC;
+  const bool live = piece * 8 < col_elems;
+  const uint32_t bs_mask = (1u << bs_log2) - 1u;
+  const uint64_t groups_per_block = row_elems >> 3;
+
+  // Short launches (COLS = 32: one load instruction covers the tile's 16 rows) request the tile's own rows before the
+  // slots have arrived: they are what single tokens and a run that starts on the tile grid need, and a short launch
+  // is one chain of memory round trips; a run that starts inside the tile loads its rows again.
+  constexpr bool EARLY = NL == 1;
+  u32x4 early{0, 0, 0, 0};
+  if constexpr (EARLY) {
+    const uint32_t tr = t0 + rsub <= (uint32_t)last ? t0 + rsub : (uint32_t)last;
+    early = ld<u32x4, true>(src + ((uint64_t)tr * stride + e0 + (live ? piece * 8 : 0)) * 2);
+  }
+  const uint32_t slo = (uint32_t)s, snlo = (uint32_t)sn;
+  const uint32_t lo = t0 == 0 ? 16u : 0u;                                    // positions below 0
+  const uint32_t hi = num_tokens - t0 + 16u < 48u ? num_tokens - t0 + 16u : 48u; // positions past the last token
+  const uint64_t in_range = ((1ull << hi) - 1ull) & ~((1ull << lo) - 1ull);
+  const uint64_t valid = __ballot((uint64_t)s < num_slots) & in_range; // slots are below 2^32 (checked by the host)
+  const uint64_t consecutive = __ballot(snlo == slo + 1u);
+  const uint64_t next_inside = __ballot((snlo & 15u) != 0u);
+  const uint64_t aligned16 = __ballot((slo & 15u) == 0u);
+  uint64_t e = valid & (valid >> 1) & consecutive & next_inside;
+  e &= e >> 1;
+  e &= e >> 2;
+  e &= e >> 4;
+  e &= e >> 7; // bit p: the 15 links p .. p + 14 are all there
+  const uint64_t starts = e & valid & aligned16;
+  const uint32_t prev_run = (uint32_t)starts & 0xfffeu;
+  const uint32_t own_run = (uint32_t)(starts >> 16) & 0xffffu;
+  const int w0 = own_run ? __builtin_ctz(own_run) : -1;
+  uint32_t lone = (uint32_t)(valid >> 16) & 0xffffu;
+  if (prev_run) lone &= ~((1u << __builtin_ctz(prev_run)) - 1u);
+  if (w0 >= 0) lone &= (1u << w0) - 1u;
+  if (w0 < 0 && lone == 0) return;
+
+  // ---- the whole run ----
+  if (w0 >= 0) {
+    const uint32_t sw = (uint32_t)__builtin_amdgcn_readlane((int)slo, 16 + w0);
+    const uint64_t wblk = sw >> bs_log2;
+    const uint32_t woff = sw & bs_mask;
+    const char *rows = src + ((uint64_t)(t0 + w0) * stride + e0 + (live ? piece * 8 : 0)) * 2;
+    u32x4 v[NL];
+    if (EARLY && w0 == 0) {
+      v[0] = early;
+    } else {
+#pragma unroll
+      for (int k = 0; k < NL; ++k) v[k] = ld<u32x4, true>(rows + (uint64_t)(k * RPI + rsub) * stride * 2);
+    }
+#pragma unroll
+    for (int k = 0; k < NL; ++k)
+      if (live) *reinterpret_cast<u32x4 *>(tile + (k * RPI + rsub) * ROW + piece * 16) = v[k];
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront"); // the wave reads what its other lanes wrote
+    __builtin_amdgcn_wave_barrier();
+    if (kv == 0) {
+      const uint32_t r = lane & 15;
+#pragma unroll
+      for (int j = 0; j < PC / 4; ++j) {
+        const uint32_t g = 4 * j + (lane >> 4);
+        const u32x4 x = *reinterpret_cast<const u32x4 *>(tile + r * ROW + g * 16);
+        if (g * 8 < col_elems)
+          st_stream<u32x4, 1>(cache + (((wblk * groups_per_block + (e0 >> 3) + g) << bs_log2) + woff + r) * 16, x);
+      }
+    } else {
+      typedef short v4i16 __attribute__((ext_vector_type(4)));
+      typedef __attribute__((address_space(3))) v4i16 lds_v4i16;
+      const uint32_t half = lane >> 5, grp = (lane >> 4) & 1, sub = lane & 15;
+#pragma unroll
+      for (int q0 = 0; q0 < COLS; q0 += 32) {
+        // in every group of 16 lanes, lane 4 j + q points at elements c .. c + 3 of token j and lane l receives
+        // element l of tokens 0 .. 3: two reads give a lane 8 tokens of its element
+        const char *from = tile + (8 * half + (sub >> 2)) * ROW + (q0 + 16 * grp + 4 * (sub & 3)) * 2;
+        uint32_t w[4];
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+          const v4i16 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16 *)(from + 4 * m * ROW));
+          w[2 * m] = (uint32_t)(uint16_t)t[0] | ((uint32_t)(uint16_t)t[1] << 16);
+          w[2 * m + 1] = (uint32_t)(uint16_t)t[2] | ((uint32_t)(uint16_t)t[3] << 16);
+        }
+        const uint32_t el = q0 + 16 * grp + sub;
+        if (el < col_elems)
+          st_stream<u32x4, 1>(cache + ((((wblk * row_elems + e0 + el) << bs_log2) + woff) * 2 + half * 16),
+                              u32x4{w[0], w[1], w[2], w[3]});
+      }
+    }
+    if (lone == 0) return;
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront"); // the tile is reused below
+    __builtin_amdgcn_wave_barrier();
+  }
+
+  // ---- the other tokens of the tile ----
+  // lane -> (token k * RPI + rsub, piece); lanes whose token is not one of these re-read the first of them
+  // (all loads are issued together and unconditionally; only what is kept is predicated)
+  const uint32_t first_lone = (uint32_t)__builtin_ctz(lone);
+  bool mine[NL];
+  u32x4 x[NL];
+  const char *rows = src + ((uint64_t)t0 * stride + e0 + (live ? piece * 8 : 0)) * 2;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t row = k * RPI + rsub;
+    mine[k] = ((lone >> row) & 1u) && live;
+    if constexpr (EARLY)
+      x[k] = early;
+    else
+      x[k] = ld<u32x4, true>(rows + (uint64_t)(mine[k] ? row : first_lone) * stride * 2);
+  }
+  if (kv == 0) {
+    uint32_t sl[NL]; // the slot of the lane's token: held by lane 16 + token
+#pragma unroll
+    for (int k = 0; k < NL; ++k) sl[k] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((16 + k * RPI + rsub) * 4), (int)slo);
+#pragma unroll
+    for (int k = 0; k < NL; ++k)
+      if (mine[k])
+        st_stream<u32x4, 1>(cache + (((((uint64_t)(sl[k] >> bs_log2)) * groups_per_block + (e0 >> 3) + piece) << bs_log2) +
+                                     (sl[k] & bs_mask)) * 16, x[k]);
+    return;
+  }
+#pragma unroll
+  for (int k = 0; k < NL; ++k)
+    if (mine[k]) *reinterpret_cast<u32x4 *>(tile + (k * RPI + rsub) * ROW + piece * 16) = x[k];
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  for (uint32_t m = lone; m;) { // at most 16 rounds
+    const int i0 = __builtin_ctz(m);
+    m &= m - 1;
+    if constexpr (COLS >= 64) {
+      const uint64_t sl = (uint32_t)__builtin_amdgcn_readlane((int)slo, 16 + i0);
+      char *dst = cache + ((((sl >> bs_log2) * row_elems + e0) << bs_log2) + (sl & bs_mask)) * 2;
+      // plain stores: neighbouring tokens of a partial run write neighbouring elements of the same sectors, which
+      // the L2 merges before they go to memory
+      for (uint32_t el = lane; el < col_elems; el += 64)
+        st<uint16_t, false>(dst + ((uint64_t)el << bs_log2) * 2, *reinterpret_cast<const uint16_t *>(tile + i0 * ROW + el * 2));
+    } else { // two tokens per store instruction
+      int i1 = -1;
+      if (m) {
+        i1 = __builtin_ctz(m);
+        m &= m - 1;
+      }
+      const uint32_t s0 = (uint32_t)__builtin_amdgcn_readlane((int)slo, 16 + i0);
+      const uint32_t s1 = (uint32_t)__builtin_amdgcn_readlane((int)slo, 16 + (i1 < 0 ? i0 : i1));
+      const bool upper = lane >= (uint32_t)COLS;
+      const int i = upper ? i1 : i0;
+      const uint64_t sl = upper ? s1 : s0;
+      const uint32_t el = lane & (COLS - 1);
+      if (i >= 0 && el < col_elems)
+        st<uint16_t, false>(cache + ((((sl >> bs_log2) * row_elems + e0 + el) << bs_log2) + (sl & bs_mask)) * 2,
+                            *reinterpret_cast<const uint16_t *>(tile + i * ROW + el * 2));
+    }
+  }
+}
+
 int append_paged(const void *const *k, const void *const *v, void *const *kc, void *const *vc, int num_layers,
                  const int64_t *slot_mapping, int64_t num_tokens, int num_heads, int head_size,
                  int block_size, int64_t num_blocks, int64_t ks, int64_t vs, int src_dtype,
@@ -1619,6 +1849,49 @@ int append_paged(const void *const *k, const void *const *v, void *const *kc, vo
       t.value[l] = (const char *)v[l];
       t.key_cache[l] = (char *)kc[l];
       t.value_cache[l] = (char *)vc[l];
+    }
+  }
+  // The usual shapes take the kernel of one-wave workgroups: 16-bit cache, 16-byte loads from the sources, block size
+  // a power of two from 16 on, all slots below 2^32 (run finding compares the low words). Benchmark builds can force
+  // the general kernel (bit 28) and either column width (bits 29-30: 1 = 128, 2 = 32).
+  const bool bs_pow2 = (block_size & (block_size - 1)) == 0;
+  const int64_t wave_tiles = (num_tokens + 15) / 16;
+  if (cache_elem_bytes == 2 && vec_src && bs_pow2 && block_size >= 16 && row_elems % 8 == 0 &&
+      num_blocks * block_size <= 0xffffffffLL && wave_tiles <= kMaxGridY && !(move_variant() & 0x10000000)) {
+    // columns of 32 row elements while a launch of 128-element columns would leave most of the device idle (a decode
+    // step: 256 tokens of Qwen2-7B rows are 128 waves of 128-element columns, 512 of 32)
+    int cols = wave_tiles * 2 * ((row_elems + 127) / 128) * num_layers < 1024 ? 32 : 128;
+    if (((move_variant() >> 29) & 3) == 1) cols = 128;
+    if (((move_variant() >> 29) & 3) == 2) cols = 32;
+    if (((move_variant() >> 29) & 3) == 3) cols = (move_variant() & 0x100) ? 256 : 512; // benchmark builds only
+    const int64_t ncols = (row_elems + cols - 1) / cols;
+    if (ncols * 2 <= 0x7fffffffLL) {
+      const dim3 wgrid((uint32_t)(ncols * 2), tables ? (uint32_t)num_layers : (uint32_t)wave_tiles,
+                       tables ? (uint32_t)wave_tiles : 1u);
+      const uint32_t nx = (uint32_t)(ncols * 2);
+      const uint32_t rot_mask = (nx & (nx - 1)) == 0 && nx <= 0x800000u ? nx - 1 : 0u;
+      const uint32_t bs_log2 = (uint32_t)__builtin_ctz((unsigned)block_size) | (rot_mask << 8);
+      const uint64_t num_slots = (uint64_t)num_blocks * (uint64_t)block_size;
+#define EMM_PAGED_WAVE(COLS_) \
+  do { \
+    if (tables) \
+      emm_append_paged_wave_kernel<COLS_, true><<<wgrid, 64, 0, s>>>( \
+          slot_mapping, nullptr, nullptr, nullptr, nullptr, (uint32_t)num_tokens, (uint32_t)row_elems, (uint32_t)ks, \
+          (uint32_t)vs, bs_log2, num_slots, t); \
+    else \
+      emm_append_paged_wave_kernel<COLS_, false><<<wgrid, 64, 0, s>>>( \
+          slot_mapping, (const char *)k[0], (const char *)v[0], (char *)kc[0], (char *)vc[0], (uint32_t)num_tokens, \
+          (uint32_t)row_elems, (uint32_t)ks, (uint32_t)vs, bs_log2, num_slots, NoTables{}); \
+  } while (0)
+#ifdef EMM_BENCH_HOOKS
+      if (cols == 512) EMM_PAGED_WAVE(512); // whole rows per wave: measured for the record, see the kernel's comment
+      else if (cols == 256) EMM_PAGED_WAVE(256);
+      else
+#endif
+      if (cols == 128) EMM_PAGED_WAVE(128);
+      else EMM_PAGED_WAVE(32);
+#undef EMM_PAGED_WAVE
+      return check_launch(what);
     }
   }
   const dim3 grid((uint32_t)tiles, (uint32_t)(segs * 2), (uint32_t)num_layers);
@@ -2093,7 +2366,7 @@ extern "C" {
 
 int emm_hook_set_move_variant(int variant) {
   const int old = g_move_variant;
-  g_move_variant = variant & 0xfffff00;
+  g_move_variant = variant & 0x7fffff00;
   return old;
 }
 

@@ -26,7 +26,10 @@ extern "C" {
  * bits 22-23: row elements per workgroup of a one-layer paged-layout append (1 = 256, 2 = 128; 0 = by launch size);
  * bit 24: fp8 append with the IEEE division instead of the reciprocal form;
  * bits 25 / 26 / 27: tile-to-XCD mapping of the block moves forced to plain / whole chunks per XCD / pairs of tiles
- *   per XCD (default: chosen per launch by kind, table length, tiles per chunk and plane size).
+ *   per XCD (default: chosen per launch by kind, table length, tiles per chunk and plane size);
+ * bit 28: the paged-layout append always through the general kernel (256-thread workgroups, block barrier) instead of
+ *   the kernel of one-wave workgroups that the usual shapes take;
+ * bits 29-30: column width of the one-wave paged-layout append (1 = 128 row elements, 2 = 32; 0 = by launch size).
  * Process-wide, not thread-safe. Returns the previous value. */
 int emm_hook_set_move_variant(int variant);
 

@@ -837,7 +837,7 @@ def test_paged_append_both_tile_widths(width, monkeypatch):
     tokens, 16-bit and fp8 caches, rows that end inside a workgroup's segment, misaligned sources."""
     hooks = _lib.load_hooks()
     monkeypatch.setattr(_lib, "_lib", hooks)
-    old = hooks.emm_hook_set_move_variant(width << 22)
+    old = hooks.emm_hook_set_move_variant((width << 22) | (1 << 28))  # bit 28: the general kernel for every shape
     try:
         for (dtype, NB, bs, H, D, T, phase, fp8, pad) in [
                 (torch.bfloat16, 700, 16, 4, 128, 5000, 3, False, 0), (torch.float16, 300, 16, 8, 128, 2500, 0, True, 0),
@@ -866,6 +866,80 @@ def test_paged_append_both_tile_widths(width, monkeypatch):
             assert same_bits(kc_g, kc) and same_bits(vc_g, vc), f"T={T} H={H} D={D} fp8={fp8}"
     finally:
         hooks.emm_hook_set_move_variant(old)
+
+
+@pytest.mark.parametrize("cols", [1, 2], ids=["columns of 128 row elements", "columns of 32 row elements"])
+def test_paged_append_one_wave_kernel_both_column_widths(cols, monkeypatch):
+    """16-bit caches with aligned sources and a power-of-two block size from 16 on take the kernel of one-wave
+    workgroups, which picks its column width by launch size; here each width is forced on launches of either size:
+    rows that end inside a column, strided sources, prompts on and off the token-tile grid, block size 32 and 64."""
+    hooks = _lib.load_hooks()
+    monkeypatch.setattr(_lib, "_lib", hooks)
+    old = hooks.emm_hook_set_move_variant(cols << 29)
+    try:
+        for (dtype, NB, bs, H, D, T, phase, pad) in [
+                (torch.bfloat16, 700, 16, 4, 128, 5000, 3, 0), (torch.float16, 300, 16, 8, 128, 2500, 0, 0),
+                (torch.bfloat16, 64, 16, 4, 128, 256, 5, 0), (torch.bfloat16, 33, 16, 5, 104, 77, 2, 0),
+                (torch.float16, 80, 16, 3, 40, 300, 4, 8), (torch.bfloat16, 48, 32, 2, 64, 700, 1, 8),
+                (torch.bfloat16, 60, 64, 1, 72, 900, 15, 0), (torch.bfloat16, 30, 16, 20, 128, 100, 1, 0),
+                (torch.float16, 40, 16, 1, 8, 333, 0, 0)]:
+            say(f"paged append, one-wave kernel, column code {cols}: {dtype} NB={NB} bs={bs} H={H} D={D} T={T} pad={pad}")
+            g = torch.Generator().manual_seed(NB * 7 + T + cols)
+            slots = paged_slots(NB, bs, T, seed=T + 1, phase=phase)
+            assert len(slots) == T
+            src = (torch.randn((T, 2 * H * D + pad), generator=g) * 3).to(dtype)
+            src_g = src.to(DEV)
+            k_g, v_g = src_g[:, :H * D].view(T, H, D), src_g[:, H * D:2 * H * D].view(T, H, D)
+            kh = src[:, :H * D].reshape(T, H, D).contiguous()
+            vh = src[:, H * D:2 * H * D].reshape(T, H, D).contiguous()
+            kc, vc = paged_caches_cpu(NB, H, D, bs, dtype)
+            kc_g, vc_g = kc.to(DEV), vc.to(DEV)
+            cache_ops.reshape_and_cache(k_g, v_g, kc_g, vc_g, slots.to(DEV))
+            orc.c_reshape_and_cache_paged(kh, vh, kc, vc, slots)
+            assert same_bits(kc_g, kc) and same_bits(vc_g, vc), f"T={T} H={H} D={D}"
+    finally:
+        hooks.emm_hook_set_move_variant(old)
+
+
+def test_paged_append_runs_at_every_position_and_broken_runs():
+    """What decides between the whole-run path and token-by-token stores, one case at a time: a 16-token run
+    starting at every position of the token list relative to the 16-token tiles, at the very start and the very
+    end of the list, runs that only look whole (a padded slot, a repeated slot, a slot past the pool, a gap, a
+    start that is not a multiple of 16 slots inside a block of 32), two whole runs back to back, and 17 / 31 / 32
+    consecutive slots."""
+    NB, bs, H, D = 40, 32, 2, 64
+    g = torch.Generator().manual_seed(1234)
+    cases = []
+    for start in range(0, 34):  # `start` single tokens, then one whole run, then 3 single tokens
+        lone = [(3 + i) * bs + 20 for i in range(start)]  # never inside the run's window
+        cases.append((f"run at token {start}", lone + list(range(20 * bs, 20 * bs + 16)) + [30 * bs + 1, 31 * bs + 2, 32 * bs + 3]))
+    run = list(range(20 * bs + 16, 20 * bs + 32))  # the second 16-slot window of block 20
+    cases.append(("run alone", run))
+    cases.append(("run at the end", [5, 70, 200] + run))
+    broken = list(run); broken[9] = -1
+    cases.append(("padded slot inside", [1] * 0 + broken + [99]))
+    broken = list(run); broken[4] = broken[3]
+    cases.append(("repeated slot inside", broken[:4] + broken[5:]))  # 15 tokens, consecutive except one step of 2
+    broken = list(run); broken[15] = NB * bs + 5
+    cases.append(("last slot past the pool", broken))
+    cases.append(("gap in the middle", run[:8] + [700] + run[8:]))
+    cases.append(("start not at a window start", list(range(20 * bs + 8, 20 * bs + 24))))
+    cases.append(("two runs back to back", list(range(20 * bs, 20 * bs + 32))))
+    cases.append(("two runs, other order", list(range(20 * bs + 16, 20 * bs + 32)) + list(range(20 * bs, 20 * bs + 16))))
+    for n in (15, 17, 31, 32, 33, 47, 48, 49, 64):
+        cases.append((f"{n} consecutive slots from 5", list(range(9 * bs + 5, 9 * bs + 5 + n))))
+        cases.append((f"{n} consecutive slots from a block start", list(range(9 * bs, 9 * bs + n))))
+    for name, sl in cases:
+        say(f"paged append, run edges: {name}")
+        slots = torch.tensor(sl, dtype=torch.long)
+        T = len(sl)
+        key = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+        value = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+        kc, vc = paged_caches_cpu(NB, H, D, bs, torch.bfloat16)
+        kc_g, vc_g = kc.to(DEV), vc.to(DEV)
+        cache_ops.reshape_and_cache(key.to(DEV), value.to(DEV), kc_g, vc_g, slots.to(DEV))
+        orc.c_reshape_and_cache_paged(key, value, kc, vc, slots)
+        assert same_bits(kc_g, kc) and same_bits(vc_g, vc), name
 
 
 def test_paged_append_seeded_sweep_of_shapes():
