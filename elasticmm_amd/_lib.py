@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p, POINTER
 
 from .build import hooks_library_path, library_path
 
-EMM_KV_ABI_VERSION = 2
+EMM_KV_ABI_VERSION = 3
 EMM_MAX_LAYERS = 96
 EMM_MAX_SEGMENTS = 128
 EMM_MAX_INLINE_IDS = 512
@@ -43,6 +43,8 @@ SIGNATURES = {
                                                  c_int64, c_int64, _P, _P, c_int, _P]),
     "emm_reshape_and_cache_strided": (c_int, [_PP, _PP, _PP, _PP, c_int, _P, c_int64, c_int, c_int64, c_int, c_int64,
                                               c_int64, c_int64, c_int64, c_int64, c_int64, _P]),
+    "emm_reshape_and_cache_strided_fp8": (c_int, [_PP, _PP, _PP, _PP, c_int, _P, c_int64, c_int, c_int64, c_int, c_int64,
+                                                  c_int64, c_int64, c_int64, c_int64, c_int64, _P, _P, c_int, _P]),
     "emm_reshape_and_cache_paged": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int64, c_int64,
                                             c_int64, c_int, c_int, _P, _P, _P]),
     "emm_reshape_and_cache_paged_layers": (c_int, [_PP, _PP, _PP, _PP, c_int, _P, c_int64, c_int, c_int, c_int,

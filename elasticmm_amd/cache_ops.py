@@ -28,7 +28,7 @@ def reshape_and_cache_flash(key: torch.Tensor, value: torch.Tensor, key_cache: t
                             value_cache: torch.Tensor, slot_mapping: torch.Tensor, kv_cache_dtype: str = "auto",
                             k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None) -> None:
     """key, value ``[num_tokens, num_heads, head_size]``; caches
-    ``[num_blocks, block_size, num_heads, head_size]`` (contiguous, or for "auto" a strided view with
+    ``[num_blocks, block_size, num_heads, head_size]`` (contiguous, or a strided view with
     contiguous head rows such as a permuted head-major pool); ``slot_mapping`` int64
     ``[num_tokens]`` with -1 for padded tokens. ``kv_cache_dtype`` is "auto" (cache
     dtype == key dtype, bit copy), "fp8" / "fp8_e4m3" (cache is 1 byte wide and
@@ -44,8 +44,12 @@ def reshape_and_cache_flash(key: torch.Tensor, value: torch.Tensor, key_cache: t
     elif kv_cache_dtype in _FP8_MODES:
         if key_cache.element_size() != 1:
             raise ValueError("fp8 KV cache must be a 1-byte tensor (float8_e4m3fn or uint8)")
-        kv_ops.reshape_and_cache(key, value, key_cache, value_cache, slot_mapping, k_scale, v_scale,
-                                 saturate=_FP8_MODES[kv_cache_dtype])
+        if key_cache.is_contiguous() and value_cache.is_contiguous():
+            kv_ops.reshape_and_cache(key, value, key_cache, value_cache, slot_mapping, k_scale, v_scale,
+                                     saturate=_FP8_MODES[kv_cache_dtype])
+        else:  # an fp8 pool in the head-major layout, passed as a permuted view
+            kv_ops.reshape_and_cache_strided([key], [value], [key_cache], [value_cache], slot_mapping, k_scale,
+                                             v_scale, saturate=_FP8_MODES[kv_cache_dtype])
     else:
         raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
 

@@ -1231,6 +1231,140 @@ int append_strided(const void *const *k, const void *const *v, void *const *kc, 
   return check_launch(what);
 }
 
+// The quantising append for the same strided caches (an fp8 pool in the head-major layout): one wave quantises
+// one token row of K or V (grid y = 2) exactly as emm_append_fp8_kernel does — 1024-element pieces, lane i converts
+// elements [8 i, 8 i + 8) and [512 + 8 i, ...), the same quotient and conversion — and cuts the row into heads on
+// the way out: element e of slot (b, o) goes to cache + b * block_stride + o * page_stride + (e / head_elems) *
+// head_stride + e % head_elems (strides in bytes = elements). VEC_ELEMS = 8 needs head rows that are a multiple of
+// 8 elements, so that an 8-byte store never crosses a head; VEC_ELEMS = 1 is the element-wise path for everything else.
+template <int SRC_DTYPE, int VEC_ELEMS, bool SAT, bool TABLES>
+__global__ __launch_bounds__(kThreads) void emm_append_strided_fp8_kernel(
+    const int64_t *__restrict__ slot_mapping, const char *key, const char *value, uint32_t num_tokens,
+    uint32_t row, uint32_t key_stride, uint32_t value_stride, const float *__restrict__ k_scales,
+    const float *__restrict__ v_scales, char *key_cache, char *value_cache, uint32_t head_elems, uint32_t block_size,
+    int64_t num_slots, int64_t block_stride, int64_t page_stride, int64_t head_stride, int32_t fast_div,
+    const std::conditional_t<TABLES, AppendTables, NoTables> tables) {
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t kv = blockIdx.y, l = TABLES ? blockIdx.z : 0;
+  const uint32_t t = blockIdx.x * kWavesPerGroup + wave;
+  if (t >= num_tokens) return;
+  if constexpr (TABLES) {
+    key = tables.key[l];
+    value = tables.value[l];
+    key_cache = tables.key_cache[l];
+    value_cache = tables.value_cache[l];
+  }
+  const char *src = (kv == 0 ? key : value) + (uint64_t)t * (kv == 0 ? key_stride : value_stride) * 2;
+  char *dst_base = kv == 0 ? key_cache : value_cache;
+  int64_t slot = slot_mapping[t];
+  const float scale = kv == 0 ? k_scales[l] : v_scales[l];
+  const bool head_pow2 = (head_elems & (head_elems - 1)) == 0;
+  auto in_heads = [&](uint32_t e) -> int64_t {
+    const uint32_t h = head_pow2 ? e >> __builtin_ctz(head_elems) : e / head_elems;
+    return (int64_t)h * head_stride + (e - h * head_elems);
+  };
+  auto row_base = [&](int64_t s) -> char * {
+    const int64_t blk = (block_size & (block_size - 1)) == 0 ? s >> __builtin_ctz(block_size) : s / block_size;
+    return dst_base + blk * block_stride + (s - blk * block_size) * page_stride;
+  };
+  if constexpr (VEC_ELEMS == 8) {
+    uint32_t e0 = lane * 8, e1 = e0 + 512;
+    u32x4 a = ld<u32x4, true>(src + (e0 < row ? e0 : 0) * 2); // issued before slot and scale are waited for
+    u32x4 b = ld<u32x4, true>(src + (e1 < row ? e1 : 0) * 2);
+    asm volatile("" : "+s"(slot) : : "memory");
+    if ((uint64_t)slot >= (uint64_t)num_slots) return;
+    const Divisor div = make_divisor(scale, fast_div != 0);
+    char *dp = row_base(slot);
+    while (e0 < row) {
+      const u32x2 qa = quant8<SRC_DTYPE, SAT>(a, div);
+      const u32x2 qb = quant8<SRC_DTYPE, SAT>(b, div);
+      st_stream<u32x2, 1>(dp + in_heads(e0), qa);
+      if (e1 < row) st_stream<u32x2, 1>(dp + in_heads(e1), qb);
+      e0 += 1024;
+      e1 += 1024;
+      if (e0 < row) {
+        a = ld<u32x4, true>(src + e0 * 2);
+        b = ld<u32x4, true>(src + (e1 < row ? e1 : e0) * 2);
+      }
+    }
+  } else {
+    if ((uint64_t)slot >= (uint64_t)num_slots) return;
+    char *dp = row_base(slot);
+    for (uint32_t e = lane; e < row; e += 64) {
+      const uint16_t h = ld<uint16_t, false>(src + (int64_t)e * 2);
+      st<uint8_t, false>(dp + in_heads(e), quant1<SRC_DTYPE, SAT>(h, scale));
+    }
+  }
+}
+
+template <int DT, int VEC, bool SAT>
+void launch_append_strided_fp8(bool tables, const AppendTables &t, const int64_t *slot_mapping, const float *k_scales,
+                               const float *v_scales, int64_t num_tokens, int64_t row, int64_t ks, int64_t vs,
+                               int64_t head_elems, int block_size, int64_t num_slots, int64_t block_stride,
+                               int64_t page_stride, int64_t head_stride, int fast_div, int num_layers, hipStream_t s) {
+  const uint32_t gx = (uint32_t)((num_tokens + kWavesPerGroup - 1) / kWavesPerGroup);
+  if (tables)
+    emm_append_strided_fp8_kernel<DT, VEC, SAT, true><<<dim3(gx, 2, (uint32_t)num_layers), kThreads, 0, s>>>(
+        slot_mapping, nullptr, nullptr, (uint32_t)num_tokens, (uint32_t)row, (uint32_t)ks, (uint32_t)vs, k_scales,
+        v_scales, nullptr, nullptr, (uint32_t)head_elems, (uint32_t)block_size, num_slots, block_stride, page_stride,
+        head_stride, fast_div, t);
+  else
+    emm_append_strided_fp8_kernel<DT, VEC, SAT, false><<<dim3(gx, 2), kThreads, 0, s>>>(
+        slot_mapping, t.key[0], t.value[0], (uint32_t)num_tokens, (uint32_t)row, (uint32_t)ks, (uint32_t)vs, k_scales,
+        v_scales, t.key_cache[0], t.value_cache[0], (uint32_t)head_elems, (uint32_t)block_size, num_slots,
+        block_stride, page_stride, head_stride, fast_div, NoTables{});
+}
+
+int append_strided_fp8(const void *const *k, const void *const *v, void *const *kc, void *const *vc, int num_layers,
+                       const int64_t *slot_mapping, int64_t num_tokens, int num_heads, int64_t head_elems,
+                       int block_size, int64_t num_blocks, int64_t ks, int64_t vs, int64_t block_stride,
+                       int64_t page_stride, int64_t head_stride, const float *k_scales, const float *v_scales,
+                       int src_dtype, hipStream_t s, const char *what) {
+  if (num_layers < 0 || num_layers > EMM_MAX_LAYERS)
+    return fail(EMM_EINVAL, "%s: num_layers=%d outside [0, %d]", what, num_layers, EMM_MAX_LAYERS);
+  if (num_tokens < 0 || num_heads < 0 || head_elems < 0 || block_size <= 0 || num_blocks < 0 || ks < 0 || vs < 0 ||
+      block_stride < 0 || page_stride < 0 || head_stride < 0)
+    return fail(EMM_EINVAL, "%s: negative size", what);
+  const bool sat = (src_dtype & EMM_FP8_SATURATE) != 0;
+  const int dt = src_dtype & ~EMM_FP8_SATURATE;
+  if (dt != EMM_DTYPE_BF16 && dt != EMM_DTYPE_F16) return fail(EMM_EINVAL, "%s: unknown src_dtype %d", what, src_dtype);
+  const int64_t row = (int64_t)num_heads * head_elems;
+  if (num_tokens == 0 || row == 0 || num_layers == 0) return EMM_OK;
+  if (head_elems > 0x7fffffffLL || row > 0x7fffffffLL) return fail(EMM_EINVAL, "%s: row too long", what);
+  if (!k || !v || !kc || !vc || !slot_mapping) return fail(EMM_EINVAL, "%s: null pointer", what);
+  if (!k_scales || !v_scales) return fail(EMM_EINVAL, "%s: scale pointer is null", what);
+  if (ks < row || vs < row) return fail(EMM_EINVAL, "%s: token stride smaller than the row", what);
+  if (head_stride < head_elems || page_stride < head_elems)
+    return fail(EMM_EINVAL, "%s: head / page stride smaller than a head row", what);
+  if (num_tokens > 0x7fffffffLL || ks > 0x7fffffffLL || vs > 0x7fffffffLL)
+    return fail(EMM_EINVAL, "%s: too many tokens / token stride too large", what);
+  AppendTables t;
+  int width = (head_elems % 8 || ks % 8 || vs % 8 || block_stride % 8 || page_stride % 8 || head_stride % 8) ? 1 : 8;
+  for (int l = 0; l < num_layers; ++l) {
+    if (!k[l] || !v[l] || !kc[l] || !vc[l]) return fail(EMM_EINVAL, "%s: null tensor pointer at layer %d", what, l);
+    if (!aligned(k[l], 2) || !aligned(v[l], 2))
+      return fail(EMM_EINVAL, "%s: 16-bit source not 2-byte aligned at layer %d", what, l);
+    if (!aligned(k[l], 16) || !aligned(v[l], 16) || !aligned(kc[l], 8) || !aligned(vc[l], 8)) width = 1;
+  }
+  fill_tables(t, k, v, kc, vc, num_layers);
+  const bool tables = num_layers > 1;
+  const int64_t num_slots = num_blocks * block_size;
+  const int fast_div = (move_variant() & 0x1000000) ? 0 : 1;
+#define EMM_SFP8_LAUNCH(DT, VEC, SAT) \
+  launch_append_strided_fp8<DT, VEC, SAT>(tables, t, slot_mapping, k_scales, v_scales, num_tokens, row, ks, vs, head_elems, \
+                                          block_size, num_slots, block_stride, page_stride, head_stride, fast_div, num_layers, s)
+  if (dt == EMM_DTYPE_BF16) {
+    if (width == 8) { if (sat) EMM_SFP8_LAUNCH(EMM_DTYPE_BF16, 8, true); else EMM_SFP8_LAUNCH(EMM_DTYPE_BF16, 8, false); }
+    else { if (sat) EMM_SFP8_LAUNCH(EMM_DTYPE_BF16, 1, true); else EMM_SFP8_LAUNCH(EMM_DTYPE_BF16, 1, false); }
+  } else {
+    if (width == 8) { if (sat) EMM_SFP8_LAUNCH(EMM_DTYPE_F16, 8, true); else EMM_SFP8_LAUNCH(EMM_DTYPE_F16, 8, false); }
+    else { if (sat) EMM_SFP8_LAUNCH(EMM_DTYPE_F16, 1, true); else EMM_SFP8_LAUNCH(EMM_DTYPE_F16, 1, false); }
+  }
+#undef EMM_SFP8_LAUNCH
+  return check_launch(what);
+}
+
 // ----------------------------------------------------------------------------
 // reshape_and_cache, paged-attention layout: the one place where source and
 // destination layouts transpose, staged through LDS
@@ -2178,6 +2312,20 @@ int emm_reshape_and_cache_strided(const void *const *key_ptrs, const void *const
                         num_tokens, num_heads, head_bytes, block_size, num_blocks, key_stride_bytes,
                         value_stride_bytes, block_stride_bytes, page_stride_bytes, head_stride_bytes,
                         as_stream(stream), "emm_reshape_and_cache_strided");
+}
+
+int emm_reshape_and_cache_strided_fp8(const void *const *key_ptrs, const void *const *value_ptrs,
+                                      void *const *key_cache_ptrs, void *const *value_cache_ptrs, int num_layers,
+                                      const int64_t *slot_mapping, int64_t num_tokens, int num_heads,
+                                      int64_t head_elems, int block_size, int64_t num_blocks,
+                                      int64_t key_stride_elems, int64_t value_stride_elems,
+                                      int64_t block_stride_bytes, int64_t page_stride_bytes,
+                                      int64_t head_stride_bytes, const float *k_scales, const float *v_scales,
+                                      int src_dtype, emm_stream_t stream) {
+  return append_strided_fp8(key_ptrs, value_ptrs, key_cache_ptrs, value_cache_ptrs, num_layers, slot_mapping,
+                            num_tokens, num_heads, head_elems, block_size, num_blocks, key_stride_elems,
+                            value_stride_elems, block_stride_bytes, page_stride_bytes, head_stride_bytes, k_scales,
+                            v_scales, src_dtype, as_stream(stream), "emm_reshape_and_cache_strided_fp8");
 }
 
 int emm_reshape_and_cache_paged(const void *key, const void *value, void *key_cache, void *value_cache,

@@ -366,10 +366,12 @@ def reshape_and_cache(key: torch.Tensor, value: torch.Tensor, key_cache: torch.T
 
 def reshape_and_cache_strided(keys: Sequence[torch.Tensor], values: Sequence[torch.Tensor],
                               key_caches: Sequence[torch.Tensor], value_caches: Sequence[torch.Tensor],
-                              slot_mapping: torch.Tensor) -> None:
+                              slot_mapping: torch.Tensor, k_scales=None, v_scales=None, saturate: bool = False) -> None:
     """The flash-layout append for caches that are strided views ``[NB, bs, H, D]`` (stride 1 along D),
-    such as a head-major pool ``[NB, H, bs, D]`` seen through ``permute(0, 2, 1, 3)``. Same-width copy;
-    one launch for all layers given (they must share shapes and strides)."""
+    such as a head-major pool ``[NB, H, bs, D]`` seen through ``permute(0, 2, 1, 3)``. Caches of the
+    sources' element width are copied bit for bit; 1-byte caches with 16-bit sources are quantised to
+    fp8-e4m3fn with the per-layer ``k_scales`` / ``v_scales`` (``saturate``: the clamping mode). One launch
+    for all layers given (they must share shapes and strides)."""
     lib = _lib.load()
     L = len(keys)
     if not (len(values) == len(key_caches) == len(value_caches) == L):
@@ -387,32 +389,42 @@ def reshape_and_cache_strided(keys: Sequence[torch.Tensor], values: Sequence[tor
     if kc.dim() != 4 or tuple(kc.shape[2:]) != (H, D) or vc.shape != kc.shape or vc.stride() != kc.stride():
         raise ValueError("caches must be [num_blocks, block_size, num_heads, head_size] views of one geometry")
     eb = k.element_size()
-    if kc.element_size() != eb or vc.element_size() != eb or v.element_size() != eb:
-        raise TypeError("reshape_and_cache_strided copies same-width elements only")
+    ceb = kc.element_size()
+    fp8 = ceb == 1 and eb == 2
+    if v.element_size() != eb or vc.element_size() != ceb or not (fp8 or ceb == eb):
+        raise TypeError(f"unsupported source/cache element sizes {eb}/{ceb}")
     if D > 1 and kc.stride(3) != 1:
         raise ValueError("head rows of the cache must be contiguous")
     _, _, ks = _row_geometry(k, "key")
     _, _, vs = _row_geometry(v, "value")
     NB, bs = int(kc.shape[0]), int(kc.shape[1])
-    geom = (T, H, D, eb, NB, bs, ks, vs, kc.stride(0), kc.stride(1), kc.stride(2))
+    sb, sp, sh = kc.stride(0), kc.stride(1), kc.stride(2)
     sig = lambda t: (t.shape, t.stride(), t.dtype, t.device)  # noqa: E731
     want = (sig(k), sig(v), sig(kc), sig(vc))
     for l in range(1, L):
         if (sig(keys[l]), sig(values[l]), sig(key_caches[l]), sig(value_caches[l])) != want:
             raise ValueError(f"layer {l}: geometry differs from layer 0")
-    T, H, D, eb, NB, bs, ks, vs, sb, sp, sh = geom
     slot_mapping = _check_slot_mapping(slot_mapping, T)
     stream = _stream_ptr(keys[0].device)
+    if fp8:
+        if k_scales is None or v_scales is None:
+            raise ValueError("fp8 cache needs k_scales and v_scales")
+        code = _half_code(k.dtype, "reshape_and_cache_strided", saturate)
+        k_s = _scales_tensor(k_scales, L, k.device)
+        v_s = _scales_tensor(v_scales, L, k.device)
     for l0 in range(0, L, EMM_MAX_LAYERS):
         sl = slice(l0, l0 + EMM_MAX_LAYERS)
         n = len(keys[sl])
-        check(lib.emm_reshape_and_cache_strided(ptr_table([t.data_ptr() for t in keys[sl]]),
-                                                ptr_table([t.data_ptr() for t in values[sl]]),
-                                                ptr_table([t.data_ptr() for t in key_caches[sl]]),
-                                                ptr_table([t.data_ptr() for t in value_caches[sl]]), n,
-                                                slot_mapping.data_ptr(), T, H, D * eb, bs, NB, ks * eb, vs * eb,
-                                                sb * eb, sp * eb, sh * eb, stream),
-              "emm_reshape_and_cache_strided")
+        tables = (ptr_table([t.data_ptr() for t in keys[sl]]), ptr_table([t.data_ptr() for t in values[sl]]),
+                  ptr_table([t.data_ptr() for t in key_caches[sl]]), ptr_table([t.data_ptr() for t in value_caches[sl]]))
+        if fp8:
+            check(lib.emm_reshape_and_cache_strided_fp8(*tables, n, slot_mapping.data_ptr(), T, H, D, bs, NB, ks, vs,
+                                                        sb, sp, sh, k_s.data_ptr() + 4 * l0, v_s.data_ptr() + 4 * l0,
+                                                        code, stream), "emm_reshape_and_cache_strided_fp8")
+        else:
+            check(lib.emm_reshape_and_cache_strided(*tables, n, slot_mapping.data_ptr(), T, H, D * eb, bs, NB, ks * eb,
+                                                    vs * eb, sb * eb, sp * eb, sh * eb, stream),
+                  "emm_reshape_and_cache_strided")
 
 
 def _paged_geometry(key: torch.Tensor, value: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor):

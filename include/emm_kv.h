@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define EMM_KV_ABI_VERSION 2
+#define EMM_KV_ABI_VERSION 3
 #define EMM_MAX_LAYERS 96   /* layer pointers carried in one kernel argument block */
 #define EMM_MAX_SEGMENTS 128 /* ragged segments carried by one emm_concat_rows launch */
 #define EMM_MAX_INLINE_IDS 512 /* block ids carried by one launch of emm_kv_*_host_ids (longer tables: several launches) */
@@ -236,7 +236,7 @@ int emm_reshape_and_cache_fp8_layers(const void *const *key_ptrs,
  * b, o = divmod(slot_mapping[t], block_size); head rows (head_bytes) stay
  * contiguous. One launch for num_layers layers (HOST pointer tables as in
  * emm_reshape_and_cache_layers; all layers share the geometry). Same-width
- * copy only. Same call sites as emm_reshape_and_cache
+ * copy only (emm_reshape_and_cache_strided_fp8 quantises). Same call sites as emm_reshape_and_cache
  * (elasticmm/engine/v0/worker_steps.py:281, :438).
  */
 int emm_reshape_and_cache_strided(const void *const *key_ptrs,
@@ -252,6 +252,40 @@ int emm_reshape_and_cache_strided(const void *const *key_ptrs,
                                   int64_t page_stride_bytes,
                                   int64_t head_stride_bytes,
                                   emm_stream_t stream);
+
+/*
+ * reshape_and_cache (flash layout, free cache strides, fp8-e4m3fn cache) — the
+ * quantising append of emm_reshape_and_cache_fp8 for the strided caches of
+ * emm_reshape_and_cache_strided: a 1-byte cache whose blocks, slots and heads are
+ * block_stride / page_stride / head_stride bytes apart (an fp8 pool in the
+ * head-major layout [num_blocks, num_heads, block_size, head_size] passed as a
+ * permuted view). Element d of head h of token t goes to
+ * cache + b * block_stride + o * page_stride + h * head_stride + d as
+ * e4m3fn(float(x) / scale), same rounding and overflow modes as
+ * emm_reshape_and_cache_fp8 (src_dtype: EMM_DTYPE_BF16 / EMM_DTYPE_F16, optionally
+ * | EMM_FP8_SATURATE). key / value strides in source elements; k_scales / v_scales
+ * are DEVICE float arrays of num_layers. One launch for num_layers layers (HOST
+ * pointer tables; all layers share the geometry). The cache dtype the reference
+ * leaves open at elasticmm/engine/v0/worker.py:194, reached from
+ * elasticmm/engine/v0/worker_steps.py:281, :438.
+ */
+int emm_reshape_and_cache_strided_fp8(const void *const *key_ptrs,
+                                      const void *const *value_ptrs,
+                                      void *const *key_cache_ptrs,
+                                      void *const *value_cache_ptrs,
+                                      int num_layers,
+                                      const int64_t *slot_mapping,
+                                      int64_t num_tokens, int num_heads,
+                                      int64_t head_elems, int block_size,
+                                      int64_t num_blocks,
+                                      int64_t key_stride_elems,
+                                      int64_t value_stride_elems,
+                                      int64_t block_stride_bytes,
+                                      int64_t page_stride_bytes,
+                                      int64_t head_stride_bytes,
+                                      const float *k_scales,
+                                      const float *v_scales, int src_dtype,
+                                      emm_stream_t stream);
 
 /*
  * reshape_and_cache (paged-attention layout) — append into the transposed pool

@@ -319,6 +319,42 @@ int main(void) {
                                 stride_elems, num_slots, h_ks[l], h_vs[l], EMM_DTYPE_F16);
       bad += same_on_device(d_p8[l], h_p8[l], layer8, "emm_reshape_and_cache_fp8_layers (f16 source)");
     }
+    /* the quantising append into a head-major fp8 cache [NB, H, BS, D] through the strided entry point: the contiguous
+     * append of the oracle on a copy of the pool, permuted, is the expected content */
+    {
+      int64_t h_slots3[T];
+      permutation(h_slots3, num_slots, T);
+      h_slots3[1] = -1;
+      int64_t *d_slots3 = (int64_t *)to_device(h_slots3, sizeof(h_slots3));
+      uint8_t *h_flat = (uint8_t *)malloc(layer8), *h_hm = (uint8_t *)malloc(layer8);
+      void *d_hm[L], *d_hk[L], *d_hv[L];
+      for (int l = 0; l < L; ++l) {
+        for (int kv = 0; kv < 2; ++kv)
+          for (int64_t b = 0; b < NB; ++b)
+            for (int o = 0; o < BS; ++o)
+              for (int h = 0; h < H; ++h)
+                memcpy(h_hm + kv * plane8 + b * chunk_elems + ((size_t)h * BS + o) * D,
+                       h_p8[l] + kv * plane8 + b * chunk_elems + ((size_t)o * H + h) * D, D);
+        d_hm[l] = to_device(h_hm, layer8);
+        d_hk[l] = d_hm[l];
+        d_hv[l] = (char *)d_hm[l] + plane8;
+      }
+      EMM(emm_reshape_and_cache_strided_fp8((const void *const *)d_keys, (const void *const *)d_vals, d_hk, d_hv, L, d_slots3,
+                                            T, H, D, BS, NB, stride_elems, stride_elems, chunk_elems, D, (int64_t)BS * D,
+                                            d_ks, d_vs, EMM_DTYPE_BF16, stream));
+      for (int l = 0; l < L; ++l) {
+        memcpy(h_flat, h_p8[l], layer8);
+        orc_reshape_and_cache_fp8(h_keys[l], h_vals[l], h_flat, h_flat + plane8, h_slots3, T, row_elems, stride_elems,
+                                  stride_elems, num_slots, h_ks[l], h_vs[l], EMM_DTYPE_BF16);
+        for (int kv = 0; kv < 2; ++kv)
+          for (int64_t b = 0; b < NB; ++b)
+            for (int o = 0; o < BS; ++o)
+              for (int h = 0; h < H; ++h)
+                memcpy(h_hm + kv * plane8 + b * chunk_elems + ((size_t)h * BS + o) * D,
+                       h_flat + kv * plane8 + b * chunk_elems + ((size_t)o * H + h) * D, D);
+        bad += same_on_device(d_hm[l], h_hm, layer8, "emm_reshape_and_cache_strided_fp8");
+      }
+    }
     /* fp8 bytes travel through pack unchanged (chunk = chunk_elems bytes); the receiving pool is bf16 */
     const size_t packed8 = (size_t)L * 2 * N * chunk_elems;
     uint8_t *h_packed8 = (uint8_t *)malloc(packed8);

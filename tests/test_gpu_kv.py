@@ -661,6 +661,64 @@ def test_append_into_head_major_and_padded_caches():
             assert same_bits(pad_g[l], pad_c[l]), f"padded, layer {l}"
 
 
+def test_fp8_append_into_head_major_and_padded_caches():
+    """The quantising append into strided fp8 caches: a head-major pool [NB, H, bs, D] seen as [NB, bs, H, D]
+    (through the vLLM-shaped call, one layer at a time) and a padded pool (all layers in one launch). Expected
+    result = the contiguous fp8 append of the C oracle, permuted: the bytes of a slot's heads are the same, only
+    where they lie differs. Both overflow modes, bf16 and f16 sources, head sizes that are not a multiple of 8
+    (the element-wise path), block sizes that are not powers of two, rows longer than 1024 elements."""
+    g = torch.Generator().manual_seed(43)
+    for dtype, NB, bs, H, D, T, L, mode in (
+            (torch.bfloat16, 48, 16, 4, 128, 500, 3, "fp8"), (torch.float16, 20, 8, 3, 20, 77, 1, "fp8"),
+            (torch.bfloat16, 300, 16, 8, 128, 2000, 2, "fp8_e4m3_sat"), (torch.float16, 30, 12, 2, 64, 100, 2, "fp8_sat"),
+            (torch.bfloat16, 64, 16, 6, 256, 601, 1, "fp8"), (torch.bfloat16, 40, 16, 5, 36, 333, 2, "fp8"),
+            (torch.float16, 25, 16, 3, 7, 90, 1, "fp8_sat")):
+        say(f"fp8 strided append: {dtype} NB={NB} bs={bs} H={H} D={D} T={T} L={L} {mode}")
+        sat = mode.endswith("_sat")
+        slots = make_slots(NB * bs, T, 43, pad_frac=0.1)
+        keys = [(torch.randn((T, H, D), generator=g) * 4).to(dtype) for _ in range(L)]
+        values = [(torch.randn((T, H, D), generator=g) * 60).to(dtype) for _ in range(L)]  # part of it overflows
+        ks = torch.linspace(0.02, 0.09, L)
+        vs = torch.linspace(0.31, 0.11, L)
+        # expected: contiguous flash-layout fp8 append of the oracle (the saturating mode through its quantiser)
+        flat = [(torch.full((NB, bs, H, D), 9, dtype=torch.uint8), torch.full((NB, bs, H, D), 9, dtype=torch.uint8))
+                for _ in range(L)]
+        valid = slots >= 0
+        b, o = slots[valid] // bs, slots[valid] % bs
+        for l in range(L):
+            if sat:
+                flat[l][0][b, o] = torch.from_numpy(orc.c_quant_fp8_sat(keys[l][valid], float(ks[l]))).view(-1, H, D)
+                flat[l][1][b, o] = torch.from_numpy(orc.c_quant_fp8_sat(values[l][valid], float(vs[l]))).view(-1, H, D)
+            else:
+                orc.c_reshape_and_cache_fp8(keys[l], values[l], flat[l][0], flat[l][1], slots, float(ks[l]), float(vs[l]))
+        assert sat or int((flat[0][1] & 0x7F).eq(0x7F).sum()) > 0, "no overflow in the values: the case is too tame"
+        # head-major storage, one layer per call
+        store_g = [torch.full((2, NB, H, bs, D), 9, dtype=torch.uint8, device=DEV) for _ in range(L)]
+        for l in range(L):
+            kc = store_g[l][0].permute(0, 2, 1, 3).view(torch.float8_e4m3fn)
+            vc = store_g[l][1].permute(0, 2, 1, 3).view(torch.float8_e4m3fn)
+            assert not kc.is_contiguous()
+            cache_ops.reshape_and_cache_flash(keys[l].to(DEV), values[l].to(DEV), kc, vc, slots.to(DEV), mode,
+                                              ks[l:l + 1].to(DEV), vs[l:l + 1].to(DEV))
+            assert same_bits(store_g[l][0], flat[l][0].permute(0, 2, 1, 3).contiguous()), f"head-major K, layer {l}"
+            assert same_bits(store_g[l][1], flat[l][1].permute(0, 2, 1, 3).contiguous()), f"head-major V, layer {l}"
+        # padded blocks, all layers in one launch; the padding must stay untouched
+        pad_g = [torch.full((2, NB, bs + 1, H, D + 8), 9, dtype=torch.uint8, device=DEV) for _ in range(L)]
+        kv_ops.reshape_and_cache_strided([k.to(DEV) for k in keys], [v.to(DEV) for v in values],
+                                         [t[0, :, :bs, :, :D] for t in pad_g], [t[1, :, :bs, :, :D] for t in pad_g],
+                                         slots.to(DEV), ks, vs, saturate=sat)
+        for l in range(L):
+            want = torch.full((2, NB, bs + 1, H, D + 8), 9, dtype=torch.uint8)
+            want[0, :, :bs, :, :D] = flat[l][0]
+            want[1, :, :bs, :, :D] = flat[l][1]
+            assert same_bits(pad_g[l], want), f"padded, layer {l}"
+    # a 16-bit cache of another width than the source is still refused
+    with pytest.raises(TypeError):
+        kv_ops.reshape_and_cache_strided([torch.zeros((1, 1, 8), dtype=torch.float32, device=DEV)] , [torch.zeros((1, 1, 8), dtype=torch.float32, device=DEV)],
+                                         [torch.zeros((2, 2, 1, 8), dtype=torch.bfloat16, device=DEV)], [torch.zeros((2, 2, 1, 8), dtype=torch.bfloat16, device=DEV)],
+                                         torch.zeros(1, dtype=torch.long, device=DEV))
+
+
 # ---------------------------------------------------------------- append, paged-attention layout
 def paged_slots(NB, bs, T, seed, whole_frac=0.6, pad_frac=0.05, phase=0):
     """A slot table shaped like a serving step: prompts that fill whole blocks in order (the first
