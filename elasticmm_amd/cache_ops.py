@@ -115,7 +115,7 @@ def paged_layered_append(keys: Sequence[torch.Tensor], values: Sequence[torch.Te
     raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r}")
 
 
-def copy_blocks(kv_caches: Sequence[torch.Tensor], *args) -> None:
+def copy_blocks(kv_caches: Sequence[torch.Tensor], *args, strict: bool = False) -> None:
     """Both call shapes vLLM has for this operator; one launch covers every layer, K and V.
 
     ``copy_blocks(kv_caches, block_mapping)`` — the attention-backend form: ``kv_caches`` is the list of
@@ -124,12 +124,15 @@ def copy_blocks(kv_caches: Sequence[torch.Tensor], *args) -> None:
     ``copy_blocks(key_caches, value_caches, block_mapping)`` — the form of ``vllm._custom_ops.copy_blocks``
     that the backends hand their split pools to: per-layer key caches and value caches ``[num_blocks, ...]``
     whose trailing shapes may differ (``[NB, H, D // x, bs, x]`` and ``[NB, H, D, bs]`` in the paged-attention
-    layout) as long as a block has the same number of bytes in both."""
+    layout) as long as a block has the same number of bytes in both.
+
+    ``strict=True`` validates a device-resident ``block_mapping`` before the launch (``IndexError`` for an id outside
+    the pool, at the cost of a synchronisation); by default such pairs are skipped by the kernel."""
     if len(args) == 1:
         (block_mapping,) = args
         if len(kv_caches) == 0 or block_mapping.numel() == 0:
             return
-        kv_ops.copy_blocks(PoolView(kv_caches), block_mapping)
+        kv_ops.copy_blocks(PoolView(kv_caches), block_mapping, strict=strict)
         return
     if len(args) != 2:
         raise TypeError("copy_blocks(kv_caches, block_mapping) or copy_blocks(key_caches, value_caches, block_mapping)")
@@ -139,7 +142,7 @@ def copy_blocks(kv_caches: Sequence[torch.Tensor], *args) -> None:
     if len(kv_caches) == 0 or block_mapping.numel() == 0:
         return
     planes = [t.view(t.shape[0], -1) for t in list(kv_caches) + list(value_caches)]  # one chunk per block and plane
-    kv_ops.copy_blocks(PoolView(planes, num_kv_dim=False), block_mapping)
+    kv_ops.copy_blocks(PoolView(planes, num_kv_dim=False), block_mapping, strict=strict)
 
 
 def swap_blocks(src_kv_cache: torch.Tensor, dst_kv_cache: torch.Tensor, src_to_dst) -> None:

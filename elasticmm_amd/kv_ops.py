@@ -79,6 +79,20 @@ def block_index_tensor(block_indices: IndexLike, num_blocks: int, device: torch.
     return host
 
 
+def check_device_block_ids(idx: torch.Tensor, num_blocks: int, what: str) -> None:
+    """Strict mode for block tables that live on the device: one ``torch.aminmax`` and one read-back (a device
+    synchronisation) before the launch; ``IndexError`` if an id lies outside ``[0, num_blocks)`` — where the
+    reference's ``layer_kv[:, idx]`` (elasticmm/engine/v0/worker.py:597, :604) would trip torch's device-side
+    assert. Without it the kernels skip such ids (a padded table is legal there) and a caller cannot tell."""
+    if idx.numel() == 0:
+        return
+    lo, hi = (int(x) for x in torch.aminmax(idx))
+    if lo < 0 or hi >= num_blocks:
+        bad = lo if lo < 0 else hi
+        raise IndexError(f"{what}: index {bad} is out of bounds for dimension 1 with size {num_blocks} "
+                         f"(device block table, strict mode)")
+
+
 class PoolView:
     """A block pool as the kernels see it: per-layer base pointers + geometry.
 
@@ -142,9 +156,17 @@ class PoolView:
         return (self.num_layers, self.num_kv, n) + self.block_shape
 
 
-def kv_pack(pool: PoolView, block_indices: IndexLike, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Gather ``n`` blocks of every layer into ``[L, num_kv, n, *block_shape]``."""
+def kv_pack(pool: PoolView, block_indices: IndexLike, out: Optional[torch.Tensor] = None,
+            strict: bool = False) -> torch.Tensor:
+    """Gather ``n`` blocks of every layer into ``[L, num_kv, n, *block_shape]``.
+
+    Host tables (lists, numpy, CPU tensors) are always checked with torch's indexing rules. A DEVICE table is
+    trusted: ids outside ``[0, num_blocks)`` are skipped by the kernel and their rows of the result keep whatever
+    the allocation held. ``strict=True`` validates a device table first (``check_device_block_ids``: one
+    reduction and a synchronisation) and raises ``IndexError`` instead."""
     lib = _lib.load()
+    if strict and isinstance(block_indices, torch.Tensor) and block_indices.is_cuda:
+        check_device_block_ids(block_indices, pool.num_blocks, "kv_pack")
     # a table held on the host (the reference's List[int]) travels in the kernel argument block, EMM_MAX_INLINE_IDS
     # ids per launch: no staging, no host-to-device copy
     host = host_block_ids(block_indices, pool.num_blocks)
@@ -172,10 +194,13 @@ def kv_pack(pool: PoolView, block_indices: IndexLike, out: Optional[torch.Tensor
     return out
 
 
-def kv_unpack(pool: PoolView, block_indices: IndexLike, packed: torch.Tensor) -> None:
-    """Scatter ``packed`` ``[L, num_kv, n, ...]`` into the pool under ``block_indices``."""
+def kv_unpack(pool: PoolView, block_indices: IndexLike, packed: torch.Tensor, strict: bool = False) -> None:
+    """Scatter ``packed`` ``[L, num_kv, n, ...]`` into the pool under ``block_indices`` (``strict``: as in
+    ``kv_pack``; without it a device table's out-of-range ids are skipped, their rows dropped)."""
     lib = _lib.load()
     _require_gpu(packed, "kv_unpack")
+    if strict and isinstance(block_indices, torch.Tensor) and block_indices.is_cuda:
+        check_device_block_ids(block_indices, pool.num_blocks, "kv_unpack")
     host = host_block_ids(block_indices, pool.num_blocks)
     inline = host is not None and not pool.on_host
     idx = None if inline else block_index_tensor(host if host is not None else block_indices, pool.num_blocks,
@@ -201,9 +226,15 @@ def kv_unpack(pool: PoolView, block_indices: IndexLike, packed: torch.Tensor) ->
                                     idx.data_ptr(), n, packed.data_ptr() + l0 * plane, stream), "emm_kv_unpack")
 
 
-def kv_migrate(src: PoolView, src_indices: IndexLike, dst: PoolView, dst_indices: IndexLike) -> None:
-    """``dst[l][:, dst_idx[j]] = src[l][:, src_idx[j]]`` in one launch, no staging buffer."""
+def kv_migrate(src: PoolView, src_indices: IndexLike, dst: PoolView, dst_indices: IndexLike,
+               strict: bool = False) -> None:
+    """``dst[l][:, dst_idx[j]] = src[l][:, src_idx[j]]`` in one launch, no staging buffer (``strict``: as in
+    ``kv_pack``, for either table)."""
     lib = _lib.load()
+    if strict:
+        for idx, pool, what in ((src_indices, src, "kv_migrate (source table)"), (dst_indices, dst, "kv_migrate (destination table)")):
+            if isinstance(idx, torch.Tensor) and idx.is_cuda:
+                check_device_block_ids(idx, pool.num_blocks, what)
     if (src.num_layers, src.num_kv, src.chunk_bytes, src.device) != (dst.num_layers, dst.num_kv, dst.chunk_bytes, dst.device):
         raise ValueError("kv_migrate: pools differ in layers / kv / chunk size / device")
     if src.on_host and dst.on_host:
@@ -218,9 +249,13 @@ def kv_migrate(src: PoolView, src_indices: IndexLike, dst: PoolView, dst_indices
                                  si.data_ptr(), di.data_ptr(), si.numel(), stream), "emm_kv_migrate")
 
 
-def copy_blocks(pool: PoolView, block_mapping: Union[torch.Tensor, Sequence[Sequence[int]]]) -> None:
-    """All layers: ``pool[:, dst] = pool[:, src]`` for the (src, dst) rows of ``block_mapping``."""
+def copy_blocks(pool: PoolView, block_mapping: Union[torch.Tensor, Sequence[Sequence[int]]],
+                strict: bool = False) -> None:
+    """All layers: ``pool[:, dst] = pool[:, src]`` for the (src, dst) rows of ``block_mapping`` (``strict``: a
+    device mapping is validated first, as in ``kv_pack``; without it pairs with an id out of range are skipped)."""
     lib = _lib.load()
+    if strict and isinstance(block_mapping, torch.Tensor) and block_mapping.is_cuda:
+        check_device_block_ids(block_mapping, pool.num_blocks, "copy_blocks")
     if isinstance(block_mapping, torch.Tensor):
         m = block_mapping
         if m.dtype != torch.long or m.dim() != 2 or m.shape[1] != 2:

@@ -12,17 +12,24 @@ are plain method calls. The reference's batching path is disabled in the product
 code refers to undefined names (:439); here the queue is keyed by (src_rank, dst_rank) and a flush
 moves the merged tables with one pack launch and one unpack launch.
 
-The coroutines (``transfer_kv_cache``, ``transfer_vision_embeddings``, ``migrate_requests``) hand
-the blocking work — kernel launches followed by the device synchronisation the workers perform, as
-the reference's do (worker.py:684, :724) — to one worker thread of the manager and await it, so the
-event loop that calls them (the reference's is stage_engine.py:1506) keeps serving other coroutines
-while a transfer runs. Transfers of one manager run one after the other in that thread. The
-``*_sync`` forms do the same work on the calling thread.
+The coroutines (``transfer_kv_cache``, ``transfer_vision_embeddings``, ``migrate_requests``) run
+their ``*_sync`` bodies on the calling (event-loop) thread without an await point in between. Two
+guarantees follow, and callers may rely on both:
+
+* the host bookkeeping of a transfer — block-manager allocations and frees, the batch queue, the
+  link's FIFOs and transfer ids — is atomic with respect to every other coroutine of the loop (a
+  scheduler coroutine allocating from the same block manager can never be handed the same ids);
+* the kernels are launched on the CALLER's current torch stream (torch's current stream is
+  per thread), so a transfer is stream-ordered with what the caller queued before and queues
+  after it on that stream: when ``migrate_requests`` returns and frees the source blocks, work the
+  caller then queues on the same stream cannot overtake the pack that read them. A caller that
+  works on other streams orders them itself (``stream.wait_stream``), as with any torch op.
+
+What a transfer costs the loop is launch time (microseconds); the device work itself is
+asynchronous except where a worker method synchronises as the reference's does (worker.py:684, :724).
 """
 from __future__ import annotations
 
-import asyncio
-import concurrent.futures
 import time
 from enum import Enum
 from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
@@ -55,21 +62,9 @@ class KVTransferManager:
         self.total_transfer_time = 0.0
         self.total_bytes_transferred = 0
         self.first_transfer_done = False
-        self._executor: Optional[concurrent.futures.ThreadPoolExecutor] = None
-
-    def _transfer_thread(self) -> concurrent.futures.ThreadPoolExecutor:
-        if self._executor is None:
-            self._executor = concurrent.futures.ThreadPoolExecutor(max_workers=1, thread_name_prefix="kv-transfer")
-        return self._executor
-
-    async def _off_loop(self, fn, *args):
-        """Run blocking transfer work on the manager's thread and await its result."""
-        return await asyncio.get_running_loop().run_in_executor(self._transfer_thread(), fn, *args)
 
     def close(self) -> None:
-        if self._executor is not None:
-            self._executor.shutdown(wait=True)
-            self._executor = None
+        """Nothing to release (kept for callers that close their managers)."""
 
     # ----- registry (kv_transfer.py:113-168) ---------------------------------
     def register_workers(self, stage: str, workers: Sequence[Any], global_ranks: Sequence[int]) -> None:
@@ -94,14 +89,12 @@ class KVTransferManager:
     # ----- transfer (kv_transfer.py:224-262) ----------------------------------
     async def transfer_kv_cache(self, request_id: str, src_rank: int, dst_rank: int, src_blocks: List[int],
                                 dst_blocks: List[int]) -> bool:
-        return await self._off_loop(self.transfer_kv_cache_sync, request_id, src_rank, dst_rank, src_blocks,
-                                    dst_blocks)
+        return self.transfer_kv_cache_sync(request_id, src_rank, dst_rank, src_blocks, dst_blocks)
 
     # ----- vision embeddings (kv_transfer.py:264-301, 've' branch of :724-728) ----
     async def transfer_vision_embeddings(self, request_id: str, src_rank: int, src_blocks: List[int],
                                          dst_rank: int, dst_blocks: List[int]) -> bool:
-        return await self._off_loop(self.transfer_vision_embeddings_sync, request_id, src_rank, src_blocks,
-                                    dst_rank, dst_blocks)
+        return self.transfer_vision_embeddings_sync(request_id, src_rank, src_blocks, dst_rank, dst_blocks)
 
     def transfer_vision_embeddings_sync(self, request_id: str, src_rank: int, src_blocks: List[int],
                                         dst_rank: int, dst_blocks: List[int]) -> bool:
@@ -247,8 +240,7 @@ class KVTransferManager:
     # ----- migration of whole requests (backend.py:674-737) -----------------------
     async def migrate_requests(self, request_ids: Sequence[str], src_rank: int, src_block_manager: Any,
                                dst_rank: int, dst_block_manager: Any) -> bool:
-        return await self._off_loop(self.migrate_requests_sync, request_ids, src_rank, src_block_manager,
-                                    dst_rank, dst_block_manager)
+        return self.migrate_requests_sync(request_ids, src_rank, src_block_manager, dst_rank, dst_block_manager)
 
     def migrate_requests_sync(self, request_ids: Sequence[str], src_rank: int, src_block_manager: Any,
                               dst_rank: int, dst_block_manager: Any) -> bool:
@@ -339,10 +331,13 @@ class KVTransferManager:
                 return False
             recv_result = dst_worker.p2p_recv_kv(src_rank, all_dst_blocks)
             if "error" in recv_result:
-                # the send went through: nothing of it may stay on the link for the next transfer
+                # the send went through: what is left of THIS transfer must not stay on the link for the next one
+                # (a receive that started has already dropped its remaining layers; one that never started has
+                # not). Other transfers between the two ranks, and pull requests, are not touched.
                 link = getattr(src_worker, "link", None)
-                if link is not None:
-                    link.drop_pending(src_rank, dst_rank)
+                sent = getattr(src_worker, "last_sent_transfer_id", None)
+                if link is not None and sent is not None:
+                    link.discard(src_rank, dst_rank, sent)
                 return False
             elapsed = time.perf_counter() - start_time
             nbytes = recv_result.get("bytes", 0)
@@ -381,25 +376,16 @@ class KVMigrationManager:
     """Cross-stage moves addressed by (stage, worker id) (kv_transfer.py:867-980, ``V0KVMigrationManager``):
     extract on the source worker, write on the destination worker, for KV blocks and for a request's vision
     embeddings. The reference's worker lookup is a placeholder that finds nobody (:961-969), so its moves always
-    report failure; here workers are registered under (stage, worker id). The coroutines run the blocking move on
-    the manager's own thread, like ``KVTransferManager``'s."""
+    report failure; here workers are registered under (stage, worker id). The coroutines run on the calling thread,
+    on the caller's current stream, like ``KVTransferManager``'s."""
 
     def __init__(self):
         self.migration_count = 0
         self.total_migration_time = 0.0
         self._workers_by_stage: Dict[Tuple[str, int], Any] = {}
-        self._executor: Optional[concurrent.futures.ThreadPoolExecutor] = None
-
-    async def _off_loop(self, fn, *args):
-        """Run a blocking move on this manager's own thread and await it (the event loop stays free)."""
-        if self._executor is None:
-            self._executor = concurrent.futures.ThreadPoolExecutor(max_workers=1, thread_name_prefix="kv-migration")
-        return await asyncio.get_running_loop().run_in_executor(self._executor, fn, *args)
 
     def close(self) -> None:
-        if self._executor is not None:
-            self._executor.shutdown(wait=True)
-            self._executor = None
+        """Nothing to release."""
 
     def register_worker(self, stage: str, worker_id: int, worker: Any) -> None:
         self._workers_by_stage[(stage.lower(), worker_id)] = worker
@@ -453,13 +439,12 @@ class KVMigrationManager:
 
     async def migrate_kv_blocks(self, request_id: str, src_stage: str, src_worker_id: int, src_blocks: List[int],
                                 dst_stage: str, dst_worker_id: int, dst_blocks: List[int]) -> bool:
-        return await self._off_loop(self.migrate_kv_blocks_sync, request_id, src_stage, src_worker_id, src_blocks,
-                                    dst_stage, dst_worker_id, dst_blocks)
+        return self.migrate_kv_blocks_sync(request_id, src_stage, src_worker_id, src_blocks, dst_stage,
+                                           dst_worker_id, dst_blocks)
 
     async def migrate_vision_embeddings(self, request_id: str, src_stage: str, src_worker_id: int, dst_stage: str,
                                         dst_worker_id: int) -> bool:
-        return await self._off_loop(self.migrate_vision_embeddings_sync, request_id, src_stage, src_worker_id,
-                                    dst_stage, dst_worker_id)
+        return self.migrate_vision_embeddings_sync(request_id, src_stage, src_worker_id, dst_stage, dst_worker_id)
 
     def get_stats(self) -> Dict[str, Any]:
         return {

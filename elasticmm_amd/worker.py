@@ -189,6 +189,10 @@ class KVWorker:
         self.swap_event_table: Dict[str, torch.cuda.Event] = {}
         self.latest_swap_in_event: Optional[torch.cuda.Event] = None
         self.latest_swap_out_event: Optional[torch.cuda.Event] = None
+        # device-resident block tables are trusted (ids out of range are skipped by the kernels); set this to have
+        # extract_kv_blocks / write_kv_blocks validate them first and raise IndexError (costs a synchronisation)
+        self.strict_device_tables = False
+        self.last_sent_transfer_id: Optional[int] = None
 
     # ----- pool -----------------------------------------------------------
     def init_kvcache(self, num_gpu_blocks: int, num_cpu_blocks: int = 0, *, num_layers: int, num_kv_heads: int,
@@ -243,7 +247,7 @@ class KVWorker:
         """-> ``[num_layers, 2, n, block_size, num_heads, head_size]``, one launch."""
         if self.kv_cache is None:
             raise RuntimeError("KV cache not initialized")
-        return kv_ops.kv_pack(self.pool, block_indices)
+        return kv_ops.kv_pack(self.pool, block_indices, strict=self.strict_device_tables)
 
     def write_kv_blocks(self, block_indices: List[int], kv_data: torch.Tensor) -> None:
         if self.kv_cache is None:
@@ -254,7 +258,7 @@ class KVWorker:
             kv_data = kv_data.to(self.pool.dtype)
         if kv_data.device != self.device:
             kv_data = kv_data.to(self.device)
-        kv_ops.kv_unpack(self.pool, block_indices, kv_data)
+        kv_ops.kv_unpack(self.pool, block_indices, kv_data, strict=self.strict_device_tables)
 
     def get_kv_cache_layout(self) -> Dict[str, Any]:
         if not self.kv_cache:
@@ -297,6 +301,9 @@ class KVWorker:
                 self.link.discard(self.global_rank, dst_rank, transfer_id)  # no half-sent transfer stays queued
                 raise
             torch.cuda.synchronize(self.device)
+            # the dict keeps the reference's shape; the id of the transfer just sent is left here so that a caller
+            # can drop exactly this transfer's messages from the link if the receiving side never takes them
+            self.last_sent_transfer_id = transfer_id
             return {"bytes": total_bytes, "blocks": len(block_indices)}
         except Exception as e:  # transport failures are reported, not raised (worker.py:686-691)
             error_msg = f"NCCL send failed: {type(e).__name__}: {str(e)}"

@@ -203,6 +203,119 @@ def test_device_indices_padding_and_out_of_range_are_skipped():
         assert same_bits(dst_g[l], dst_c[l])
 
 
+def test_strict_mode_catches_bad_device_ids_and_the_default_skips_them():
+    """A device-resident block table with ids outside the pool: by default the kernels skip those ids and touch
+    nothing else (neighbouring blocks keep their canary); with strict=True the caller gets IndexError before
+    anything is launched — on kv_pack, kv_unpack, kv_migrate, copy_blocks and through the worker's switch."""
+    L, NB, bs, H, D = 2, 24, 16, 2, 64
+    src_c = cpu_pool(L, NB, bs, H, D, torch.bfloat16, seed=3)
+    src = PoolView(to_dev(src_c))
+    good = torch.tensor([5, 0, 23, 7], device=DEV)
+    for bad_id in (-1, NB, 10 ** 9):
+        bad = torch.tensor([5, bad_id, 23, 7], device=DEV)
+        # default: skipped, the other rows are right
+        buf = kv_ops.kv_pack(src, bad)
+        want = orc.ref_extract_kv_blocks(src_c, [5, 0, 23, 7])
+        for j in (0, 2, 3):
+            assert same_bits(buf[:, :, j], want[:, :, j])
+        dst_c = cpu_pool(L, NB, bs, H, D, torch.bfloat16, seed=4, fill=7.0)
+        dst = PoolView(to_dev(dst_c))
+        kv_ops.kv_unpack(dst, bad, kv_ops.kv_pack(src, good))
+        for l in range(L):
+            for j, b in enumerate([5, 0, 23, 7]):
+                if j != 1:
+                    dst_c[l][:, b] = want[l][:, j]
+            assert same_bits(dst.layers[l], dst_c[l]), "a skipped id touched a neighbour"
+        # strict: IndexError, nothing written
+        for call in (lambda: kv_ops.kv_pack(src, bad, strict=True),
+                     lambda: kv_ops.kv_unpack(dst, bad, buf, strict=True),
+                     lambda: kv_ops.kv_migrate(src, bad, dst, good, strict=True),
+                     lambda: kv_ops.kv_migrate(src, good, dst, bad, strict=True),
+                     lambda: kv_ops.copy_blocks(dst, torch.stack([good, bad], 1).contiguous(), strict=True),
+                     lambda: cache_ops.copy_blocks(dst.layers, torch.stack([bad, good], 1).contiguous(), strict=True)):
+            with pytest.raises(IndexError, match="out of bounds"):
+                call()
+        torch.cuda.synchronize()
+        for l in range(L):
+            assert same_bits(dst.layers[l], dst_c[l]), "a strict call that raised wrote something"
+    # good tables pass in strict mode and give the same result
+    assert same_bits(kv_ops.kv_pack(src, good, strict=True), orc.ref_extract_kv_blocks(src_c, [5, 0, 23, 7]))
+    w = KVWorker(0, DEV, bs)
+    w.bind_kv_cache(src.layers)
+    w.strict_device_tables = True
+    with pytest.raises(IndexError):
+        w.extract_kv_blocks(torch.tensor([1, NB], device=DEV))
+    assert same_bits(w.extract_kv_blocks(good), orc.ref_extract_kv_blocks(src_c, [5, 0, 23, 7]))
+
+
+def test_two_host_threads_on_two_streams_at_once():
+    """The library is re-entrant: two host threads, each with its own stream and its own pair of pools, issue 200
+    rounds of pack / unpack / append at the same time (the pattern of the reference's side streams,
+    elasticmm/engine/v0/worker.py:496-516). Every round's transfer buffer and both final pools are compared with
+    the oracle replaying the same sequence; thread 0 also makes an invalid call now and then, and thread 1's
+    error string (per host thread) must stay empty throughout."""
+    import threading
+
+    lib = _lib.load()
+    L, NB, bs, H, D, rounds = 3, 96, 16, 2, 64, 200
+    results = {}
+
+    def work(tid):
+        try:
+            g = torch.Generator().manual_seed(100 + tid)
+            src_c = cpu_pool(L, NB, bs, H, D, torch.bfloat16, seed=50 + tid)
+            dst_c = cpu_pool(L, NB, bs, H, D, torch.bfloat16, seed=60 + tid, fill=float(tid + 1))
+            stream = torch.cuda.Stream()
+            bufs, errors = [], []
+            with torch.cuda.stream(stream):
+                src_g, dst_g = to_dev(src_c), to_dev(dst_c)
+                sp, dp = PoolView(src_g), PoolView(dst_g)
+                plan = []
+                for r in range(rounds):
+                    n = int(torch.randint(1, 9, (1,), generator=g))
+                    si = torch.randperm(NB, generator=g)[:n]
+                    di = torch.randperm(NB, generator=g)[:n]
+                    T = int(torch.randint(1, 40, (1,), generator=g))
+                    slots = torch.randperm(NB * bs, generator=g)[:T]
+                    slots[::7] = -1
+                    key = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+                    value = torch.randn((T, H, D), generator=g).to(torch.bfloat16)
+                    l = r % L
+                    plan.append((si, di, slots, key, value, l))
+                    # tables alternate between host lists and device tensors (both entry-point families)
+                    buf = kv_ops.kv_pack(sp, si.tolist() if r & 1 else si.to(DEV))
+                    kv_ops.kv_unpack(dp, di.to(DEV) if r & 1 else di.tolist(), buf)
+                    cache_ops.reshape_and_cache_flash(key.to(DEV), value.to(DEV), src_g[l][0], src_g[l][1],
+                                                      slots.to(DEV), "auto")
+                    bufs.append(buf)
+                    if tid == 0 and r % 50 == 0:
+                        assert lib.emm_kv_pack(None, -1, 2, NB, 64, None, 1, None, None) != 0
+                    errors.append(lib.emm_last_error())
+            stream.synchronize()
+            # the oracle replays the sequence
+            for r, (si, di, slots, key, value, l) in enumerate(plan):
+                want = orc.ref_extract_kv_blocks(src_c, si.tolist())
+                assert same_bits(bufs[r], want), f"thread {tid} round {r}: pack"
+                orc.ref_write_kv_blocks(dst_c, di.tolist(), want)
+                orc.c_reshape_and_cache(key, value, src_c[l][0], src_c[l][1], slots)
+            for l in range(L):
+                assert same_bits(src_g[l], src_c[l]) and same_bits(dst_g[l], dst_c[l]), f"thread {tid} layer {l}"
+            results[tid] = errors
+        except BaseException as e:  # noqa: BLE001 - reported by the main thread
+            results[tid] = e
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for tid in (0, 1):
+        if isinstance(results[tid], BaseException):
+            raise results[tid]
+    assert all(e == b"" for e in results[1]), "thread 1 saw an error string it did not cause"
+    assert any(b"num_layers" in e for e in results[0]), "thread 0's invalid calls left no message"
+
+
 def test_more_layers_than_one_argument_block():
     L = _lib.EMM_MAX_LAYERS + 5
     src_c = cpu_pool(L, 5, 1, 1, 8, torch.float16, 8)
@@ -2067,6 +2180,61 @@ def test_migrate_requests_between_two_workers():
         src_bm.allocate_blocks("huge", NB - 2)
         assert m.migrate_requests_sync(["huge"], 0, src_bm, 1, dst_bm) is False
         assert len(src_bm.get_block_table("huge")) == NB - 2 and dst_bm.get_block_table("huge") == []
+
+
+def test_migration_coroutine_is_ordered_with_the_callers_side_stream():
+    """A caller that works on a side stream: it fills the source blocks with a long kernel chain on that stream,
+    awaits ``migrate_requests`` inside ``torch.cuda.stream(side)``, and overwrites the (freed) source blocks on
+    the same stream right afterwards, never synchronising in between. The transfer is launched on the caller's
+    current stream, so the pack sees the filled blocks and the overwrite cannot overtake it — for the methods
+    that do not synchronise the device themselves (P2P_COPY, CUDA_IPC)."""
+    import asyncio
+
+    from elasticmm_amd.kv_transfer import KVMigrationManager, KVTransferManager, TransferMethod
+
+    for method in (TransferMethod.P2P_COPY, TransferMethod.CUDA_IPC):
+        src, dst = make_pair(L=6, NB=600, bs=16, H=4, D=128)
+        NB = src.pool.num_blocks
+        src_bm, dst_bm = BlockManager(NB), BlockManager(NB)
+        dst_bm.allocate_blocks("resident", 7)
+        for rid, n in (("a", 200), ("b", 150)):
+            src_bm.allocate_blocks(rid, n)
+        tables = {r: list(src_bm.get_block_table(r)) for r in ("a", "b")}
+        m = KVTransferManager(method)
+        m.register_workers("prefill", [src], [0])
+        m.register_workers("decoding", [dst], [1])
+        side = torch.cuda.Stream()
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            for t in src.kv_cache:            # queued on the side stream only; still running when the pack is queued
+                for _ in range(4):
+                    t.normal_()
+                t.mul_(0.5)
+            ok = asyncio.run(m.migrate_requests(["a", "b"], 0, src_bm, 1, dst_bm))
+            want = [t.clone() for t in src.kv_cache]     # what the pack must have seen
+            for t in src.kv_cache:            # the source blocks are free now: the caller reuses them at once
+                t.zero_()
+        side.synchronize()
+        assert ok is True
+        for r, si in tables.items():
+            di = dst_bm.get_block_table(r)
+            for l in range(len(want)):
+                assert torch.equal(dst.kv_cache[l][:, di], want[l][:, si]), f"{method}: request {r} layer {l}"
+        # the (stage, worker id) manager the same way
+        mm = KVMigrationManager()
+        mm.register_worker("prefill", 0, src)
+        mm.register_worker("decoding", 0, dst)
+        with torch.cuda.stream(side):
+            for t in src.kv_cache:
+                t.normal_()
+            ok = asyncio.run(mm.migrate_kv_blocks("x", "prefill", 0, [1, 2, 3], "decoding", 0, [9, 8, 7]))
+            want = [t.clone() for t in src.kv_cache]
+            for t in src.kv_cache:
+                t.zero_()
+        side.synchronize()
+        assert ok is True
+        for l in range(len(want)):
+            assert torch.equal(dst.kv_cache[l][:, [9, 8, 7]], want[l][:, [1, 2, 3]])
 
 
 def test_step_from_block_tables_to_both_cache_layouts():

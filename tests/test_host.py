@@ -491,45 +491,117 @@ def test_batched_migration_rollback_leaves_nothing_queued():
     assert tm.flush_all() is True and w0.calls == [("send", 1, [9])] and w1.calls == [("recv", 0, [3])]
 
 
-def test_transfer_coroutines_do_not_block_the_event_loop():
-    """The blocking part of a transfer (launches + the workers' device synchronisation) runs on the manager's
-    own thread: other coroutines of the loop keep running while it is in progress."""
+def test_concurrent_coroutines_keep_block_tables_disjoint_and_run_on_the_calling_thread():
+    """Two migrations and a scheduler that allocates from the same destination block manager, all in flight
+    on one event loop: a transfer has no await point inside, so its bookkeeping is atomic with respect to the
+    other coroutines — no block id is ever handed out twice — and it runs on the calling thread (where torch's
+    current stream is the caller's)."""
     import asyncio
     import threading
-    import time as _time
+
+    from elasticmm_amd.block_manager import BlockManager
 
     loop_thread = threading.get_ident()
-    seen = {}
+    threads = set()
 
-    class _SlowWorker(_FakeWorker):
+    class _W(_FakeWorker):
         def extract_kv_blocks(self, blocks):
-            seen["thread"] = threading.get_ident()
-            _time.sleep(0.25)                    # stands for a long device synchronisation
+            threads.add(threading.get_ident())
             return super().extract_kv_blocks(blocks)
 
     tm = KVTransferManager(TransferMethod.P2P_COPY)
-    tm.register_worker(0, _SlowWorker(0), "prefill")
-    tm.register_worker(1, _FakeWorker(1), "decoding")
-    ticks = []
+    tm.register_worker(0, _W(0), "prefill")
+    tm.register_worker(1, _W(1), "decoding")
+    src_bm, dst_bm = BlockManager(64), BlockManager(64)
+    for i in range(8):
+        src_bm.allocate_blocks(f"r{i}", 3)
+    taken = {}
 
-    async def ticker():
-        for _ in range(20):
-            ticks.append(_time.perf_counter())
-            await asyncio.sleep(0.01)
+    async def scheduler():
+        for i in range(10):
+            dst_bm.allocate_blocks(f"s{i}", 2)
+            taken[f"s{i}"] = list(dst_bm.get_block_table(f"s{i}"))
+            await asyncio.sleep(0)
 
     async def main():
-        t = asyncio.ensure_future(ticker())
-        t0 = _time.perf_counter()
-        ok = await tm.transfer_kv_cache("r", 0, 1, [1, 2], [3, 4])
-        t1 = _time.perf_counter()
-        await t
-        return ok, t0, t1
+        return await asyncio.gather(tm.migrate_requests([f"r{i}" for i in range(4)], 0, src_bm, 1, dst_bm), scheduler(),
+                                    tm.migrate_requests([f"r{i}" for i in range(4, 8)], 0, src_bm, 1, dst_bm))
 
-    ok, t0, t1 = asyncio.run(main())
-    assert ok is True and seen["thread"] != loop_thread
-    during = [x for x in ticks if t0 < x < t1]
-    assert len(during) >= 10, f"the loop ran only {len(during)} other steps during a 0.25 s transfer"
+    ok1, _, ok2 = asyncio.run(main())
+    assert ok1 is True and ok2 is True and threads == {loop_thread}
+    tables = [dst_bm.get_block_table(f"r{i}") for i in range(8)] + list(taken.values())
+    flat = [b for t in tables for b in t]
+    assert len(flat) == 8 * 3 + 10 * 2 and len(set(flat)) == len(flat), "a block id was handed out twice"
+    assert all(src_bm.get_block_table(f"r{i}") in (None, []) for i in range(8))   # the source blocks were freed
     tm.close()
+
+
+def test_two_managers_share_one_link_without_mixing_their_transfers():
+    """A KVTransferManager (NCCL method, batched) and a KVMigrationManager working over the same two workers and
+    the same link: the layers of one transfer are never interleaved with another's, and a failed receive drops
+    only its own transfer's messages."""
+    import asyncio
+
+    from elasticmm_amd.kv_transfer import KVMigrationManager
+    from elasticmm_amd.worker import LoopbackLink
+
+    link = LoopbackLink(2)
+
+    class _LinkWorker:
+        """The link protocol of KVWorker.p2p_send_kv / p2p_recv_kv (three layer messages per transfer) on plain lists."""
+        def __init__(self, rank):
+            self.rank, self.link, self.store, self.fail_recv = rank, link, {}, False
+
+        def p2p_send_kv(self, dst_rank, blocks):
+            tid = self.link.new_transfer_id()
+            for l in range(3):
+                self.link.send([(l, b, self.store.get(b)) for b in blocks], src=self.rank, dst=dst_rank, transfer_id=tid)
+            self.last_sent_transfer_id = tid
+            return {"bytes": 3 * len(blocks), "blocks": len(blocks)}
+
+        def p2p_recv_kv(self, src_rank, blocks):
+            if self.fail_recv:
+                return {"error": "refused", "bytes": 0, "blocks": 0}
+            tid = self.link.head_id(src_rank, self.rank)
+            for l in range(3):
+                got_tid, msg = self.link.recv_with_id(src_rank, self.rank)
+                assert got_tid == tid and [m[0] for m in msg] == [l] * len(blocks), "layers of two transfers interleaved"
+                for (_, _, val), b in zip(msg, blocks):
+                    self.store[b] = val
+            return {"bytes": 3 * len(blocks), "blocks": len(blocks)}
+
+        def extract_kv_blocks(self, blocks):
+            return [self.store[b] for b in blocks]
+
+        def write_kv_blocks(self, blocks, data):
+            self.store.update(zip(blocks, data))
+
+    a, b = _LinkWorker(0), _LinkWorker(1)
+    a.store = {i: f"v{i}" for i in range(10)}
+    tm = KVTransferManager(TransferMethod.NCCL, enable_batching=True, batch_size=2, batch_timeout=1e9)
+    tm.register_worker(0, a, "prefill")
+    tm.register_worker(1, b, "decoding")
+    mm = KVMigrationManager()
+    mm.register_worker("prefill", 0, a)
+    mm.register_worker("decoding", 0, b)
+
+    async def main():
+        return await asyncio.gather(tm.transfer_kv_cache("x", 0, 1, [0, 1], [20, 21]),
+                                    mm.migrate_kv_blocks("m", "prefill", 0, [2], "decoding", 0, [22]),
+                                    tm.transfer_kv_cache("y", 0, 1, [3], [23]),        # second of the batch: flushes
+                                    mm.migrate_kv_blocks("n", "prefill", 0, [4], "decoding", 0, [24]))
+
+    assert asyncio.run(main()) == [True, True, True, True]
+    assert {k: b.store[k] for k in (20, 21, 22, 23, 24)} == {20: "v0", 21: "v1", 22: "v2", 23: "v3", 24: "v4"}
+    assert link.pending(0, 1) == 0
+    # a receive that refuses: only that transfer's three messages leave the link; a transfer queued earlier by
+    # somebody else between the same ranks stays
+    other = link.new_transfer_id()
+    link.send(["somebody else's layer"], src=0, dst=1, transfer_id=other)
+    b.fail_recv = True
+    assert tm.transfer_kv_cache_sync("z", 0, 1, [5], [25]) is True                      # queued
+    assert tm.transfer_kv_cache_sync("w", 0, 1, [6], [26]) is False                     # flush: receive refused
+    assert link.pending(0, 1) == 1 and link.head_id(0, 1) == other
 
 
 def test_vision_transfer_through_the_manager_with_fake_workers():
