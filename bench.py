@@ -48,7 +48,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-ALL_SECTIONS = ["batched", "ceilings", "append", "paged", "lists", "modes", "cfg1", "fp8", "rebalance", "swap"]
+ALL_SECTIONS = ["batched", "ceilings", "append", "paged", "lists", "modes", "cfg1", "fp8", "rebalance", "swap", "variants"]
 
 
 def parse():
@@ -64,9 +64,12 @@ def parse():
                     help="comma-separated secondary measurements to run: " + ",".join(ALL_SECTIONS) + " (all | none)")
     ap.add_argument("--variant", type=lambda v: int(v, 0), default=0,
                     help="launch variant of the hooks build (tuning; routes every call through libemm_kv_hooks.so)")
-    ap.add_argument("--spread", type=int, default=4,
-                    help="stripes per pool of the headline: each pool's layers are allocated in this many pieces spread "
-                         "over the free device memory (0 or 1: one allocation per pool)")
+    ap.add_argument("--spread", type=int, default=0,
+                    help="stripes per pool of the headline: k > 1 allocates each pool's layers in k pieces spread over the "
+                         "free device memory (KVWorker.init_kvcache(spread_stripes=k)); 0 (default): the reference's own "
+                         "layout, one torch.empty per layer (what bind_kv_cache adopts from vLLM)")
+    ap.add_argument("--monolithic", action="store_true",
+                    help="with --spread 0: one allocation per pool (init_kvcache's default) instead of one per layer")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB copy with the same tile engine (a kernel of known traffic, "
                          "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -195,12 +198,37 @@ def release(*workers):
 
 
 # ---------------------------------------------------------------------------------------------- CPU baselines
+def host_cpu():
+    """Threads for the CPU legs and what the host is: every core this process may use — os.cpu_count(), capped by
+    OMP_NUM_THREADS where the environment sets it (a GPU box gives each job a share of its cores)."""
+    n = os.cpu_count() or 1
+    try:
+        n = min(n, len(os.sched_getaffinity(0)))
+    except (AttributeError, OSError):
+        pass
+    cap = os.environ.get("OMP_NUM_THREADS", "")
+    if cap.isdigit() and int(cap) > 0:
+        n = min(n, int(cap))
+    torch.set_num_threads(n)
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"cores": torch.get_num_threads(), "os_cpu_count": os.cpu_count(), "cpu_model": model}
+
+
 def cpu_baseline(tables, L, bs, H, D, dtype, budget_s=8.0):
     """The reference's torch path on the host cores: the same batch (same block counts per
     request) on pools reduced to just hold it — bytes moved depend on the blocks per request,
     not on the pool size. Passes repeat until about `budget_s` seconds of CPU work are done."""
     from oracle import kv_oracle as orc
 
+    host_cpu()  # sets the thread count before anything is timed
     nb = sum(len(s) for s, _ in tables)
     NBc = nb + 512
     torch.manual_seed(0)
@@ -229,7 +257,7 @@ def cpu_baseline(tables, L, bs, H, D, dtype, budget_s=8.0):
     return {
         "value": round(bytes_per_pass / med / 1e9, 3),
         "unit": "GB/s",
-        "cores": torch.get_num_threads(),
+        **host_cpu(),
         "kind": "port",
         "sample": f"the whole batch ({len(tabs)} requests, {nb} blocks, {bytes_per_pass / 1e9:.2f} GB algorithmic per "
                   f"pass) on host pools reduced to {NBc} blocks; the reference's torch indexing + stack / indexed "
@@ -242,6 +270,7 @@ def cpu_baseline_append(budget_s=5.0, L=28, bs=16, H=4, D=128, T=8448):
     layer, same T, same 5 % padded slots, pool reduced to 2048 blocks (bytes moved depend on T, not on the pool)."""
     from oracle import kv_oracle as orc
 
+    host_cpu()
     NBc = 2048
     g = torch.Generator().manual_seed(3)
     slots = torch.randperm(NBc * bs, generator=g)[:T].clone()
@@ -270,6 +299,7 @@ def cpu_baseline_cfg1(budget_s=2.0):
     """Config 1 exactly as specified, on the host."""
     from oracle import kv_oracle as orc
 
+    host_cpu()
     L, NB, bs, H, D = 4, 1024, 16, 8, 128
     g = torch.Generator().manual_seed(0)
     src = [torch.randn((2, NB, bs, H, D), generator=g).to(torch.float16) for _ in range(L)]
@@ -289,6 +319,15 @@ def cpu_baseline_cfg1(budget_s=2.0):
             "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"config 1 (4 layers x [2,1024,16,8,128] fp16, one request of 32 blocks), extract + write on "
                       f"CPU tensors; median of {len(times)} passes"}
+
+
+def layout_name(args):
+    if args.spread > 1:
+        return "pools allocated with init_kvcache(spread_stripes=%d)" % args.spread
+    if args.monolithic:
+        return "one allocation per pool (init_kvcache's default)"
+    return ("the reference's pool layout: one torch.empty per layer and pool, as vLLM's CacheEngine allocates and "
+            "bind_kv_cache adopts (elasticmm/engine/v0/worker.py:388-394)")
 
 
 # ---------------------------------------------------------------------------------------------- main
@@ -326,7 +365,10 @@ def main():
     payload = total_blocks * L * 2 * chunk       # bytes held by the batch's blocks
     bytes_per_step = 4 * payload                 # pack: read + write, unpack: read + write
 
-    src_w, dst_w = make_workers(NB, L, bs, H, D, dtype, dev, args.spread)
+    # The headline runs on the reference's own pool layout: one torch.empty per layer (the list bind_kv_cache adopts
+    # from vLLM's CacheEngine, elasticmm/engine/v0/worker.py:388-394). Other layouts: --spread / --monolithic, and
+    # extra.allocation_modes.
+    src_w, dst_w = make_workers(NB, L, bs, H, D, dtype, dev, args.spread, monolithic=args.monolithic)
     dev_tables = [(s.to(dev), d.to(dev)) for s, d in tables]
     torch.cuda.synchronize()
 
@@ -334,7 +376,7 @@ def main():
     # HBM bytes per launch from rocprofv3: FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 (factors from a plain 1 GiB
     # copy in the same profile run) came to TRAFFIC_RATIO x the algorithmic bytes for this kernel on this
     # workload (profiles/block_move_qwen2_7b_migrate_pmc.txt). A counter cannot be read inside this process;
-    # the figure below is that measured ratio applied to this run's bytes per launch.
+    # the figure below is that constant applied to this run's bytes per launch, not a reading of this run.
     TRAFFIC_RATIO = 1.0004
     roofline = {
         "bound": "hbm",
@@ -344,8 +386,10 @@ def main():
         "unit": "GB/s",
         "frac": round(m["kernel_GBps"] / HBM_PEAK_GBPS, 4),
         "traffic": int(m["avg_bytes_per_launch"] * TRAFFIC_RATIO),
-        "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by a plain copy of known size: "
-                          "%.4f x algorithmic (profiles/block_move_qwen2_7b_migrate_pmc.txt)" % TRAFFIC_RATIO,
+        "traffic_source": "a constant, not a counter read in this run: %.4f x this run's algorithmic bytes per launch. The "
+                          "ratio is rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch of this kernel on this workload, "
+                          "scaled by a plain copy of known size, as recorded in profiles/block_move_qwen2_7b_migrate_pmc.txt "
+                          "(regenerated whenever the kernel changes; the file states its command)" % TRAFFIC_RATIO,
         "launches": m["launches"],
         "avg_launch_us": round(m["avg_launch_us"], 2),
         "avg_bytes_per_launch": int(m["avg_bytes_per_launch"]),
@@ -378,6 +422,8 @@ def main():
         extra.update(batched(src_w, dst_w, dev_tables, payload, L, chunk, NB, dev))
     if "ceilings" in sections:
         extra["ceilings"] = ceilings(src_w, dst_w, dev_tables, payload, dev)
+    if "variants" in sections:
+        extra["pack_variants"] = pack_variants(src_w, dev_tables, payload, dev)
     if "append" in sections:
         extra["append"] = append_bench(src_w.kv_cache, NB, bs, H, D, None, None, dev)
     if "paged" in sections:
@@ -387,7 +433,7 @@ def main():
 
     if "modes" in sections:
         modes = {}
-        for name, spread, mono in (("one_allocation_per_pool", 0, True), ("one_allocation_per_layer", 0, False)):
+        for name, spread, mono in (("one_allocation_per_pool", 0, True), ("four_stripes_per_pool", 4, False)):
             sw, dw = make_workers(NB, L, bs, H, D, dtype, dev, spread, monolithic=mono)
             tabs = [(s.to(dev), d.to(dev)) for s, d in tables]
             mm = measure_migrate(sw, dw, tabs, max(3, args.steps // 4), 2, payload)
@@ -401,14 +447,14 @@ def main():
             release(sw, dw)
             del tabs
         modes["what"] = ("the headline workload on pools allocated differently: 'one_allocation_per_pool' is "
-                         "init_kvcache's default (spread_stripes=0), 'one_allocation_per_layer' is what a pool adopted "
-                         "from vLLM's CacheEngine through bind_kv_cache looks like (28 separate torch.empty); the "
-                         "headline itself uses %d stripes per pool" % args.spread)
+                         "init_kvcache's default (spread_stripes=0), 'four_stripes_per_pool' is init_kvcache("
+                         "spread_stripes=4): the layers in 4 pieces pushed apart in device memory with temporary spacer "
+                         "allocations. The headline itself runs on " + layout_name(args))
         extra["allocation_modes"] = modes
     if "cfg1" in sections:
         extra["cfg1_latency"] = cfg1_latency(dev)
     if "fp8" in sections:
-        extra["fp8_70b_shape"] = fp8_shape(dev, args.spread)
+        extra["fp8_70b_shape"] = fp8_shape(dev, args.spread, args.monolithic)
     if "rebalance" in sections:
         extra["rebalance_200GB"] = rebalance(dev)
     if "swap" in sections:
@@ -425,7 +471,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "u8",
+        "dtype": "bf16",
         "data": "synthetic",
         "pct_hbm_peak": round(100.0 * m["value"] / HBM_PEAK_GBPS, 2),
         "config": {
@@ -434,9 +480,7 @@ def main():
                         % (NB, len(tables), total_blocks, payload / 1e9),
             "num_layers": L, "num_blocks": NB, "block_size": bs, "kv_heads": H, "head_dim": D,
             "requests": len(tables), "blocks_moved": total_blocks, "algorithmic_bytes_per_step": bytes_per_step,
-            "pool_allocation": ("each pool allocated on its own, layers in %d stripes spread over the free device "
-                                "memory (extra.allocation_modes has the other layouts)" % args.spread)
-            if args.spread > 1 else "each pool one allocation",
+            "pool_allocation": layout_name(args) + " (extra.allocation_modes has the other layouts)",
         },
         "roofline": roofline,
         "extra": extra,
@@ -598,6 +642,44 @@ def pack_chain_probes(src_w, dev_tables, payload, dev):
     return out
 
 
+def pack_variants(src_w, dev_tables, payload, dev):
+    """The pack through the other kernel shapes kept in the hooks build (csrc/emm_kv_hooks.h: two / four tiles per
+    workgroup, loads straight into LDS, loader and storer waves), next to the product kernel: the whole batch in one
+    launch, and the 32 per-request launches."""
+    from elasticmm_amd import _lib, kv_ops
+
+    hooks = _lib.load_hooks()
+    sp = src_w.pool
+    all_si = torch.cat([s for s, _ in dev_tables]).contiguous()
+    n = all_si.numel()
+    buf = torch.empty(sp.packed_shape(n), dtype=sp.dtype, device=dev)
+    stab = _lib.ptr_table(sp.ptrs)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def variant(code, idx, out):
+        rc = hooks.emm_hook_pack_variant(code, stab, sp.num_layers, sp.num_kv, sp.num_blocks, sp.chunk_bytes,
+                                         idx.data_ptr(), idx.numel(), out.data_ptr(), stream)
+        if rc != 0:
+            raise RuntimeError(hooks.emm_last_error().decode())
+
+    bufs = [torch.empty(sp.packed_shape(s.numel()), dtype=sp.dtype, device=dev) for s, _ in dev_tables]
+    out = {}
+    med, _ = timed(lambda: kv_ops.kv_pack(sp, all_si, out=buf), 10)
+    med_r, _ = timed(lambda: [kv_ops.kv_pack(sp, s, out=b) for (s, _), b in zip(dev_tables, bufs)], 10)
+    out["product_kernel"] = {"whole_batch": rec(2 * payload, med, 1, "emm_block_move_kernel<pack>"),
+                             "per_request": rec(2 * payload, med_r, len(bufs), "emm_block_move_kernel<pack>")}
+    want = buf.clone()
+    for name, code in _lib.EMM_PACK_VARIANTS.items():
+        buf.zero_()
+        med, _ = timed(lambda: variant(code, all_si, buf), 10)
+        same = bool(torch.equal(buf, want))
+        med_r, _ = timed(lambda: [variant(code, s, b) for (s, _), b in zip(dev_tables, bufs)], 10)
+        out[name] = {"whole_batch": rec(2 * payload, med, 1, "emm_pack_variant_kernel<%d>" % code),
+                     "per_request": rec(2 * payload, med_r, len(bufs), "emm_pack_variant_kernel<%d>" % code),
+                     "same_result_as_product": same}
+    return out
+
+
 def paged_append_bench(kv, NB, bs, H, D, dev, T=8448, decode=256):
     """The same step appended into the paged-attention layout (key [NB,H,D/8,bs,8], value [NB,H,D,bs],
     viewed over the same pool memory): `decode` single tokens in random blocks, then one prompt of
@@ -742,6 +824,52 @@ def append_bench(kv, NB, bs, H, D, k_scales, v_scales, dev, T=8448):
     plan = cache_ops.layered_append(keys, values, kv, mode, k_scales, v_scales)
     med, _ = timed(lambda: plan(slots), 20)
     res["one_launch_all_layers"] = entry(med, 1)
+    # The per-layer launch where it really runs. (1) The same L launches as INDEPENDENT graph nodes: forked over k
+    # streams of the same priority inside the capture and joined at the end, so that nothing orders one layer's append
+    # after another's (what a runtime could do if the appends of several layers were ready at once). (2) Inside a
+    # forward: a kernel of the duration of a layer's other work between two appends (here the QKV projection that
+    # produces the K / V the append stores: [T, 3584] x [3584, 4608] bf16), L times, replayed from a graph with and
+    # without the appends; the difference per layer is what the forward pays for an append.
+    side_streams = [torch.cuda.Stream() for _ in range(3)]
+
+    def forked(k):
+        main = torch.cuda.current_stream()
+        for st in side_streams[:k - 1]:
+            st.wait_stream(main)
+        for l in range(L):
+            st = main if l % k == 0 else side_streams[l % k - 1]
+            with torch.cuda.stream(st):
+                cache_ops.reshape_and_cache_flash(keys[l], values[l], kv[l][0], kv[l][1], slots, mode, ks[l], vs[l])
+        for st in side_streams[:k - 1]:
+            main.wait_stream(st)
+
+    ctx = {}
+    for k in (2, 4):
+        med, _ = timed(graphed(lambda: forked(k)).replay, 20)
+        ctx["independent_graph_nodes_over_%d_streams" % k] = entry(med, L)
+    hidden, qkv = 3584, 3584 + 2 * H * D
+    xin = torch.randn((T, hidden), device=dev, generator=g).to(torch.bfloat16)
+    wqkv = (torch.randn((hidden, qkv), device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    yout = torch.empty((T, qkv), dtype=torch.bfloat16, device=dev)
+
+    def forward_like(with_append):
+        for l in range(L):
+            torch.mm(xin, wqkv, out=yout)
+            if with_append:
+                cache_ops.reshape_and_cache_flash(keys[l], values[l], kv[l][0], kv[l][1], slots, mode, ks[l], vs[l])
+
+    med_with, _ = timed(graphed(lambda: forward_like(True)).replay, 20)
+    med_without, _ = timed(graphed(lambda: forward_like(False)).replay, 20)
+    marginal_us = (med_with - med_without) * 1e3 / L
+    ctx["between_projection_kernels"] = {
+        "filler": "torch.mm [%d, %d] x [%d, %d] bf16 per layer" % (T, hidden, hidden, qkv),
+        "filler_us_per_layer": round(med_without * 1e3 / L, 2),
+        "with_append_us_per_layer": round(med_with * 1e3 / L, 2),
+        "append_marginal_us_per_layer": round(marginal_us, 2),
+        "append_marginal": rec(step_bytes, marginal_us * L * 1e-3, L, kernel, tokens_per_s=round(valid / (marginal_us * L * 1e-6))),
+    }
+    del xin, wqkv, yout
+    res["in_context"] = ctx
     # a decode step: 256 tokens, one per sequence, per-layer launches from a HIP graph (the most frequent step of a
     # serving loop; 1 MB per launch, so the figure of merit is microseconds per launch against the empty launch)
     Td = 256
@@ -783,27 +911,27 @@ def append_bench(kv, NB, bs, H, D, k_scales, v_scales, dev, T=8448):
     return res
 
 
-def cfg1_latency(dev):
-    """Config 1: 4 layers x [2,1024,16,8,128] fp16, one request of 32 blocks (8 MiB buffer). Latency of one
-    extract_kv_blocks + one write_kv_blocks; 32 disjoint block tables are cycled so that consecutive calls
-    touch different blocks (512 MiB of pools in total, twice the last-level cache)."""
+def latency_case(dev, L, NB, bs, H, D, dtype, n):
+    """Latency of one extract_kv_blocks + one write_kv_blocks for a request of `n` blocks: back to back in a chain
+    (the GPU never idles), and one isolated call with the device idle before and after (host launch + kernels +
+    completion). Disjoint block tables are cycled so that consecutive calls touch different blocks."""
     from elasticmm_amd.worker import KVWorker
 
-    L, NB, bs, H, D = 4, 1024, 16, 8, 128
     sw, dw = KVWorker(0, "cuda:0", bs), KVWorker(1, "cuda:0", bs)
     for w in (sw, dw):
-        w.init_kvcache(NB, num_layers=L, num_kv_heads=H, head_size=D, dtype=torch.float16)
+        w.init_kvcache(NB, num_layers=L, num_kv_heads=H, head_size=D, dtype=dtype, monolithic=False)
     for t in sw.kv_cache:
         t.normal_()
     g = torch.Generator().manual_seed(0)
     sp, dp = torch.randperm(NB, generator=g), torch.randperm(NB, generator=torch.Generator().manual_seed(1))
-    tabs = [(sp[i * 32:(i + 1) * 32].to(dev), dp[i * 32:(i + 1) * 32].to(dev)) for i in range(32)]
+    cycle = min(32, NB // n)
+    tabs = [(sp[i * n:(i + 1) * n].to(dev), dp[i * n:(i + 1) * n].to(dev)) for i in range(cycle)]
     lists = [(s.tolist(), d.tolist()) for s, d in tabs]
-    nbytes = 4 * 32 * L * 2 * bs * H * D * 2
+    nbytes = 4 * n * L * 2 * bs * H * D * torch.empty((), dtype=dtype).element_size()
     state = {"i": 0}
 
     def one(tables):
-        s, d = tables[state["i"] % 32]
+        s, d = tables[state["i"] % cycle]
         state["i"] += 1
         dw.write_kv_blocks(d, sw.extract_kv_blocks(s))
 
@@ -811,26 +939,53 @@ def cfg1_latency(dev):
         for _ in range(k):
             one(tables)
 
+    def isolated(tables):
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(50):
+            t0 = time.perf_counter()
+            one(tables)
+            torch.cuda.synchronize()
+            ts.append(time.perf_counter() - t0)
+        ts.sort()
+        return round(ts[len(ts) // 2] * 1e6, 1)
+
     med, _ = timed(lambda: many(tabs), 10)
     out = {"device_tables": rec(nbytes * 32, med, 64, "emm_block_move_kernel", us_per_pack_plus_unpack=round(med * 1e3 / 32, 2))}
     med, _ = timed(lambda: many(lists), 10)
     out["list_indices"] = rec(nbytes * 32, med, 64, "emm_block_move_kernel", us_per_pack_plus_unpack=round(med * 1e3 / 32, 2))
-    # one isolated call, device idle before and after (host launch + kernel + completion)
-    torch.cuda.synchronize()
-    ts = []
-    for _ in range(20):
-        t0 = time.perf_counter()
-        one(tabs)
-        torch.cuda.synchronize()
-        ts.append(time.perf_counter() - t0)
-    ts.sort()
-    out["isolated_call_wall_us"] = round(ts[len(ts) // 2] * 1e6, 1)
+    out["isolated_call_wall_us"] = isolated(tabs)
+    out["isolated_call_wall_us_list_indices"] = isolated(lists)
     out["bytes_per_pack_plus_unpack"] = nbytes
     release(sw, dw)
     return out
 
 
-def fp8_shape(dev, spread=4):
+def cfg1_latency(dev):
+    """Small requests: config 1 (4 layers x [2,1024,16,8,128] fp16, one request of 32 blocks, 8 MiB buffer) and the
+    reference's own typical transfer (15 blocks = 234 tokens, elasticmm/engine/v0/README.md:38-47) on the Qwen2-7B
+    layout (28 layers x [2,NB,16,4,128] bf16: 13.1 MiB per request). The floor under an isolated call is what two
+    kernels that do nothing cost the same way (launch, launch, synchronise)."""
+    from elasticmm_amd import _lib
+
+    out = latency_case(dev, 4, 1024, 16, 8, 128, torch.float16, 32)
+    out["typical_request_15_blocks_qwen2_7b_layout"] = latency_case(dev, 28, 2048, 16, 4, 128, torch.bfloat16, 15)
+    hooks = _lib.load_hooks()
+    stream = torch.cuda.current_stream().cuda_stream
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(50):
+        t0 = time.perf_counter()
+        hooks.emm_hook_empty_launch(stream)
+        hooks.emm_hook_empty_launch(stream)
+        torch.cuda.synchronize()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    out["two_empty_kernels_isolated_wall_us"] = round(ts[len(ts) // 2] * 1e6, 1)
+    return out
+
+
+def fp8_shape(dev, spread=0, monolithic=False):
     """Config 4: 80 layers x [2, NB, 16, 8, 128] e4m3, 64 requests of U{1024..8192} tokens: pack / unpack of fp8
     bytes, the quantising append (bf16 -> fp8), the dequantising unpack (fp8 -> bf16 pool)."""
     from elasticmm_amd import kv_ops
@@ -852,7 +1007,9 @@ def fp8_shape(dev, spread=4):
         shape = (2, NB, bs, H, D)
         if spread > 1:
             return allocate_layers_spread(L, shape, dtype, dev, spread)
-        return list(torch.empty((L,) + shape, dtype=dtype, device=dev).unbind(0))
+        if monolithic:
+            return list(torch.empty((L,) + shape, dtype=dtype, device=dev).unbind(0))
+        return [torch.empty(shape, dtype=dtype, device=dev) for _ in range(L)]  # the reference's layout
 
     src = make_pool(torch.uint8)
     dst = make_pool(torch.uint8)
@@ -873,6 +1030,8 @@ def fp8_shape(dev, spread=4):
         off += n
         del buf
     out = {"layers": L, "pool_blocks": NB, "requests": 64, "blocks": total, "payload_GB": round(payload / 1e9, 2),
+           "pool_allocation": "spread_stripes=%d" % spread if spread > 1 else "one allocation per pool" if monolithic
+           else "one torch.empty per layer",
            "pack": rec(2 * payload, ts_pack, 64, "emm_block_move_kernel<pack>"),
            "unpack": rec(2 * payload, ts_unpack, 64, "emm_block_move_kernel<unpack>"),
            "pack_plus_unpack": rec(4 * payload, ts_pack + ts_unpack, 128, "emm_block_move_kernel")}

@@ -57,12 +57,15 @@ SIGNATURES = {
 HOOK_SIGNATURES = {
     "emm_hook_set_move_variant": (c_int, [c_int]),
     "emm_hook_probe": (c_int, [c_int, _PP, c_int, c_int, c_int64, c_int64, _P, c_int64, _P, _P, _P]),
+    "emm_hook_pack_variant": (c_int, [c_int, _PP, c_int, c_int, c_int64, c_int64, _P, c_int64, _P, _P]),
     "emm_hook_empty_launch": (c_int, [_P]),
     "emm_hook_fp8_quotient_sweep": (c_int, [c_int, c_int, ctypes.c_uint32, ctypes.c_uint32, _P, _P]),
 }
 EMM_PROBE_SEQ_READ, EMM_PROBE_SEQ_WRITE, EMM_PROBE_GATHER_READ, EMM_PROBE_SCATTER_WRITE = 0, 1, 2, 3
 EMM_PROBE_GATHER_READ_COMPUTED_IDS, EMM_PROBE_PACK_COMPUTED_IDS, EMM_PROBE_PACK = 4, 5, 6
 EMM_PROBE_PACK_NOTHING_FETCHED = 7
+EMM_PACK_VARIANTS = {"two_tiles_per_workgroup": 1, "whole_chunk_per_workgroup": 2, "lds_dma_4KiB_one_wave": 3,
+                     "lds_dma_16KiB_four_waves": 4, "lds_dma_8KiB_one_wave": 5, "loader_storer_split": 6}
 
 _lib = None
 _hooks = None

@@ -2459,6 +2459,95 @@ __global__ __launch_bounds__(kThreads) void emm_probe_kernel(const int64_t *__re
   }
 }
 
+// Other shapes of the pack kernel, kept so that the choice of the product's shape (one 16-byte load and one 16-byte
+// store per lane, a 4 KiB tile per 256-thread workgroup) can be re-measured: same gather, same transfer buffer, same
+// store policy; grid (pieces per chunk, blocks, planes). The chunk must be a multiple of the variant's piece.
+//   U2         a workgroup moves two neighbouring tiles (8 KiB): both loads of a lane in flight before its first store
+//   CHUNK      a workgroup moves four tiles (16 KiB, a whole Qwen2-7B chunk): four loads in flight, then four stores
+//   LDS_1W     one-wave workgroups; the wave requests 4 x 1 KiB straight into LDS (global_load_lds_dwordx4: no data
+//              registers, the loads never follow a store of the same wave), waits once, reads the LDS and stores
+//   LDS_4W     the same with four waves per workgroup (16 KiB per workgroup)
+//   LDS_8K     one-wave workgroups, 8 x 1 KiB per wave in flight
+//   SPLIT      loader and storer waves: waves 0-1 only load (each 4 x 1 KiB per step, straight into LDS), waves 2-3
+//              only store what the loaders fetched in the previous step (double buffer, one block barrier per step;
+//              a workgroup walks kSplitSteps pieces of 8 KiB); a storer never waits for a load of its own and a
+//              loader never for a write acknowledgement
+constexpr int kSplitSteps = 8;
+template <int VAR>
+__global__ __launch_bounds__(VAR == EMM_PACK_VARIANT_LDS_1W || VAR == EMM_PACK_VARIANT_LDS_8K ? 64 : 256)
+void emm_pack_variant_kernel(const int64_t *__restrict__ idx, char *lin, int64_t lin_plane_stride, int64_t chunk,
+                             uint32_t nb, uint32_t n, const PlaneTables<1> tables) {
+  typedef __attribute__((address_space(3))) void lds_void;
+  const uint32_t pl = blockIdx.z, j = blockIdx.y, tid = threadIdx.x;
+  if constexpr (VAR == EMM_PACK_VARIANT_SPLIT) {
+    // grid x = groups of kSplitSteps pieces of 8 KiB along (block, offset in chunk) of this plane; y unused
+    __shared__ __attribute__((aligned(16))) char buf[2][8192];
+    const uint32_t wave = tid >> 6, lane = tid & 63;
+    const uint64_t pieces_per_chunk = (uint64_t)chunk / 8192;
+    const uint64_t first = (uint64_t)blockIdx.x * kSplitSteps, total = (uint64_t)n * pieces_per_chunk;
+    char *plane = tables.t[0].base[pl];
+    for (int step = 0; step <= kSplitSteps; ++step) {
+      const uint64_t p = first + step;
+      if (wave < 2) { // loaders: piece `p` into buffer step & 1
+        if (step < kSplitSteps && p < total) {
+          const uint64_t jb = p / pieces_per_chunk, part = p - jb * pieces_per_chunk;
+          const int64_t b = idx[jb];
+          if ((uint64_t)b < (uint64_t)nb) {
+            const char *src = plane + b * chunk + part * 8192 + wave * 4096 + lane * 16;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              __builtin_amdgcn_global_load_lds((const EMM_GLOBAL void *)(src + i * 1024),
+                                               (lds_void *)(buf[step & 1] + wave * 4096 + i * 1024), 16, 0, 0);
+          }
+          __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): the piece is in LDS before the barrier
+        }
+      } else if (step > 0 && p - 1 < total) { // storers: the piece of the previous step
+        const uint64_t q = p - 1, jb = q / pieces_per_chunk, part = q - jb * pieces_per_chunk;
+        if ((uint64_t)idx[jb] < (uint64_t)nb) {
+          char *dst = lin + (int64_t)pl * lin_plane_stride + (int64_t)jb * chunk + part * 8192 + (wave - 2) * 4096 + lane * 16;
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            st_stream<u32x4, 1>(dst + i * 1024,
+                                *reinterpret_cast<const u32x4 *>(buf[(step - 1) & 1] + (wave - 2) * 4096 + i * 1024 + lane * 16));
+        }
+      }
+      __syncthreads(); // every wave reaches every barrier: the loop bounds are the same for all
+    }
+    return;
+  } else {
+    int64_t b = idx[j];
+    char *plane = tables.t[0].base[pl];
+    asm volatile("" : "+s"(b), "+s"(plane) : : "memory");
+    if ((uint64_t)b >= (uint64_t)nb) return;
+    const char *src = plane + b * chunk;
+    char *dst = lin + (int64_t)pl * lin_plane_stride + (int64_t)j * chunk;
+    if constexpr (VAR == EMM_PACK_VARIANT_U2 || VAR == EMM_PACK_VARIANT_CHUNK) {
+      constexpr int U = VAR == EMM_PACK_VARIANT_U2 ? 2 : 4;
+      const int64_t off = (int64_t)blockIdx.x * (U * 4096) + tid * 16;
+      u32x4 v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = ld_stream<u32x4, 1>(src + off + u * 4096);
+#pragma unroll
+      for (int u = 0; u < U; ++u) st_stream<u32x4, 1>(dst + off + u * 4096, v[u]);
+    } else {
+      constexpr int K = VAR == EMM_PACK_VARIANT_LDS_8K ? 8 : 4;               // 1 KiB loads per wave
+      constexpr int W = VAR == EMM_PACK_VARIANT_LDS_4W ? 4 : 1;               // waves per workgroup
+      __shared__ __attribute__((aligned(16))) char tile[W * K * 1024];
+      const uint32_t wave = tid >> 6, lane = tid & 63;
+      const int64_t off = ((int64_t)blockIdx.x * W + wave) * (K * 1024) + lane * 16;
+#pragma unroll
+      for (int i = 0; i < K; ++i)
+        __builtin_amdgcn_global_load_lds((const EMM_GLOBAL void *)(src + off + i * 1024),
+                                         (lds_void *)(tile + (wave * K + i) * 1024), 16, 0, 0);
+      __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0)
+      __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+#pragma unroll
+      for (int i = 0; i < K; ++i)
+        st_stream<u32x4, 1>(dst + off + i * 1024, *reinterpret_cast<const u32x4 *>(tile + (wave * K + i) * 1024 + lane * 16));
+    }
+  }
+}
+
 // A kernel that does nothing: a chain of these measures what a dependent launch costs by itself.
 __global__ void emm_empty_kernel() {}
 
@@ -2559,6 +2648,45 @@ int emm_hook_probe(int kind, void *const *layer_ptrs, int num_layers, int num_kv
   case EMM_PROBE_PACK_NOTHING_FETCHED: emm_probe_kernel<EMM_PROBE_PACK_NOTHING_FETCHED><<<grid, kThreads, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, sink, t); break;
   default: return fail(EMM_EINVAL, "%s: unknown kind %d", what, kind);
   }
+  return check_launch(what);
+}
+
+int emm_hook_pack_variant(int variant, const void *const *layer_ptrs, int num_layers, int num_kv, int64_t num_blocks,
+                          int64_t chunk_bytes, const int64_t *block_idx, int64_t n, void *packed, emm_stream_t stream) {
+  const char *what = "emm_hook_pack_variant";
+  if (variant < EMM_PACK_VARIANT_U2 || variant > EMM_PACK_VARIANT_SPLIT) return fail(EMM_EINVAL, "%s: unknown variant %d", what, variant);
+  if (num_layers <= 0 || num_layers > EMM_MAX_LAYERS || num_kv <= 0 || n <= 0 || n > kMaxGridY || num_blocks <= 0 ||
+      num_blocks > 0x7fffffffLL || !layer_ptrs || !block_idx || !packed || !aligned(packed, 16))
+    return fail(EMM_EINVAL, "%s: bad geometry / null pointer", what);
+  const int64_t piece = variant == EMM_PACK_VARIANT_U2 || variant == EMM_PACK_VARIANT_LDS_8K || variant == EMM_PACK_VARIANT_SPLIT ? 8192
+                        : variant == EMM_PACK_VARIANT_LDS_1W ? 4096 : 16384;
+  if (chunk_bytes <= 0 || chunk_bytes % piece) return fail(EMM_EINVAL, "%s: chunk must be a multiple of %lld bytes", what, (long long)piece);
+  PlaneTables<1> t;
+  memset(&t, 0, sizeof(t));
+  const int planes = num_layers * num_kv;
+  for (int i = 0; i < planes; ++i) {
+    if (!layer_ptrs[i / num_kv] || !aligned(layer_ptrs[i / num_kv], 16)) return fail(EMM_EINVAL, "%s: bad layer pointer", what);
+    t.t[0].base[i] = (char *)layer_ptrs[i / num_kv] + (int64_t)(i % num_kv) * num_blocks * chunk_bytes;
+  }
+  hipStream_t s = as_stream(stream);
+  char *lin = (char *)packed;
+  const int64_t stride = n * chunk_bytes;
+  const dim3 grid((uint32_t)(chunk_bytes / piece), (uint32_t)n, (uint32_t)planes);
+#define EMM_PV(V_, T_) emm_pack_variant_kernel<V_><<<grid, T_, 0, s>>>(block_idx, lin, stride, chunk_bytes, (uint32_t)num_blocks, (uint32_t)n, t)
+  switch (variant) {
+  case EMM_PACK_VARIANT_U2: EMM_PV(EMM_PACK_VARIANT_U2, 256); break;
+  case EMM_PACK_VARIANT_CHUNK: EMM_PV(EMM_PACK_VARIANT_CHUNK, 256); break;
+  case EMM_PACK_VARIANT_LDS_1W: EMM_PV(EMM_PACK_VARIANT_LDS_1W, 64); break;
+  case EMM_PACK_VARIANT_LDS_4W: EMM_PV(EMM_PACK_VARIANT_LDS_4W, 256); break;
+  case EMM_PACK_VARIANT_LDS_8K: EMM_PV(EMM_PACK_VARIANT_LDS_8K, 64); break;
+  default: {
+    const int64_t pieces = n * (chunk_bytes / 8192);
+    const dim3 sgrid((uint32_t)((pieces + kSplitSteps - 1) / kSplitSteps), 1, (uint32_t)planes);
+    emm_pack_variant_kernel<EMM_PACK_VARIANT_SPLIT><<<sgrid, 256, 0, s>>>(block_idx, lin, stride, chunk_bytes,
+                                                                          (uint32_t)num_blocks, (uint32_t)n, t);
+  }
+  }
+#undef EMM_PV
   return check_launch(what);
 }
 

@@ -52,6 +52,22 @@ int emm_hook_probe(int kind, void *const *layer_ptrs, int num_layers, int num_kv
                    int64_t chunk_bytes, const int64_t *block_idx, int64_t n, void *linear, uint32_t *sink,
                    emm_stream_t stream);
 
+/* The pack (device table, whole call in one launch) through another kernel shape, so that the product's choice — one
+ * 16-byte load and one 16-byte store per lane, a 4 KiB tile per 256-thread workgroup — can be re-measured against:
+ * two tiles per workgroup with both loads in flight before the first store; four tiles (a whole 16 KiB chunk) per
+ * workgroup; loads straight into LDS (global_load_lds_dwordx4) with 4 KiB per one-wave workgroup, 4 x 4 KiB per
+ * four-wave workgroup, 8 KiB per one-wave workgroup; loader waves and storer waves split inside a workgroup
+ * (double-buffered LDS, one barrier per 8 KiB step). Same result as emm_kv_pack. n <= 65535; chunk_bytes a
+ * multiple of the variant's piece (8 KiB: U2, LDS_8K, SPLIT; 4 KiB: LDS_1W; 16 KiB: CHUNK, LDS_4W). */
+#define EMM_PACK_VARIANT_U2 1
+#define EMM_PACK_VARIANT_CHUNK 2
+#define EMM_PACK_VARIANT_LDS_1W 3
+#define EMM_PACK_VARIANT_LDS_4W 4
+#define EMM_PACK_VARIANT_LDS_8K 5
+#define EMM_PACK_VARIANT_SPLIT 6
+int emm_hook_pack_variant(int variant, const void *const *layer_ptrs, int num_layers, int num_kv, int64_t num_blocks,
+                          int64_t chunk_bytes, const int64_t *block_idx, int64_t n, void *packed, emm_stream_t stream);
+
 /* Launch a kernel that does nothing (one wave): a chain of these in a HIP graph measures the cost of a
  * dependent launch by itself, the floor under every per-layer launch. */
 int emm_hook_empty_launch(emm_stream_t stream);

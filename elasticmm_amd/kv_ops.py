@@ -156,6 +156,44 @@ class PoolView:
         return (self.num_layers, self.num_kv, n) + self.block_shape
 
 
+def _table_for_launch(block_indices: IndexLike, pool: PoolView, strict: bool, what: str):
+    """(n, pointer argument, host?, keep-alive) of a block table for the pack / unpack entry points.
+
+    This sits in front of every launch, and a request of a few dozen blocks is a few microseconds of kernel, so the
+    two usual cases are kept short: a contiguous int64 device tensor is passed as it is (trusted, or validated
+    when ``strict``), and a short Python list becomes a ctypes array directly (range check with min / max, negative
+    ids counted from the end, as torch's indexing does) without a detour through numpy. Everything else goes through
+    ``host_block_ids`` / ``block_index_tensor``. Host tables travel in the kernel argument block
+    (``*_host_ids`` entry points) unless the pool itself lives in host memory."""
+    nb = pool.num_blocks
+    if type(block_indices) is torch.Tensor and block_indices.is_cuda:
+        idx = block_indices
+        if idx.dtype != torch.long:
+            raise TypeError(f"block index tensor must be int64, got {idx.dtype}")
+        if not idx.is_contiguous():
+            idx = idx.contiguous()
+        if strict:
+            check_device_block_ids(idx, nb, what)
+        return idx.numel(), idx.data_ptr(), False, idx
+    if type(block_indices) is list and 0 < len(block_indices) <= 64 and not pool.on_host:
+        ids = block_indices
+        lo, hi = min(ids), max(ids)
+        if lo < -nb or hi >= nb:
+            raise IndexError(f"index {lo if lo < -nb else hi} is out of bounds for dimension 1 with size {nb}")
+        if lo < 0:
+            ids = [i + nb if i < 0 else i for i in ids]
+        try:
+            arr = (_lib.c_int64 * len(ids))(*ids)
+            return len(ids), arr, True, arr
+        except TypeError:  # not plain Python ints (numpy scalars, nested lists): the general path sorts it out
+            pass
+    host = host_block_ids(block_indices, nb)
+    if host is not None and not pool.on_host:
+        return host.size, host.ctypes.data, True, host
+    idx = block_index_tensor(host if host is not None else block_indices, nb, pool.device)
+    return idx.numel(), idx.data_ptr(), False, idx
+
+
 def kv_pack(pool: PoolView, block_indices: IndexLike, out: Optional[torch.Tensor] = None,
             strict: bool = False) -> torch.Tensor:
     """Gather ``n`` blocks of every layer into ``[L, num_kv, n, *block_shape]``.
@@ -165,32 +203,21 @@ def kv_pack(pool: PoolView, block_indices: IndexLike, out: Optional[torch.Tensor
     the allocation held. ``strict=True`` validates a device table first (``check_device_block_ids``: one
     reduction and a synchronisation) and raises ``IndexError`` instead."""
     lib = _lib.load()
-    if strict and isinstance(block_indices, torch.Tensor) and block_indices.is_cuda:
-        check_device_block_ids(block_indices, pool.num_blocks, "kv_pack")
-    # a table held on the host (the reference's List[int]) travels in the kernel argument block, EMM_MAX_INLINE_IDS
-    # ids per launch: no staging, no host-to-device copy
-    host = host_block_ids(block_indices, pool.num_blocks)
-    inline = host is not None and not pool.on_host
-    idx = None if inline else block_index_tensor(host if host is not None else block_indices, pool.num_blocks,
-                                                 pool.device)
-    n = host.size if inline else idx.numel()
-    shape = pool.packed_shape(n)
+    n, table_arg, inline, keep = _table_for_launch(block_indices, pool, strict, "kv_pack")
     if out is None:
-        out = torch.empty(shape, dtype=pool.dtype, device=pool.device)
-    else:
-        if out.device != pool.device or out.dtype != pool.dtype or not out.is_contiguous() \
-                or out.numel() != int(np.prod(shape, dtype=np.int64)):
-            raise ValueError("kv_pack: `out` must be a contiguous pool-dtype tensor of the packed size")
+        out = torch.empty((pool.num_layers, pool.num_kv, n) + pool.block_shape, dtype=pool.dtype, device=pool.device)
+    elif out.device != pool.device or out.dtype != pool.dtype or not out.is_contiguous() \
+            or out.numel() != pool.num_layers * pool.num_kv * n * pool.chunk_elems:
+        raise ValueError("kv_pack: `out` must be a contiguous pool-dtype tensor of the packed size")
     stream = _stream_ptr(pool.device)
     plane = pool.num_kv * n * pool.chunk_bytes
-    for l0, table in pool.layer_groups():
-        if inline:
-            check(lib.emm_kv_pack_host_ids(table, len(table), pool.num_kv, pool.num_blocks, pool.chunk_bytes,
-                                           host.ctypes.data, n, out.data_ptr() + l0 * plane, stream),
-                  "emm_kv_pack_host_ids")
-        else:
-            check(lib.emm_kv_pack(table, len(table), pool.num_kv, pool.num_blocks, pool.chunk_bytes,
-                                  idx.data_ptr(), n, out.data_ptr() + l0 * plane, stream), "emm_kv_pack")
+    fn = lib.emm_kv_pack_host_ids if inline else lib.emm_kv_pack
+    base = out.data_ptr()
+    for l0, table in pool._groups:
+        rc = fn(table, len(table), pool.num_kv, pool.num_blocks, pool.chunk_bytes, table_arg, n, base + l0 * plane, stream)
+        if rc:
+            check(rc, "emm_kv_pack_host_ids" if inline else "emm_kv_pack")
+    del keep
     return out
 
 
@@ -198,32 +225,26 @@ def kv_unpack(pool: PoolView, block_indices: IndexLike, packed: torch.Tensor, st
     """Scatter ``packed`` ``[L, num_kv, n, ...]`` into the pool under ``block_indices`` (``strict``: as in
     ``kv_pack``; without it a device table's out-of-range ids are skipped, their rows dropped)."""
     lib = _lib.load()
-    _require_gpu(packed, "kv_unpack")
-    if strict and isinstance(block_indices, torch.Tensor) and block_indices.is_cuda:
-        check_device_block_ids(block_indices, pool.num_blocks, "kv_unpack")
-    host = host_block_ids(block_indices, pool.num_blocks)
-    inline = host is not None and not pool.on_host
-    idx = None if inline else block_index_tensor(host if host is not None else block_indices, pool.num_blocks,
-                                                 pool.device)
-    n = host.size if inline else idx.numel()
-    want = pool.num_layers * pool.num_kv * n * pool.chunk_bytes
+    if not packed.is_cuda:
+        _require_gpu(packed, "kv_unpack")
+    n, table_arg, inline, keep = _table_for_launch(block_indices, pool, strict, "kv_unpack")
     if packed.device != pool.device:
         raise ValueError("kv_unpack: packed buffer is on another device")
-    if packed.numel() * packed.element_size() != want:
-        raise ValueError(f"kv_unpack: packed buffer holds {packed.numel() * packed.element_size()} bytes, "
-                         f"pool geometry needs {want}")
+    have = packed.numel() * packed.element_size()
+    if have != pool.num_layers * pool.num_kv * n * pool.chunk_bytes:
+        raise ValueError(f"kv_unpack: packed buffer holds {have} bytes, "
+                         f"pool geometry needs {pool.num_layers * pool.num_kv * n * pool.chunk_bytes}")
     if not packed.is_contiguous():
         packed = packed.contiguous()
     stream = _stream_ptr(pool.device)
     plane = pool.num_kv * n * pool.chunk_bytes
-    for l0, table in pool.layer_groups():
-        if inline:
-            check(lib.emm_kv_unpack_host_ids(table, len(table), pool.num_kv, pool.num_blocks, pool.chunk_bytes,
-                                             host.ctypes.data, n, packed.data_ptr() + l0 * plane, stream),
-                  "emm_kv_unpack_host_ids")
-        else:
-            check(lib.emm_kv_unpack(table, len(table), pool.num_kv, pool.num_blocks, pool.chunk_bytes,
-                                    idx.data_ptr(), n, packed.data_ptr() + l0 * plane, stream), "emm_kv_unpack")
+    fn = lib.emm_kv_unpack_host_ids if inline else lib.emm_kv_unpack
+    base = packed.data_ptr()
+    for l0, table in pool._groups:
+        rc = fn(table, len(table), pool.num_kv, pool.num_blocks, pool.chunk_bytes, table_arg, n, base + l0 * plane, stream)
+        if rc:
+            check(rc, "emm_kv_unpack_host_ids" if inline else "emm_kv_unpack")
+    del keep
 
 
 def kv_migrate(src: PoolView, src_indices: IndexLike, dst: PoolView, dst_indices: IndexLike,

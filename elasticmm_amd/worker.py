@@ -245,20 +245,22 @@ class KVWorker:
     # ----- extract / write (worker.py:578-647) ------------------------------
     def extract_kv_blocks(self, block_indices: List[int]) -> torch.Tensor:
         """-> ``[num_layers, 2, n, block_size, num_heads, head_size]``, one launch."""
-        if self.kv_cache is None:
+        pool = self._pool
+        if self.kv_cache is None or pool is None:
             raise RuntimeError("KV cache not initialized")
-        return kv_ops.kv_pack(self.pool, block_indices, strict=self.strict_device_tables)
+        return kv_ops.kv_pack(pool, block_indices, strict=self.strict_device_tables)
 
     def write_kv_blocks(self, block_indices: List[int], kv_data: torch.Tensor) -> None:
-        if self.kv_cache is None:
+        pool = self._pool
+        if self.kv_cache is None or pool is None:
             raise RuntimeError("KV cache not initialized")
         assert kv_data.shape[2] == len(block_indices), \
             f"Block count mismatch: {kv_data.shape[2]} vs {len(block_indices)}"
-        if kv_data.dtype != self.pool.dtype:
-            kv_data = kv_data.to(self.pool.dtype)
+        if kv_data.dtype != pool.dtype:
+            kv_data = kv_data.to(pool.dtype)
         if kv_data.device != self.device:
             kv_data = kv_data.to(self.device)
-        kv_ops.kv_unpack(self.pool, block_indices, kv_data, strict=self.strict_device_tables)
+        kv_ops.kv_unpack(pool, block_indices, kv_data, strict=self.strict_device_tables)
 
     def get_kv_cache_layout(self) -> Dict[str, Any]:
         if not self.kv_cache:

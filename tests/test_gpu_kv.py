@@ -316,6 +316,31 @@ def test_two_host_threads_on_two_streams_at_once():
     assert any(b"num_layers" in e for e in results[0]), "thread 0's invalid calls left no message"
 
 
+def test_pack_variants_of_the_hooks_build_give_the_pack():
+    """The alternative kernel shapes kept in the hooks build for re-measuring (two and four tiles per workgroup,
+    loads straight into LDS, loader / storer waves) must compute the same pack, skipped ids included."""
+    hooks = _lib.load_hooks()
+    for H, n in ((4, 37), (8, 130), (4, 1)):          # 16 KiB and 32 KiB chunks
+        L, NB, bs, D = 3, 200, 16, 128
+        pool_c = cpu_pool(L, NB, bs, H, D, torch.bfloat16, seed=H + n)
+        pool = PoolView(to_dev(pool_c))
+        g = torch.Generator().manual_seed(n)
+        ids = torch.randperm(NB, generator=g)[:n].clone()
+        if n > 4:
+            ids[3], ids[n - 2] = -1, NB + 5
+        ids_g = ids.to(DEV)
+        want = torch.full(pool.packed_shape(n), 7.0, dtype=torch.bfloat16, device=DEV)
+        kv_ops.kv_pack(pool, ids_g, out=want)
+        table = _lib.ptr_table(pool.ptrs)
+        for name, code in _lib.EMM_PACK_VARIANTS.items():
+            say(f"pack variant {name}: chunk {pool.chunk_bytes} bytes, {n} blocks")
+            got = torch.full(pool.packed_shape(n), 7.0, dtype=torch.bfloat16, device=DEV)
+            rc = hooks.emm_hook_pack_variant(code, table, L, 2, NB, pool.chunk_bytes, ids_g.data_ptr(), n, got.data_ptr(),
+                                             torch.cuda.current_stream().cuda_stream)
+            assert rc == 0, hooks.emm_last_error()
+            assert same_bits(got, want.cpu()), name
+
+
 def test_more_layers_than_one_argument_block():
     L = _lib.EMM_MAX_LAYERS + 5
     src_c = cpu_pool(L, 5, 1, 1, 8, torch.float16, 8)
