@@ -1697,8 +1697,9 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
 // The paged-attention append for the usual shapes (16-bit cache, sources that allow 16-byte loads, block size a
 // power of two >= 16): workgroups of ONE wave, no block barrier.
 //
-// A wave owns a tile of 16 token positions x COLS row elements of K or of V (grid: x = 2 * column + (K | V),
-// y = tile, z = layer; x runs fastest, so the waves of one tile are dispatched side by side).
+// A wave owns a tile of 16 token positions x COLS row elements of K and V (FUSED) or of one of them (grid: x = the
+// waves of a tile, then the layers of a whole-step launch, tiles slowest; x runs fastest, so the waves of one tile
+// are dispatched side by side).
 //
 // Who stores what. 16 consecutive tokens whose slots fill one 16-slot-aligned window of a block are a whole run;
 // the run belongs to the tile its first token lies in (it may reach 15 tokens into the next tile). Every other
@@ -1716,24 +1717,28 @@ __global__ __launch_bounds__(kThreads) void emm_append_paged_kernel(
 // transposed: K as 16-byte pieces, lane -> (group, token), every store instruction 1 KiB of contiguous cache;
 // V through the transposing LDS read ds_read_b64_tr_b16, lanes 0-31 the tokens 0-7 and lanes 32-63 the tokens
 // 8-15 of the same 32 elements, again 1 KiB of whole sectors per store instruction.
-// Other tokens: lane -> (token, piece) loads the row piece and the token's slot; K is stored from the registers
-// as 16-byte pieces; V passes through the LDS tile so that a store instruction writes 64 (COLS = 32: 2 x 32)
-// consecutive elements of a token — element-sized writes, each a partial sector: what this layout costs for a
-// token that does not fill a block.
-// COLS = 128 for long launches; 32 for launches of few tokens, which then spread over four times as many waves.
+// Other tokens: lane -> (token, piece) loads the row piece; K is stored from the registers as 16-byte pieces (the
+// token's slot comes from the lane that holds it, one ds_bpermute); V passes through the LDS tile so that a store
+// instruction writes 64 (COLS = 32: 2 x 32) consecutive elements of a token — element-sized writes, each a write
+// request of its own: what this layout costs for a token that does not fill a block.
+//
 // Measured on MI355X, Qwen2-7B rows, 28 layers (per-layer launches replayed from a HIP graph / one launch for all
-// layers; the flash-layout append on the same slots and memory beside it):
-//   8192-token prompt of whole runs   8.4-8.6 us per launch, 148 us (6.35 TB/s)     flash layout 7.0 us, 145 us
-//   256 single tokens                  4.8 us per launch, 39 us                      flash layout 2.2 us, 8 us
-//   256 single tokens + that prompt   12.6 us per launch, 251 us                     flash layout 7.2 us, 151 us
+// layers; the general kernel below and the flash-layout append on the same slots and memory beside it):
+//   8192-token prompt of whole runs   8.4 us per launch, 149 us (6.3 TB/s)   general 8.0, 152   flash layout 7.0, 146
+//   2048-token prompt of whole runs   3.7 us per launch                       general 4.1
+//   256 single tokens                  4.7 us per launch, 35-39 us             general 4.6, 41     flash layout 2.2, 8
+//   256 single tokens + the prompt    12.7-13.2 us per launch, 247-251 us     general 13.1-15.9, 246   flash 7.2, 151
 // Whole runs move at the speed of the flash-layout append; what is left is the single tokens: each of a token's 512 V
 // elements and 64 K pieces is a write request of its own, whatever kernel issues it (K alone: 2.2 us for the 256
 // tokens, the launch floor; V alone: 4.6). Tried on the single tokens' V stores and not kept: reading the word first so
 // that the line is valid in the L2 (256 tokens x 28 layers in one launch: 69 us against 43), merging with a pair of
-// 32-bit atomics (151 us), write-through stores (45 us). Whole rows per wave (COLS = 512, benchmark builds) bring the
-// per-layer launch of a prompt of whole runs to 7.1-7.3 us but leave a tile of 16 single tokens to two waves (a
-// decode step: 9.5 us per launch); the tile order (tiles slowest, layers inside) is worth 4 % on the one-launch form.
-template <int COLS, bool TABLES>
+// 32-bit atomics (151 us), write-through stores (45 us), and rewriting whole 32-byte sectors (read the element's 16
+// tokens, replace one, write back, 16 loads in flight per lane; only safe where no other token of the call shares the
+// 16-slot window): the mixed step in one launch 237 us against 251, but 31 us against 12.7 per layer and a decode step
+// 10 us against 4.8 — the cost is not that the writes are partial. The tile order (tiles slowest, layers inside) is
+// worth 4 % on the one-launch form. How many row elements a wave takes, and whether K and V share a wave, follows the
+// launch size (append_paged below).
+template <int COLS, bool FUSED, bool TABLES>
 __global__ __launch_bounds__(64) void emm_append_paged_wave_kernel(
     const int64_t *__restrict__ slot_mapping, const char *key, const char *value, char *key_cache,
     char *value_cache, uint32_t num_tokens, uint32_t row_elems, uint32_t key_stride, uint32_t value_stride,
@@ -1743,16 +1748,20 @@ __global__ __launch_bounds__(64) void emm_append_paged_wave_kernel(
   constexpr int NL = 16 / RPI;     // load instructions for 16 rows
   constexpr int ROW = COLS * 2 + 16; // LDS row stride in bytes
   static_assert(COLS == 512 || COLS == 256 || COLS == 128 || COLS == 32, "column width");
-  __shared__ __attribute__((aligned(16))) char tile[16 * ROW];
+  __shared__ __attribute__((aligned(16))) char tiles[FUSED ? 2 : 1][16 * ROW]; // FUSED: K, V
+  char *const ktile = tiles[0];
+  char *const vtile = tiles[FUSED ? 1 : 0];
   const uint32_t lane = threadIdx.x;
-  // grid: x = the 2 * columns waves of a tile, then the layers (TABLES), tiles slowest. Workgroups go to the 8 XCDs
-  // round-robin in dispatch order; rotating the (column, K | V) assignment by the tile index spreads the V waves of
-  // consecutive tiles over all XCDs (the single tokens of V are eight times the write requests of K).
+  // grid: x = the waves of a tile (FUSED: one per column, K and V both; else two per column, K | V in bit 0), then the
+  // layers (TABLES), tiles slowest. Workgroups go to the 8 XCDs round-robin in dispatch order; rotating the assignment
+  // by the tile index spreads the V waves of consecutive tiles over all XCDs (the single tokens of V are eight times
+  // the write requests of K).
   const uint32_t tile_idx = TABLES ? blockIdx.z : blockIdx.y;
   const uint32_t rot_mask = bs_log2 >> 8;
   bs_log2 &= 0xffu;
   const uint32_t xi = rot_mask ? (blockIdx.x + tile_idx) & rot_mask : blockIdx.x;
-  const uint32_t kv = xi & 1u, col = xi >> 1;
+  const uint32_t col = FUSED ? xi : xi >> 1;
+  const bool do_k = FUSED || (xi & 1u) == 0, do_v = FUSED || (xi & 1u) != 0;
   const uint32_t t0 = tile_idx * 16u;
 
   // ---- the 48 slots around the tile -> whole runs and single tokens (wave-uniform) ----
@@ -1768,24 +1777,22 @@ __global__ __launch_bounds__(64) void emm_append_paged_wave_kernel(
     key_cache = tables.key_cache[l];
     value_cache = tables.value_cache[l];
   }
-  const char *src = kv == 0 ? key : value;
-  char *cache = kv == 0 ? key_cache : value_cache;
-  const uint32_t stride = kv == 0 ? key_stride : value_stride;
   const uint32_t e0 = col * COLS;
   const uint32_t col_elems = row_elems - e0 < (uint32_t)COLS ? row_elems - e0 : (uint32_t)COLS; // multiple of 8
   const uint32_t piece = lane % PC, rsub = lane / PC;
   const bool live = piece * 8 < col_elems;
   const uint32_t bs_mask = (1u << bs_log2) - 1u;
   const uint64_t groups_per_block = row_elems >> 3;
-
+  const uint32_t col_off = (e0 + (live ? piece * 8 : 0)) * 2; // the lane's byte offset inside a source row
   // Short launches (COLS = 32: one load instruction covers the tile's 16 rows) request the tile's own rows before the
   // slots have arrived: they are what single tokens and a run that starts on the tile grid need, and a short launch
   // is one chain of memory round trips; a run that starts inside the tile loads its rows again.
   constexpr bool EARLY = NL == 1;
-  u32x4 early{0, 0, 0, 0};
+  u32x4 early_k{0, 0, 0, 0}, early_v{0, 0, 0, 0};
   if constexpr (EARLY) {
     const uint32_t tr = t0 + rsub <= (uint32_t)last ? t0 + rsub : (uint32_t)last;
-    early = ld<u32x4, true>(src + ((uint64_t)tr * stride + e0 + (live ? piece * 8 : 0)) * 2);
+    if (do_k) early_k = ld<u32x4, true>(key + (uint64_t)tr * key_stride * 2 + col_off);
+    if (do_v) early_v = ld<u32x4, true>(value + (uint64_t)tr * value_stride * 2 + col_off);
   }
   const uint32_t slo = (uint32_t)s, snlo = (uint32_t)sn;
   const uint32_t lo = t0 == 0 ? 16u : 0u;                                    // positions below 0
@@ -1809,42 +1816,58 @@ __global__ __launch_bounds__(64) void emm_append_paged_wave_kernel(
   if (w0 >= 0) lone &= (1u << w0) - 1u;
   if (w0 < 0 && lone == 0) return;
 
-  // ---- the whole run ----
+  // ---- the whole run: K and V rows -> LDS -> caches ----
   if (w0 >= 0) {
     const uint32_t sw = (uint32_t)__builtin_amdgcn_readlane((int)slo, 16 + w0);
     const uint64_t wblk = sw >> bs_log2;
     const uint32_t woff = sw & bs_mask;
-    const char *rows = src + ((uint64_t)(t0 + w0) * stride + e0 + (live ? piece * 8 : 0)) * 2;
-    u32x4 v[NL];
+    u32x4 vk[NL], vv[NL];
     if (EARLY && w0 == 0) {
-      v[0] = early;
+      vk[0] = early_k;
+      vv[0] = early_v;
     } else {
+      const char *krows = key + (uint64_t)(t0 + w0) * key_stride * 2 + col_off;
+      const char *vrows = value + (uint64_t)(t0 + w0) * value_stride * 2 + col_off;
+      if (do_k) {
 #pragma unroll
-      for (int k = 0; k < NL; ++k) v[k] = ld<u32x4, true>(rows + (uint64_t)(k * RPI + rsub) * stride * 2);
+        for (int k = 0; k < NL; ++k) vk[k] = ld<u32x4, true>(krows + (uint64_t)(k * RPI + rsub) * key_stride * 2);
+      }
+      if (do_v) {
+#pragma unroll
+        for (int k = 0; k < NL; ++k) vv[k] = ld<u32x4, true>(vrows + (uint64_t)(k * RPI + rsub) * value_stride * 2);
+      }
     }
+    if (live && do_k) {
 #pragma unroll
-    for (int k = 0; k < NL; ++k)
-      if (live) *reinterpret_cast<u32x4 *>(tile + (k * RPI + rsub) * ROW + piece * 16) = v[k];
+      for (int k = 0; k < NL; ++k) *reinterpret_cast<u32x4 *>(ktile + (k * RPI + rsub) * ROW + piece * 16) = vk[k];
+    }
+    if (live && do_v) {
+#pragma unroll
+      for (int k = 0; k < NL; ++k) *reinterpret_cast<u32x4 *>(vtile + (k * RPI + rsub) * ROW + piece * 16) = vv[k];
+    }
     __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront"); // the wave reads what its other lanes wrote
     __builtin_amdgcn_wave_barrier();
-    if (kv == 0) {
+    if (do_k) {
+      // K: lane -> (group 4 j + lane / 16, token lane % 16): a store instruction covers 1 KiB of contiguous cache
       const uint32_t r = lane & 15;
+      char *kdst = key_cache + (((wblk * groups_per_block + (e0 >> 3)) << bs_log2) + woff + r) * 16;
 #pragma unroll
       for (int j = 0; j < PC / 4; ++j) {
         const uint32_t g = 4 * j + (lane >> 4);
-        const u32x4 x = *reinterpret_cast<const u32x4 *>(tile + r * ROW + g * 16);
-        if (g * 8 < col_elems)
-          st_stream<u32x4, 1>(cache + (((wblk * groups_per_block + (e0 >> 3) + g) << bs_log2) + woff + r) * 16, x);
+        const u32x4 x = *reinterpret_cast<const u32x4 *>(ktile + r * ROW + g * 16);
+        if (g * 8 < col_elems) st_stream<u32x4, 1>(kdst + ((uint64_t)g << bs_log2) * 16, x);
       }
-    } else {
+    }
+    if (do_v) {
       typedef short v4i16 __attribute__((ext_vector_type(4)));
       typedef __attribute__((address_space(3))) v4i16 lds_v4i16;
       const uint32_t half = lane >> 5, grp = (lane >> 4) & 1, sub = lane & 15;
+      char *vdst = value_cache + (((wblk * row_elems + e0) << bs_log2) + woff) * 2 + half * 16;
 #pragma unroll
       for (int q0 = 0; q0 < COLS; q0 += 32) {
         // in every group of 16 lanes, lane 4 j + q points at elements c .. c + 3 of token j and lane l receives
         // element l of tokens 0 .. 3: two reads give a lane 8 tokens of its element
-        const char *from = tile + (8 * half + (sub >> 2)) * ROW + (q0 + 16 * grp + 4 * (sub & 3)) * 2;
+        const char *from = vtile + (8 * half + (sub >> 2)) * ROW + (q0 + 16 * grp + 4 * (sub & 3)) * 2;
         uint32_t w[4];
 #pragma unroll
         for (int m = 0; m < 2; ++m) {
@@ -1853,13 +1876,11 @@ __global__ __launch_bounds__(64) void emm_append_paged_wave_kernel(
           w[2 * m + 1] = (uint32_t)(uint16_t)t[2] | ((uint32_t)(uint16_t)t[3] << 16);
         }
         const uint32_t el = q0 + 16 * grp + sub;
-        if (el < col_elems)
-          st_stream<u32x4, 1>(cache + ((((wblk * row_elems + e0 + el) << bs_log2) + woff) * 2 + half * 16),
-                              u32x4{w[0], w[1], w[2], w[3]});
+        if (el < col_elems) st_stream<u32x4, 1>(vdst + ((uint64_t)el << bs_log2) * 2, u32x4{w[0], w[1], w[2], w[3]});
       }
     }
     if (lone == 0) return;
-    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront"); // the tile is reused below
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront"); // the V tile is reused below
     __builtin_amdgcn_wave_barrier();
   }
 
@@ -1868,31 +1889,35 @@ __global__ __launch_bounds__(64) void emm_append_paged_wave_kernel(
   // (all loads are issued together and unconditionally; only what is kept is predicated)
   const uint32_t first_lone = (uint32_t)__builtin_ctz(lone);
   bool mine[NL];
-  u32x4 x[NL];
-  const char *rows = src + ((uint64_t)t0 * stride + e0 + (live ? piece * 8 : 0)) * 2;
+  u32x4 xk[NL], xv[NL];
 #pragma unroll
   for (int k = 0; k < NL; ++k) {
     const uint32_t row = k * RPI + rsub;
     mine[k] = ((lone >> row) & 1u) && live;
-    if constexpr (EARLY)
-      x[k] = early;
-    else
-      x[k] = ld<u32x4, true>(rows + (uint64_t)(mine[k] ? row : first_lone) * stride * 2);
+    if constexpr (EARLY) {
+      xk[k] = early_k;
+      xv[k] = early_v;
+    } else {
+      const uint64_t tr = t0 + (mine[k] ? row : first_lone);
+      if (do_k) xk[k] = ld<u32x4, true>(key + tr * key_stride * 2 + col_off);
+      if (do_v) xv[k] = ld<u32x4, true>(value + tr * value_stride * 2 + col_off);
+    }
   }
-  if (kv == 0) {
-    uint32_t sl[NL]; // the slot of the lane's token: held by lane 16 + token
+  // K: 16-byte pieces straight from the registers; the slot of the lane's token is held by lane 16 + token
+  if (do_k) {
 #pragma unroll
-    for (int k = 0; k < NL; ++k) sl[k] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((16 + k * RPI + rsub) * 4), (int)slo);
-#pragma unroll
-    for (int k = 0; k < NL; ++k)
+    for (int k = 0; k < NL; ++k) {
+      const uint32_t sl = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((16 + k * RPI + rsub) * 4), (int)slo);
       if (mine[k])
-        st_stream<u32x4, 1>(cache + (((((uint64_t)(sl[k] >> bs_log2)) * groups_per_block + (e0 >> 3) + piece) << bs_log2) +
-                                     (sl[k] & bs_mask)) * 16, x[k]);
-    return;
+        st_stream<u32x4, 1>(key_cache + (((((uint64_t)(sl >> bs_log2)) * groups_per_block + (e0 >> 3) + piece) << bs_log2) +
+                                         (sl & bs_mask)) * 16, xk[k]);
+    }
   }
+  if (!do_v) return;
+  // V: through the LDS tile, one token at a time
 #pragma unroll
   for (int k = 0; k < NL; ++k)
-    if (mine[k]) *reinterpret_cast<u32x4 *>(tile + (k * RPI + rsub) * ROW + piece * 16) = x[k];
+    if (mine[k]) *reinterpret_cast<u32x4 *>(vtile + (k * RPI + rsub) * ROW + piece * 16) = xv[k];
   __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
   __builtin_amdgcn_wave_barrier();
   for (uint32_t m = lone; m;) { // at most 16 rounds
@@ -1900,11 +1925,11 @@ __global__ __launch_bounds__(64) void emm_append_paged_wave_kernel(
     m &= m - 1;
     if constexpr (COLS >= 64) {
       const uint64_t sl = (uint32_t)__builtin_amdgcn_readlane((int)slo, 16 + i0);
-      char *dst = cache + ((((sl >> bs_log2) * row_elems + e0) << bs_log2) + (sl & bs_mask)) * 2;
+      char *dst = value_cache + ((((sl >> bs_log2) * row_elems + e0) << bs_log2) + (sl & bs_mask)) * 2;
       // plain stores: neighbouring tokens of a partial run write neighbouring elements of the same sectors, which
       // the L2 merges before they go to memory
       for (uint32_t el = lane; el < col_elems; el += 64)
-        st<uint16_t, false>(dst + ((uint64_t)el << bs_log2) * 2, *reinterpret_cast<const uint16_t *>(tile + i0 * ROW + el * 2));
+        st<uint16_t, false>(dst + ((uint64_t)el << bs_log2) * 2, *reinterpret_cast<const uint16_t *>(vtile + i0 * ROW + el * 2));
     } else { // two tokens per store instruction
       int i1 = -1;
       if (m) {
@@ -1918,8 +1943,8 @@ __global__ __launch_bounds__(64) void emm_append_paged_wave_kernel(
       const uint64_t sl = upper ? s1 : s0;
       const uint32_t el = lane & (COLS - 1);
       if (i >= 0 && el < col_elems)
-        st<uint16_t, false>(cache + ((((sl >> bs_log2) * row_elems + e0 + el) << bs_log2) + (sl & bs_mask)) * 2,
-                            *reinterpret_cast<const uint16_t *>(tile + i * ROW + el * 2));
+        st<uint16_t, false>(value_cache + ((((sl >> bs_log2) * row_elems + e0 + el) << bs_log2) + (sl & bs_mask)) * 2,
+                            *reinterpret_cast<const uint16_t *>(vtile + i * ROW + el * 2));
     }
   }
 }
@@ -1987,43 +2012,61 @@ int append_paged(const void *const *k, const void *const *v, void *const *kc, vo
   }
   // The usual shapes take the kernel of one-wave workgroups: 16-bit cache, 16-byte loads from the sources, block size
   // a power of two from 16 on, all slots below 2^32 (run finding compares the low words). Benchmark builds can force
-  // the general kernel (bit 28) and either column width (bits 29-30: 1 = 128, 2 = 32).
+  // the general kernel (bit 28), the column width (bits 29-30: 1 = 128, 2 = 32, 3 = 256) and K and V in one wave or
+  // in two (bits 20-21: 1 / 2).
   const bool bs_pow2 = (block_size & (block_size - 1)) == 0;
   const int64_t wave_tiles = (num_tokens + 15) / 16;
   if (cache_elem_bytes == 2 && vec_src && bs_pow2 && block_size >= 16 && row_elems % 8 == 0 &&
       num_blocks * block_size <= 0xffffffffLL && wave_tiles <= kMaxGridY && !(move_variant() & 0x10000000)) {
-    // columns of 32 row elements while a launch of 128-element columns would leave most of the device idle (a decode
-    // step: 256 tokens of Qwen2-7B rows are 128 waves of 128-element columns, 512 of 32)
-    int cols = wave_tiles * 2 * ((row_elems + 127) / 128) * num_layers < 1024 ? 32 : 128;
-    if (((move_variant() >> 29) & 3) == 1) cols = 128;
-    if (((move_variant() >> 29) & 3) == 2) cols = 32;
-    if (((move_variant() >> 29) & 3) == 3) cols = (move_variant() & 0x100) ? 256 : 512; // benchmark builds only
+    // How fat a wave is follows the launch: a wave moves 16 tokens x `cols` row elements of K, of V, or of both
+    // (`fused`). Measured per layer on Qwen2-7B rows (512 elements), prompts of whole runs / off the tile grid / single
+    // tokens only / 256 single tokens + a prompt, 256 .. 16384 tokens: up to about a thousand tokens the narrow
+    // shape (32 elements, K and V in separate waves) wins wherever single tokens are involved (512 single tokens: 7.3 us
+    // against 9.1; 256 + a prompt of 768: 6.4 against 7.1) and loses little on pure prompts (3.3 against 3.0); beyond,
+    // 128 elements with K and V in one wave is the best or within 3 % of it everywhere (8192-token prompt 8.4 us,
+    // 2048: 3.7 where the general kernel takes 4.1). 256-element waves bring a long prompt of whole runs to the
+    // flash-layout append's 7.15 us but cost a step with single tokens 1.2 us; benchmark builds keep them.
+    const int64_t per128 = (row_elems + 127) / 128;
+    int cols = 128;
+    bool fused = true;
+    if (num_layers == 1 && wave_tiles * per128 < 256) {
+      cols = 32;
+      fused = false;
+    }
+    const int forced = (move_variant() >> 29) & 3; // benchmark builds: bits 29-30 the width, bits 20-21 K and V fused or not
+    if (forced == 1) cols = 128;
+    if (forced == 2) cols = 32;
+    if (forced == 3) cols = 256;
+    if (((move_variant() >> 20) & 3) == 1) fused = true;
+    if (((move_variant() >> 20) & 3) == 2) fused = false;
     const int64_t ncols = (row_elems + cols - 1) / cols;
-    if (ncols * 2 <= 0x7fffffffLL) {
-      const dim3 wgrid((uint32_t)(ncols * 2), tables ? (uint32_t)num_layers : (uint32_t)wave_tiles,
+    const int64_t nxw = fused ? ncols : 2 * ncols;
+    if (nxw <= 0x7fffffffLL) {
+      const dim3 wgrid((uint32_t)nxw, tables ? (uint32_t)num_layers : (uint32_t)wave_tiles,
                        tables ? (uint32_t)wave_tiles : 1u);
-      const uint32_t nx = (uint32_t)(ncols * 2);
+      const uint32_t nx = (uint32_t)nxw;
       const uint32_t rot_mask = (nx & (nx - 1)) == 0 && nx <= 0x800000u ? nx - 1 : 0u;
       const uint32_t bs_log2 = (uint32_t)__builtin_ctz((unsigned)block_size) | (rot_mask << 8);
       const uint64_t num_slots = (uint64_t)num_blocks * (uint64_t)block_size;
-#define EMM_PAGED_WAVE(COLS_) \
+#define EMM_PAGED_WAVE(COLS_, FUSED_) \
   do { \
     if (tables) \
-      emm_append_paged_wave_kernel<COLS_, true><<<wgrid, 64, 0, s>>>( \
+      emm_append_paged_wave_kernel<COLS_, FUSED_, true><<<wgrid, 64, 0, s>>>( \
           slot_mapping, nullptr, nullptr, nullptr, nullptr, (uint32_t)num_tokens, (uint32_t)row_elems, (uint32_t)ks, \
           (uint32_t)vs, bs_log2, num_slots, t); \
     else \
-      emm_append_paged_wave_kernel<COLS_, false><<<wgrid, 64, 0, s>>>( \
+      emm_append_paged_wave_kernel<COLS_, FUSED_, false><<<wgrid, 64, 0, s>>>( \
           slot_mapping, (const char *)k[0], (const char *)v[0], (char *)kc[0], (char *)vc[0], (uint32_t)num_tokens, \
           (uint32_t)row_elems, (uint32_t)ks, (uint32_t)vs, bs_log2, num_slots, NoTables{}); \
   } while (0)
 #ifdef EMM_BENCH_HOOKS
-      if (cols == 512) EMM_PAGED_WAVE(512); // whole rows per wave: measured for the record, see the kernel's comment
-      else if (cols == 256) EMM_PAGED_WAVE(256);
+      if (cols == 256) { if (fused) EMM_PAGED_WAVE(256, true); else EMM_PAGED_WAVE(256, false); }
+      else if (cols == 128 && !fused) EMM_PAGED_WAVE(128, false);
+      else if (cols == 32 && fused) EMM_PAGED_WAVE(32, true);
       else
 #endif
-      if (cols == 128) EMM_PAGED_WAVE(128);
-      else EMM_PAGED_WAVE(32);
+      if (cols == 128) EMM_PAGED_WAVE(128, true);
+      else EMM_PAGED_WAVE(32, false);
 #undef EMM_PAGED_WAVE
       return check_launch(what);
     }

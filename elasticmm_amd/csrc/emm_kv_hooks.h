@@ -29,7 +29,8 @@ extern "C" {
  *   per XCD (default: chosen per launch by kind, table length, tiles per chunk and plane size);
  * bit 28: the paged-layout append always through the general kernel (256-thread workgroups, block barrier) instead of
  *   the kernel of one-wave workgroups that the usual shapes take;
- * bits 29-30: column width of the one-wave paged-layout append (1 = 128 row elements, 2 = 32; 0 = by launch size).
+ * bits 29-30: column width of the one-wave paged-layout append (1 = 128 row elements, 2 = 32, 3 = 256; 0 = by launch
+ *   size); with it bits 20-21: 1 = K and V of a column in one wave, 2 = in two waves (0 = by launch size).
  * Process-wide, not thread-safe. Returns the previous value. */
 int emm_hook_set_move_variant(int variant);
 

@@ -1064,14 +1064,18 @@ def test_paged_append_both_tile_widths(width, monkeypatch):
         hooks.emm_hook_set_move_variant(old)
 
 
-@pytest.mark.parametrize("cols", [1, 2], ids=["columns of 128 row elements", "columns of 32 row elements"])
-def test_paged_append_one_wave_kernel_both_column_widths(cols, monkeypatch):
+@pytest.mark.parametrize("cols,fused", [(1, 1), (1, 2), (2, 1), (2, 2), (3, 1), (3, 2)],
+                         ids=["128 row elements, K and V in one wave", "128 row elements, K and V in two waves",
+                              "32 row elements, one wave", "32 row elements, two waves",
+                              "256 row elements, one wave", "256 row elements, two waves"])
+def test_paged_append_one_wave_kernel_every_wave_shape(cols, fused, monkeypatch):
     """16-bit caches with aligned sources and a power-of-two block size from 16 on take the kernel of one-wave
-    workgroups, which picks its column width by launch size; here each width is forced on launches of either size:
-    rows that end inside a column, strided sources, prompts on and off the token-tile grid, block size 32 and 64."""
+    workgroups, which picks how many row elements a wave takes, and whether K and V share a wave, by launch size;
+    here each shape is forced on launches of either size: rows that end inside a column, strided sources, prompts
+    on and off the token-tile grid, block size 32 and 64."""
     hooks = _lib.load_hooks()
     monkeypatch.setattr(_lib, "_lib", hooks)
-    old = hooks.emm_hook_set_move_variant(cols << 29)
+    old = hooks.emm_hook_set_move_variant((cols << 29) | (fused << 20))
     try:
         for (dtype, NB, bs, H, D, T, phase, pad) in [
                 (torch.bfloat16, 700, 16, 4, 128, 5000, 3, 0), (torch.float16, 300, 16, 8, 128, 2500, 0, 0),
@@ -1079,7 +1083,8 @@ def test_paged_append_one_wave_kernel_both_column_widths(cols, monkeypatch):
                 (torch.float16, 80, 16, 3, 40, 300, 4, 8), (torch.bfloat16, 48, 32, 2, 64, 700, 1, 8),
                 (torch.bfloat16, 60, 64, 1, 72, 900, 15, 0), (torch.bfloat16, 30, 16, 20, 128, 100, 1, 0),
                 (torch.float16, 40, 16, 1, 8, 333, 0, 0)]:
-            say(f"paged append, one-wave kernel, column code {cols}: {dtype} NB={NB} bs={bs} H={H} D={D} T={T} pad={pad}")
+            say(f"paged append, one-wave kernel, column code {cols}, fused code {fused}: {dtype} NB={NB} bs={bs} H={H} D={D} "
+                f"T={T} pad={pad}")
             g = torch.Generator().manual_seed(NB * 7 + T + cols)
             slots = paged_slots(NB, bs, T, seed=T + 1, phase=phase)
             assert len(slots) == T
