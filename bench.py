@@ -48,7 +48,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-ALL_SECTIONS = ["batched", "ceilings", "append", "paged", "lists", "modes", "cfg1", "fp8", "rebalance", "swap", "variants"]
+ALL_SECTIONS = ["batched", "ceilings", "append", "paged", "lists", "modes", "cfg1", "fp8", "rebalance", "swap", "variants", "placement"]
 
 
 def parse():
@@ -70,6 +70,9 @@ def parse():
                          "layout, one torch.empty per layer (what bind_kv_cache adopts from vLLM)")
     ap.add_argument("--monolithic", action="store_true",
                     help="with --spread 0: one allocation per pool (init_kvcache's default) instead of one per layer")
+    ap.add_argument("--no-append-context", action="store_true",
+                    help="skip extra.append.in_context (HIP graphs that fork over several streams or contain library GEMMs; "
+                         "rocprofv3 --pmc has crashed replaying them)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB copy with the same tile engine (a kernel of known traffic, "
                          "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -352,6 +355,8 @@ def main():
 
     from elasticmm_amd import _lib, kv_ops
 
+    global APPEND_CONTEXT
+    APPEND_CONTEXT = not args.no_append_context
     if args.variant:
         # launch variants exist only in the hooks build of the library: route this process through it
         _lib.use_hooks_build().emm_hook_set_move_variant(args.variant)
@@ -377,7 +382,7 @@ def main():
     # copy in the same profile run) came to TRAFFIC_RATIO x the algorithmic bytes for this kernel on this
     # workload (profiles/block_move_qwen2_7b_migrate_pmc.txt). A counter cannot be read inside this process;
     # the figure below is that constant applied to this run's bytes per launch, not a reading of this run.
-    TRAFFIC_RATIO = 1.0004
+    TRAFFIC_RATIO = 1.0005
     roofline = {
         "bound": "hbm",
         "kernel": "emm_block_move_kernel (pack + unpack instances)",
@@ -428,6 +433,8 @@ def main():
         extra["append"] = append_bench(src_w.kv_cache, NB, bs, H, D, None, None, dev)
     if "paged" in sections:
         extra["append_paged_layout"] = paged_append_bench(src_w.kv_cache, NB, bs, H, D, dev)
+    if "placement" in sections:
+        extra["placement"] = placement(src_w, dst_w, dev_tables, payload, dev)
     release(src_w, dst_w)
     dev_tables = None
 
@@ -642,6 +649,47 @@ def pack_chain_probes(src_w, dev_tables, payload, dev):
     return out
 
 
+def placement(src_w, dst_w, dev_tables, payload, dev):
+    """Where an allocation lands in device memory decides how fast scattered writes into it are, and that differs from
+    process to process for the same program (same virtual addresses): the batch's per-request unpacks into the
+    destination pool and, from the same buffers, into the source pool of this process; and a scatter-write / gather-read
+    probe (hooks build) of the batch's chunks into every layer — every allocation — of both pools by itself."""
+    from elasticmm_amd import _lib, kv_ops
+
+    hooks = _lib.load_hooks()
+    sp, dp = src_w.pool, dst_w.pool
+    bufs = [kv_ops.kv_pack(sp, s) for s, _ in dev_tables]
+    out = {}
+    for name, pool in (("unpack_into_destination_pool", dp), ("unpack_into_source_pool", sp)):
+        med, _ = timed(lambda: [kv_ops.kv_unpack(pool, d, b) for (_, d), b in zip(dev_tables, bufs)], 10)
+        out[name] = rec(2 * payload, med, len(bufs), "emm_block_move_kernel<unpack>")
+    del bufs
+    all_di = torch.cat([d for _, d in dev_tables]).contiguous()
+    n = all_di.numel()
+    lin = torch.empty(sp.num_kv * n * sp.chunk_bytes, dtype=torch.uint8, device=dev)
+    sink = torch.zeros(1024, dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    layer_bytes = sp.num_kv * n * sp.chunk_bytes
+    for pname, pool in (("destination_pool", dp), ("source_pool", sp)):
+        for kname, kind in (("scatter_write", _lib.EMM_PROBE_SCATTER_WRITE), ("gather_read", _lib.EMM_PROBE_GATHER_READ)):
+            rates = []
+            for l in range(pool.num_layers):
+                tab = _lib.ptr_table(pool.ptrs[l:l + 1])
+
+                def probe():
+                    rc = hooks.emm_hook_probe(kind, tab, 1, pool.num_kv, pool.num_blocks, pool.chunk_bytes, all_di.data_ptr(),
+                                              n, lin.data_ptr(), sink.data_ptr(), stream)
+                    if rc != 0:
+                        raise RuntimeError(hooks.emm_last_error().decode())
+
+                med, _ = timed(probe, 5, warmup=1)
+                rates.append(round(layer_bytes / med / 1e6))
+            out["%s_%s_GBps_per_layer" % (pname, kname)] = rates
+    out["note"] = ("each layer is an allocation of its own; the probes touch the batch's %d chunks of 16 KiB in both planes of "
+                   "one layer per launch (%.0f MB)" % (n, layer_bytes / 1e6))
+    return out
+
+
 def pack_variants(src_w, dev_tables, payload, dev):
     """The pack through the other kernel shapes kept in the hooks build (csrc/emm_kv_hooks.h: two / four tiles per
     workgroup, loads straight into LDS, loader and storer waves), next to the product kernel: the whole batch in one
@@ -772,6 +820,9 @@ def paged_append_bench(kv, NB, bs, H, D, dev, T=8448, decode=256):
     return res
 
 
+APPEND_CONTEXT = True  # main() clears it for --no-append-context
+
+
 def append_bench(kv, NB, bs, H, D, k_scales, v_scales, dev, T=8448):
     """reshape_and_cache for one step: 256 decode tokens + one 8192-token prefill chunk, slots random
     over the pool, 5 % padded (-1). Three ways of issuing it: the vLLM-shaped call once per layer
@@ -830,6 +881,19 @@ def append_bench(kv, NB, bs, H, D, k_scales, v_scales, dev, T=8448):
     # forward: a kernel of the duration of a layer's other work between two appends (here the QKV projection that
     # produces the K / V the append stores: [T, 3584] x [3584, 4608] bf16), L times, replayed from a graph with and
     # without the appends; the difference per layer is what the forward pays for an append.
+    if APPEND_CONTEXT:
+        res["in_context"] = append_in_context(keys, values, kv, slots, mode, ks, vs, entry, graphed, step_bytes, valid,
+                                              kernel, T, H, D, L, dev, g)
+    # a decode step: 256 tokens, one per sequence, per-layer launches from a HIP graph (the most frequent step of a
+    # serving loop; 1 MB per launch, so the figure of merit is microseconds per launch against the empty launch)
+    Td = 256
+    dslots = slots[slots >= 0][:Td].contiguous()
+    return _append_bench_tail(res, keys, values, kv, slots, dslots, Td, mode, ks, vs, graphed, kernel, row, step_bytes, L, dev)
+
+
+def append_in_context(keys, values, kv, slots, mode, ks, vs, entry, graphed, step_bytes, valid, kernel, T, H, D, L, dev, g):
+    from elasticmm_amd import cache_ops
+
     side_streams = [torch.cuda.Stream() for _ in range(3)]
 
     def forked(k):
@@ -869,11 +933,11 @@ def append_bench(kv, NB, bs, H, D, k_scales, v_scales, dev, T=8448):
         "append_marginal": rec(step_bytes, marginal_us * L * 1e-3, L, kernel, tokens_per_s=round(valid / (marginal_us * L * 1e-6))),
     }
     del xin, wqkv, yout
-    res["in_context"] = ctx
-    # a decode step: 256 tokens, one per sequence, per-layer launches from a HIP graph (the most frequent step of a
-    # serving loop; 1 MB per launch, so the figure of merit is microseconds per launch against the empty launch)
-    Td = 256
-    dslots = slots[slots >= 0][:Td].contiguous()
+    return ctx
+
+
+def _append_bench_tail(res, keys, values, kv, slots, dslots, Td, mode, ks, vs, graphed, kernel, row, step_bytes, L, dev):
+    from elasticmm_amd import cache_ops, kv_ops
 
     def decode_per_layer():
         for l in range(L):
