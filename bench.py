@@ -728,15 +728,20 @@ def pack_variants(src_w, dev_tables, payload, dev):
     return out
 
 
-def paged_append_bench(kv, NB, bs, H, D, dev, T=8448, decode=256):
-    """The same step appended into the paged-attention layout (key [NB,H,D/8,bs,8], value [NB,H,D,bs],
-    viewed over the same pool memory): `decode` single tokens in random blocks, then one prompt of
-    T - decode tokens that fills blocks in order (its blocks start off the 16-token grid of the token
-    list). Bytes: 2 x 2 x row per token, as for the flash layout."""
+def paged_append_bench(kv, NB, bs, H, D, dev, T=8448, decode=256, k_scales=None, v_scales=None):
+    """The same step appended into the paged-attention layout (key [NB,H,D/x,bs,x], value [NB,H,D,bs],
+    x = 16 bytes of cache elements, viewed over the same pool memory): `decode` single tokens in random
+    blocks, then one prompt of T - decode tokens that fills blocks in order (its blocks start off the
+    16-token grid of the token list). Bytes per token and layer: the K and V rows read (16-bit) and written
+    (the cache's element size), as for the flash layout. With scales the cache is fp8 (quantising append)."""
     from elasticmm_amd import cache_ops
 
     L = len(kv)
-    x = 16 // kv[0].element_size()
+    ce = kv[0].element_size()
+    fp8 = k_scales is not None
+    cache_dtype = "fp8" if fp8 else "auto"
+    kernel = "emm_append_paged_kernel" if fp8 else "emm_append_paged_wave_kernel"
+    x = 16 // ce
     g = torch.Generator(device=dev).manual_seed(4)
     blocks = torch.randperm(NB, device=dev, generator=g)
     dec = blocks[:decode] * bs + torch.randint(bs, (decode,), device=dev, generator=g)
@@ -748,14 +753,16 @@ def paged_append_bench(kv, NB, bs, H, D, dev, T=8448, decode=256):
     values = [torch.randn((T, H, D), device=dev, generator=g).to(torch.bfloat16) for _ in range(L)]
     kcs = [kv[l][0].view(NB, H, D // x, bs, x) for l in range(L)]
     vcs = [kv[l][1].view(NB, H, D, bs) for l in range(L)]
-    step_bytes = L * (T * 2 * H * D * 2 * 2 + 8 * T)
+    step_bytes = L * (T * 2 * H * D * (2 + ce) + 8 * T)
+    ks = [k_scales[l:l + 1] for l in range(L)] if fp8 else [None] * L
+    vs = [v_scales[l:l + 1] for l in range(L)] if fp8 else [None] * L
 
     def per_layer():
         for l in range(L):
-            cache_ops.reshape_and_cache(keys[l], values[l], kcs[l], vcs[l], slots, "auto")
+            cache_ops.reshape_and_cache(keys[l], values[l], kcs[l], vcs[l], slots, cache_dtype, ks[l], vs[l])
 
     def entry(ms, launches):
-        return rec(step_bytes, ms, launches, "emm_append_paged_kernel", tokens_per_s=round(T / (ms * 1e-3)))
+        return rec(step_bytes, ms, launches, kernel, tokens_per_s=round(T / (ms * 1e-3)))
 
     res = {"T": T, "decode_tokens": decode, "layers": L}
     med, _ = timed(per_layer, 20)
@@ -770,21 +777,38 @@ def paged_append_bench(kv, NB, bs, H, D, dev, T=8448, decode=256):
         per_layer()
     med, _ = timed(graph.replay, 20)
     res["per_layer_calls_hip_graph"] = entry(med, L)
-    plan = cache_ops.paged_layered_append(keys, values, kcs, vcs)
+    plan = cache_ops.paged_layered_append(keys, values, kcs, vcs, cache_dtype, k_scales, v_scales)
     med, _ = timed(lambda: plan(slots), 20)
     res["one_launch_all_layers"] = entry(med, 1)
     # a decode-only step: every token alone in its block (each 2-byte V element and each 16-byte K piece
     # lands in a cache line of its own, so the memory system rewrites the token's whole block region)
     Td = 256
-    dplan = cache_ops.paged_layered_append([k[:Td] for k in keys], [v[:Td] for v in values], kcs, vcs)
+    dplan = cache_ops.paged_layered_append([k[:Td] for k in keys], [v[:Td] for v in values], kcs, vcs,
+                                           cache_dtype, k_scales, v_scales)
     dslots = dec[:Td].contiguous() if decode >= Td else slots[:Td].contiguous()
     med, _ = timed(lambda: dplan(dslots), 20)
-    res["decode_only_256_tokens_one_launch"] = rec(L * Td * 2 * H * D * 4, med, 1, "emm_append_paged_kernel",
+    res["decode_only_256_tokens_one_launch"] = rec(L * Td * 2 * H * D * (2 + ce), med, 1, kernel,
                                                    tokens_per_s=round(Td / (med * 1e-3)))
 
     def decode_per_layer():
         for l in range(L):
-            cache_ops.reshape_and_cache(keys[l][:Td], values[l][:Td], kcs[l], vcs[l], dslots, "auto")
+            cache_ops.reshape_and_cache(keys[l][:Td], values[l][:Td], kcs[l], vcs[l], dslots, cache_dtype, ks[l], vs[l])
+
+    def decode_graph():
+        dgraph = torch.cuda.CUDAGraph()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            decode_per_layer()
+        torch.cuda.current_stream().wait_stream(side)
+        with torch.cuda.graph(dgraph):
+            decode_per_layer()
+        med, _ = timed(dgraph.replay, 20)
+        res["decode_step_256_tokens_per_layer_hip_graph"] = rec(L * Td * 2 * H * D * (2 + ce), med, L, kernel,
+                                                                tokens_per_s=round(Td / (med * 1e-3)))
+
+    if fp8:
+        decode_graph()
+        return res
 
     # the flash layout behind a head-major pool [NB, H, bs, D], handed over as the permuted view vLLM builds: the
     # strided append kernel, all layers in one launch
@@ -807,16 +831,7 @@ def paged_append_bench(kv, NB, bs, H, D, dev, T=8448, decode=256):
     med, _ = timed(head_major, 20)
     res["head_major_pool_one_launch_all_layers"]["eager_call_us"] = round(med * 1e3, 1)
 
-    dgraph = torch.cuda.CUDAGraph()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        decode_per_layer()
-    torch.cuda.current_stream().wait_stream(side)
-    with torch.cuda.graph(dgraph):
-        decode_per_layer()
-    med, _ = timed(dgraph.replay, 20)
-    res["decode_step_256_tokens_per_layer_hip_graph"] = rec(L * Td * 2 * H * D * 4, med, L, "emm_append_paged_kernel",
-                                                            tokens_per_s=round(Td / (med * 1e-3)))
+    decode_graph()
     return res
 
 
@@ -1100,6 +1115,7 @@ def fp8_shape(dev, spread=0, monolithic=False):
            "unpack": rec(2 * payload, ts_unpack, 64, "emm_block_move_kernel<unpack>"),
            "pack_plus_unpack": rec(4 * payload, ts_pack + ts_unpack, 128, "emm_block_move_kernel")}
     out["append"] = append_bench(src, NB, bs, H, D, k_scales, v_scales, dev)
+    out["append_paged_layout"] = paged_append_bench(src, NB, bs, H, D, dev, k_scales=k_scales, v_scales=v_scales)
     del dst, dp
     torch.cuda.empty_cache()
     # dequantising unpack into a bf16 pool (first 16 requests)
