@@ -42,10 +42,10 @@ def hooks_library_path() -> str:
 
 
 def build_library(verbose: bool = False, hooks: bool = False) -> str:
-    """Compile csrc/emm_kv.hip -> libemm_kv.so (always recompiles). ``hooks=True`` builds
+    """Compile csrc/emm_kv.hip (which includes the csrc/*.inc kernel files) -> libemm_kv.so (always recompiles). ``hooks=True`` builds
     libemm_kv_hooks.so instead: the same source with -DEMM_BENCH_HOOKS, which adds the launch-variant
     switch, the memory-system probes and the quotient sweep that bench.py and the GPU tests use
-    (csrc/emm_kv_hooks.h). The product library never contains them."""
+    (csrc/emm_kv_hooks.h, csrc/emm_kv_hooks.inc). The product library never contains them."""
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     out = _OUT_HOOKS if hooks else _OUT
     extra = ["-DEMM_BENCH_HOOKS", f"-I{os.path.join(_PKG, 'csrc')}"] if hooks else []
