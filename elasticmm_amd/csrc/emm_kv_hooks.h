@@ -20,7 +20,8 @@ extern "C" {
  * bits 8-11: 1 = non-temporal stores in the 16-byte block moves (default: sc0 sc1);
  * bits 12-15: shape of the 16-byte copy append (token rows per wave, waves per workgroup):
  *   0 = default ((4, 1) for a per-layer launch, (1, 1) for a whole-step launch), 1 = (1, 4), 2 = (2, 4),
- *   3 = (4, 1), 4 = (1, 1), 5 = (2, 1);
+ *   3 = (4, 1), 4 = (1, 1), 5 = (2, 1); for the fp8 append the same bits read: bit 12 = waves that convert a whole
+ *   row, bit 13 = waves that convert 512 elements (0 = by launch size);
  * bits 16-19: log2 of the blocks per plane visit of pack / unpack (15 = plain order);
  * bits 20-21: token tile of the paged-layout append (1 = 16 tokens, 2 = 4 tokens; 0 = by token count);
  * bits 22-23: row elements per workgroup of a one-layer paged-layout append (1 = 256, 2 = 128; 0 = by launch size);

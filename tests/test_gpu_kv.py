@@ -1309,6 +1309,49 @@ def test_cfg4_fp8_append_pack_dequant_reduced():
         assert same_bits(torch.stack(dq_g), torch.stack(dq_c)), str(dt)
 
 
+@pytest.mark.parametrize("bit,name", [(0x1000, "whole-row waves"), (0x2000, "512-element waves")])
+def test_fp8_append_both_wave_shapes(bit, name, monkeypatch):
+    """The fp8 append picks between waves that convert a whole row (pieces of 1024 elements) and waves that convert
+    512 elements by launch size; here each is forced, per layer and as one launch for all layers, on rows that end
+    inside a piece, rows longer than two pieces, strided sources, padded slots and both overflow modes."""
+    hooks = _lib.load_hooks()
+    monkeypatch.setattr(_lib, "_lib", hooks)
+    old = hooks.emm_hook_set_move_variant(bit)
+    try:
+        for (dtype, L, NB, bs, H, D, T, pad, mode) in [
+                (torch.bfloat16, 3, 64, 16, 8, 128, 700, 0, "fp8"), (torch.float16, 2, 40, 16, 5, 104, 333, 8, "fp8"),
+                (torch.bfloat16, 2, 20, 16, 1, 8, 100, 0, "fp8_e4m3_sat"), (torch.bfloat16, 2, 24, 8, 20, 128, 150, 0, "fp8"),
+                (torch.float16, 1, 16, 16, 3, 200, 77, 16, "fp8_e4m3_sat"), (torch.bfloat16, 2, 200, 16, 8, 128, 2500, 0, "fp8")]:
+            say(f"fp8 append, {name}: {dtype} L={L} NB={NB} bs={bs} H={H} D={D} T={T} pad={pad} {mode}")
+            g = torch.Generator().manual_seed(NB + T)
+            ks = (torch.rand(L, generator=g) * 0.09 + 0.01).float()
+            vs = (torch.rand(L, generator=g) * 0.09 + 0.01).float()
+            slots = make_slots(NB * bs, T, T)
+            pool_c = [torch.full((2, NB, bs, H, D), 0x5A, dtype=torch.uint8) for _ in range(L)]
+            pool_g, pool_g2 = to_dev(pool_c), to_dev(pool_c)
+            keys, values = [], []
+            for l in range(L):
+                src = (torch.randn((T, 2 * H * D + pad), generator=g) * 40).to(dtype)
+                src[::17, ::5] = 1e30 if dtype == torch.bfloat16 else 60000.0  # overflows of both signs
+                src[3::19, 1::7] *= -1
+                src_g = src.to(DEV)
+                keys.append(src_g[:, :H * D].view(T, H, D))
+                values.append(src_g[:, H * D:2 * H * D].view(T, H, D))
+                quant = orc.c_quant_fp8_sat if mode.endswith("sat") else orc.c_quant_fp8
+                live = slots >= 0  # the slots are distinct: a plain scatter of the quantised rows is the append
+                for kv, lo, scale in ((0, 0, ks[l]), (1, H * D, vs[l])):
+                    q = torch.from_numpy(quant(src[:, lo:lo + H * D].contiguous(), float(scale)))
+                    pool_c[l][kv].view(NB * bs, H * D)[slots[live]] = q[live]
+                cache_ops.reshape_and_cache_flash(keys[l], values[l], pool_g[l][0], pool_g[l][1], slots.to(DEV), mode,
+                                                  ks[l:l + 1].to(DEV), vs[l:l + 1].to(DEV))
+            cache_ops.reshape_and_cache_flash_layers(keys, values, pool_g2, slots.to(DEV), mode, ks, vs)
+            for l in range(L):
+                assert same_bits(pool_g[l], pool_c[l]), f"per layer, layer {l}"
+                assert same_bits(pool_g2[l], pool_c[l]), f"one launch, layer {l}"
+    finally:
+        hooks.emm_hook_set_move_variant(old)
+
+
 def test_fp8_dequant_all_bytes_all_scales(golden_dir):
     kat = json.load(open(os.path.join(golden_dir, "fp8_kat.json")))
     scales = kat["scales"]
