@@ -68,6 +68,10 @@ def parse():
                     help="stripes per pool of the headline: k > 1 allocates each pool's layers in k pieces spread over the "
                          "free device memory (KVWorker.init_kvcache(spread_stripes=k)); 0 (default): the reference's own "
                          "layout, one torch.empty per layer (what bind_kv_cache adopts from vLLM)")
+    ap.add_argument("--weights-gib", type=float, default=-1.0,
+                    help="size of the allocation made before the pools, standing for the model's weights, which a "
+                         "serving worker loads before it sizes and allocates its KV pool (default: the weights of the "
+                         "configuration's model; 0 = allocate the pools first)")
     ap.add_argument("--monolithic", action="store_true",
                     help="with --spread 0: one allocation per pool (init_kvcache's default) instead of one per layer")
     ap.add_argument("--no-append-context", action="store_true",
@@ -198,6 +202,25 @@ def release(*workers):
         w.kv_cache = None
         w._pool = None
     torch.cuda.empty_cache()
+
+
+# Bytes of the models' weights. A worker of the reference loads the model (elasticmm/engine/v0/worker.py:256), measures
+# what is left (:271-356) and only then allocates the KV pool (:358-394), so a pool never lies where a fresh process's
+# first allocations land. Where the pools land matters for scattered writes on this part (bench `extra.placement`).
+QWEN2_7B_WEIGHT_BYTES = 7_615_616_512 * 2   # bf16
+LLAMA_70B_FP8_WEIGHT_BYTES = 70_553_706_496  # 70B-class, fp8 weights beside the fp8 KV cache
+
+
+def weights_placeholder(args, nbytes, dev):
+    """One allocation of the model's weight bytes (or of --weights-gib), made before the pools and kept alive while
+    they are measured. Returns (tensor or None, GiB)."""
+    if args.weights_gib >= 0:
+        nbytes = int(args.weights_gib * (1 << 30))
+    if nbytes <= 0:
+        return None, 0.0
+    w = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    w.zero_()
+    return w, round(nbytes / (1 << 30), 3)
 
 
 # ---------------------------------------------------------------------------------------------- CPU baselines
@@ -373,6 +396,7 @@ def main():
     # The headline runs on the reference's own pool layout: one torch.empty per layer (the list bind_kv_cache adopts
     # from vLLM's CacheEngine, elasticmm/engine/v0/worker.py:388-394). Other layouts: --spread / --monolithic, and
     # extra.allocation_modes.
+    weights, weights_gib = weights_placeholder(args, QWEN2_7B_WEIGHT_BYTES, dev)
     src_w, dst_w = make_workers(NB, L, bs, H, D, dtype, dev, args.spread, monolithic=args.monolithic)
     dev_tables = [(s.to(dev), d.to(dev)) for s, d in tables]
     torch.cuda.synchronize()
@@ -453,17 +477,41 @@ def main():
                 modes["pack_probes_one_allocation"] = pack_chain_probes(sw, tabs, payload, dev)
             release(sw, dw)
             del tabs
+        if weights is not None:
+            # the reference's layout again, but with nothing allocated before the pools (what a process that only
+            # allocates pools gets; not fresh here: this process has allocated and freed other pools before)
+            weights = None
+            torch.cuda.empty_cache()
+            sw, dw = make_workers(NB, L, bs, H, D, dtype, dev, args.spread, monolithic=args.monolithic)
+            tabs = [(s.to(dev), d.to(dev)) for s, d in tables]
+            mm = measure_migrate(sw, dw, tabs, max(3, args.steps // 4), 2, payload)
+            modes["no_weights_resident"] = {
+                "value_GBps": round(mm["value"], 1), "frac": round(mm["value"] / HBM_PEAK_GBPS, 4),
+                "pack_GBps": round(mm["pack_GBps"], 1), "unpack_GBps": round(mm["unpack_GBps"], 1),
+                "note": "in a fresh process (--weights-gib 0) this layout measures 6.07-6.09 TB/s (unpack 5.93-5.97)"}
+            release(sw, dw)
+            del tabs
         modes["what"] = ("the headline workload on pools allocated differently: 'one_allocation_per_pool' is "
                          "init_kvcache's default (spread_stripes=0), 'four_stripes_per_pool' is init_kvcache("
                          "spread_stripes=4): the layers in 4 pieces pushed apart in device memory with temporary spacer "
                          "allocations. The headline itself runs on " + layout_name(args))
         extra["allocation_modes"] = modes
+    weights = None
+    torch.cuda.empty_cache()
     if "cfg1" in sections:
         extra["cfg1_latency"] = cfg1_latency(dev)
     if "fp8" in sections:
+        w8, g8 = weights_placeholder(args, LLAMA_70B_FP8_WEIGHT_BYTES, dev)
         extra["fp8_70b_shape"] = fp8_shape(dev, args.spread, args.monolithic)
+        extra["fp8_70b_shape"]["allocated_before_the_pools_GiB"] = g8
+        del w8
+        torch.cuda.empty_cache()
     if "rebalance" in sections:
+        w5, g5 = weights_placeholder(args, QWEN2_7B_WEIGHT_BYTES, dev)
         extra["rebalance_200GB"] = rebalance(dev)
+        extra["rebalance_200GB"]["allocated_before_the_pool_GiB"] = g5
+        del w5
+        torch.cuda.empty_cache()
     if "swap" in sections:
         extra["swap_pcie"] = swap_bench(dev)
 
@@ -488,6 +536,10 @@ def main():
             "num_layers": L, "num_blocks": NB, "block_size": bs, "kv_heads": H, "head_dim": D,
             "requests": len(tables), "blocks_moved": total_blocks, "algorithmic_bytes_per_step": bytes_per_step,
             "pool_allocation": layout_name(args) + " (extra.allocation_modes has the other layouts)",
+            "allocated_before_the_pools": ("%.3f GiB standing for the model's weights (Qwen2-7B, bf16): the reference's "
+                                           "worker loads the model, then sizes and allocates its pool "
+                                           "(elasticmm/engine/v0/worker.py:256, :271-394); --weights-gib 0 allocates the "
+                                           "pools first" % weights_gib) if weights_gib else "nothing (--weights-gib 0)",
         },
         "roofline": roofline,
         "extra": extra,
@@ -937,14 +989,24 @@ def append_in_context(keys, values, kv, slots, mode, ks, vs, entry, graphed, ste
             if with_append:
                 cache_ops.reshape_and_cache_flash(keys[l], values[l], kv[l][0], kv[l][1], slots, mode, ks[l], vs[l])
 
-    med_with, _ = timed(graphed(lambda: forward_like(True)).replay, 20)
-    med_without, _ = timed(graphed(lambda: forward_like(False)).replay, 20)
-    marginal_us = (med_with - med_without) * 1e3 / L
+    # the difference of two chains of ~240 us per layer: the two graphs are replayed alternately, round after round, so
+    # that clock and temperature drift hits both alike; the figure is the median of the rounds' differences
+    g_with, g_without = graphed(lambda: forward_like(True)), graphed(lambda: forward_like(False))
+    rounds = []
+    for _ in range(9):
+        a, _ = timed(g_with.replay, 5, warmup=1)
+        b, _ = timed(g_without.replay, 5, warmup=1)
+        rounds.append((a, b))
+    diffs = sorted((a - b) * 1e3 / L for a, b in rounds)
+    marginal_us = diffs[len(diffs) // 2]
+    med_with = sorted(a for a, _ in rounds)[len(rounds) // 2]
+    med_without = sorted(b for _, b in rounds)[len(rounds) // 2]
     ctx["between_projection_kernels"] = {
         "filler": "torch.mm [%d, %d] x [%d, %d] bf16 per layer" % (T, hidden, hidden, qkv),
         "filler_us_per_layer": round(med_without * 1e3 / L, 2),
         "with_append_us_per_layer": round(med_with * 1e3 / L, 2),
         "append_marginal_us_per_layer": round(marginal_us, 2),
+        "append_marginal_us_per_layer_rounds_min_max": [round(diffs[0], 2), round(diffs[-1], 2)],
         "append_marginal": rec(step_bytes, marginal_us * L * 1e-3, L, kernel, tokens_per_s=round(valid / (marginal_us * L * 1e-6))),
     }
     del xin, wqkv, yout
