@@ -461,6 +461,10 @@ def main():
         extra["placement"] = placement(src_w, dst_w, dev_tables, payload, dev)
     release(src_w, dst_w)
     dev_tables = None
+    if "placement" in sections:
+        # with the weights' allocation still in place: the same pools freed and allocated again
+        extra["placement"]["headline_on_pools_freed_and_allocated_again"] = reallocation_cycles(
+            args, tables, NB, L, bs, H, D, dtype, payload, dev)
 
     if "modes" in sections:
         modes = {}
@@ -739,6 +743,29 @@ def placement(src_w, dst_w, dev_tables, payload, dev):
             out["%s_%s_GBps_per_layer" % (pname, kname)] = rates
     out["note"] = ("each layer is an allocation of its own; the probes touch the batch's %d chunks of 16 KiB in both planes of "
                    "one layer per launch (%.0f MB)" % (n, layer_bytes / 1e6))
+    return out
+
+
+def reallocation_cycles(args, tables, NB, L, bs, H, D, dtype, payload, dev, cycles=4):
+    """The headline workload on pools that this process frees and allocates again, cycle after cycle (same layout, same
+    virtual addresses; the memory goes back to the driver in between). What the driver hands out changes with every
+    cycle of allocating and freeing — in this process and in the processes that ran on the device before — and with it
+    the rate of scattered writes into the pools: a fresh device gives its first process the slowest placement seen,
+    after three cycles of this size the figures settle."""
+    out = []
+    for _ in range(cycles):
+        sw, dw = make_workers(NB, L, bs, H, D, dtype, dev, args.spread, monolithic=args.monolithic)
+        tabs = [(s.to(dev), d.to(dev)) for s, d in tables]
+        mm = measure_migrate(sw, dw, tabs, 5, 2, payload)
+        bufs = [sw.extract_kv_blocks(s) for s, _ in tabs]
+        med, _ = timed(lambda: [sw.write_kv_blocks(d, b) for (_, d), b in zip(tabs, bufs)], 5)
+        out.append({"value_GBps": round(mm["value"], 1), "pack_GBps": round(mm["pack_GBps"], 1),
+                    "unpack_GBps": round(mm["unpack_GBps"], 1),
+                    "unpack_into_source_pool_GBps": round(2 * payload / med / 1e6, 1)})
+        del bufs, tabs
+        release(sw, dw)
+        del sw, dw
+        torch.cuda.empty_cache()
     return out
 
 
