@@ -170,6 +170,8 @@ def _table_for_launch(block_indices: IndexLike, pool: PoolView, strict: bool, wh
         idx = block_indices
         if idx.dtype != torch.long:
             raise TypeError(f"block index tensor must be int64, got {idx.dtype}")
+        if idx.device != pool.device:  # a table on another GPU: the kernel must not dereference a foreign pointer
+            idx = idx.to(pool.device)
         if not idx.is_contiguous():
             idx = idx.contiguous()
         if strict:
