@@ -706,8 +706,8 @@ def pack_chain_probes(src_w, dev_tables, payload, dev):
 
 
 def placement(src_w, dst_w, dev_tables, payload, dev):
-    """Where an allocation lands in device memory decides how fast scattered writes into it are, and that differs from
-    process to process for the same program (same virtual addresses): the batch's per-request unpacks into the
+    """Where an allocation lands in device memory decides how fast scattered writes into it are, and that follows what
+    the device's memory manager handed out and took back before (same virtual addresses every time): the batch's per-request unpacks into the
     destination pool and, from the same buffers, into the source pool of this process; and a scatter-write / gather-read
     probe (hooks build) of the batch's chunks into every layer — every allocation — of both pools by itself."""
     from elasticmm_amd import _lib, kv_ops
